@@ -1,0 +1,40 @@
+// C interface of the kernel library.  Every function returns 0 on success, a negative
+// value when it refuses its arguments or a launch fails; fl_last_error() then gives
+// the reason.  Pointers are device pointers unless a name says otherwise; `stream` is a
+// hipStream_t.  dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* fl_last_error(void);
+int fl_abi_version(void);
+
+// ---- plain kernels (plain.hip) ----
+int fl_embed(const void* table, int dtype, const int* tokens, float* out, int n, int H, int V,
+             hipStream_t stream);
+int fl_rmsnorm(const float* x, const float* delta, float* resid_out, const int* rows,
+               const float* w, void* out, int out_dtype, int n_rows, int H, float eps,
+               hipStream_t stream);
+int fl_add_inplace(float* x, const float* delta, long n, hipStream_t stream);
+int fl_gemm_plain(const void* x, const void* w, void* out, int in_dtype, int out_dtype, int M,
+                  int N, int K, hipStream_t stream);
+int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int* positions,
+                     const int* tok_seq, const int* block_table, int max_blocks, void* q_out,
+                     void* cache_base, int dtype, int n, int nh, int nkv, int hd, int page_size,
+                     int n_pages, int rot, float theta, int write_cache, hipStream_t stream);
+int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
+                  const int* positions, const int* tok_seq, const int* block_table,
+                  int max_blocks, int n, int nh, int nkv, int hd, int page_size, int n_pages,
+                  float scale, int window, hipStream_t stream);
+int fl_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n, int I,
+                hipStream_t stream);
+int fl_argmax(const float* logits, int* out, int rows, int V, hipStream_t stream);
+int fl_sample(const float* logits, const float* inv_temp, const float* uniform, int* out,
+              int rows, int V, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

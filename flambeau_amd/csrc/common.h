@@ -1,0 +1,89 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions,
+// wave64 reductions, the paged-cache address rule and host-side error reporting.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define FL_WAVE 64
+
+// dtype codes of the C interface
+#define FL_F32 0
+#define FL_BF16 1
+
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, FL_WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, FL_WAVE));
+    return v;
+}
+
+// Sum over a block of NW waves; every thread gets the total.  `lds` holds NW floats.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __syncthreads();
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += lds[w];
+    return t;
+}
+
+// Paged cache of one layer: [n_pages][2 (K,V)][n_kv_heads][page_size][head_dim].
+// Token t of a request lives in page table[t / page_size] at row t % page_size.
+struct PagedCache {
+    void* base;        // this layer's pool
+    int n_kv_heads;
+    int page_size;
+    int head_dim;
+    int n_pages;
+};
+
+__device__ __forceinline__ size_t cache_row_offset(const PagedCache& c, int page, int is_v,
+                                                   int kv_head, int row) {
+    return ((((size_t)page * 2 + is_v) * c.n_kv_heads + kv_head) * c.page_size + row) *
+           (size_t)c.head_dim;
+}
+
+// ---- host side -----------------------------------------------------------
+void fl_set_error(const char* fmt, ...);
+
+#define FL_CHECK(cond, ...)                \
+    do {                                   \
+        if (!(cond)) {                     \
+            fl_set_error(__VA_ARGS__);     \
+            return -1;                     \
+        }                                  \
+    } while (0)
+
+#define FL_LAUNCH_CHECK()                                                    \
+    do {                                                                     \
+        hipError_t e_ = hipGetLastError();                                   \
+        if (e_ != hipSuccess) {                                              \
+            fl_set_error("%s:%d launch failed: %s", __FILE__, __LINE__,      \
+                         hipGetErrorString(e_));                             \
+            return -2;                                                       \
+        }                                                                    \
+    } while (0)
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

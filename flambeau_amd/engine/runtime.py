@@ -1,0 +1,81 @@
+"""The device context parts run in: dtype, activation buffers, matrix products.
+
+All activation buffers are allocated once at ``max_batch_tokens`` rows and handed out as
+row prefixes, so addresses never change between steps (a captured graph replays on the
+same memory).  The reference does the same with its ``ScratchPool``
+(crates/forward/src/core/scratch.rs:819-1058).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..kernels.library import KernelError, load
+
+
+class Runtime:
+    def __init__(self, device="cuda:0", dtype=torch.bfloat16, max_batch_tokens: int = 2048,
+                 tuned: bool = True):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"dtype must be float32 or bfloat16, got {dtype}")
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("flambeau_amd runs on the GPU only: there is no CPU path")
+        if not torch.cuda.is_available():
+            raise RuntimeError("flambeau_amd: no GPU visible to this process")
+        torch.cuda.set_device(self.device)
+        load()   # fails loudly when the kernel library cannot be built or loaded
+        self.dtype = dtype
+        # tuned kernels exist for bfloat16 only; the 32-bit path always runs the plain ones
+        self.tuned = bool(tuned) and dtype == torch.bfloat16
+        self.max_batch_tokens = int(max_batch_tokens)
+        self._buffers: dict = {}
+        self._scope = ""
+
+    # ------------------------------------------------------------ buffers
+    def buffer(self, name: str, rows: int, cols: int, dtype=None, max_rows: int | None = None):
+        """A ``[rows, cols]`` view of the buffer ``name``.  A buffer grows (to the next power of
+        two of rows, never beyond its maximum) when a step needs more rows than any before."""
+        dtype = dtype or self.dtype
+        cap = max_rows if max_rows is not None else self.max_batch_tokens
+        if rows > cap:
+            raise KernelError(f"buffer '{name}': {rows} rows asked, at most {cap} allowed")
+        key = (self._scope, name, cols, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.shape[0] < rows:
+            size = min(cap, max(16, 1 << max(rows - 1, 0).bit_length()))
+            buf = torch.empty((size, cols), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:rows]
+
+    def scope(self, name: str):
+        """Buffers asked for inside ``with rt.scope(name)`` are separate from all others (a
+        captured graph keeps its own, which never move)."""
+        rt = self
+
+        class _Scope:
+            def __enter__(self_inner):
+                self_inner.prev, rt._scope = rt._scope, name
+            def __exit__(self_inner, *exc):
+                rt._scope = self_inner.prev
+        return _Scope()
+
+    def to_device(self, t: torch.Tensor, role: str) -> torch.Tensor:
+        """A loaded tensor in the dtype its role asks for, on the device."""
+        if role in ("matrix", "table"):
+            want = self.dtype
+        elif role == "vector32":
+            want = torch.float32
+        elif role == "int32":
+            want = torch.int32
+        else:
+            raise ValueError(f"unknown tensor role '{role}'")
+        return t.to(device=self.device, dtype=want).contiguous()
+
+    # ------------------------------------------------------------ matrix products
+    def gemm(self, x, w, out):
+        """``out = x @ w.T``; ``w`` is ``[out_features, in_features]``."""
+        if self.tuned:
+            from ..kernels import tuned
+            return tuned.gemm(x, w, out)
+        return ops.gemm_plain(x, w, out)

@@ -1,0 +1,156 @@
+"""Typed wrappers of the plain kernels.
+
+Each wrapper checks on the host that the tensors have the device, dtype, contiguity
+and shape the kernel and its grid assume, and only then launches on torch's current
+stream.  (The reference keeps the same split: typed, bounds-checked leaf functions
+above raw launches, crates/model-ops/src/lib.rs:47-82.)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .library import KernelError, call
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {dtype}: the kernels take float32 and bfloat16") from None
+
+
+def stream_handle() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(t: torch.Tensor, name: str, dtype=None, shape=None):
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}, the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor is not contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    if shape is not None:
+        if t.dim() != len(shape) or any(e is not None and e != s for s, e in zip(t.shape, shape)):
+            raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+    return t.data_ptr()
+
+
+@dataclass
+class PagedLayerCache:
+    """The key/value pool of one layer: ``pool[n_pages, 2, n_kv_heads, page_size, head_dim]``."""
+    pool: torch.Tensor
+
+    @property
+    def n_pages(self): return self.pool.shape[0]
+    @property
+    def n_kv_heads(self): return self.pool.shape[2]
+    @property
+    def page_size(self): return self.pool.shape[3]
+    @property
+    def head_dim(self): return self.pool.shape[4]
+
+
+def embed(table, tokens, out):
+    V, H = table.shape
+    n = tokens.shape[0]
+    call("fl_embed", _check(table, "embed.table"), dtype_code(table.dtype),
+         _check(tokens, "embed.tokens", torch.int32, (n,)),
+         _check(out, "embed.out", torch.float32, (n, H)), n, H, V, stream_handle())
+    return out
+
+
+def rmsnorm(x, weight, out, eps, delta=None, store_sum=False, rows=None):
+    """``out = rmsnorm(x (+ delta)) * weight``; ``store_sum`` writes x + delta back into x;
+    ``rows`` (int32) picks the rows of x that are normed, one output row each."""
+    n, H = x.shape
+    px = _check(x, "rmsnorm.x", torch.float32, (n, H))
+    pd = _check(delta, "rmsnorm.delta", torch.float32, (n, H)) if delta is not None else None
+    pr = _check(rows, "rmsnorm.rows", torch.int32) if rows is not None else None
+    n_out = rows.shape[0] if rows is not None else n
+    if store_sum and delta is None:
+        store_sum = False
+    call("fl_rmsnorm", px, pd, px if store_sum else None, pr,
+         _check(weight, "rmsnorm.weight", torch.float32, (H,)),
+         _check(out, "rmsnorm.out", None, (n_out, H)), dtype_code(out.dtype), n_out, H, float(eps),
+         stream_handle())
+    return out
+
+
+def add_inplace(x, delta):
+    if x.shape != delta.shape:
+        raise KernelError(f"add: shapes {tuple(x.shape)} and {tuple(delta.shape)} differ")
+    call("fl_add_inplace", _check(x, "add.x", torch.float32), _check(delta, "add.delta", torch.float32),
+         x.numel(), stream_handle())
+    return x
+
+
+def gemm_plain(x, w, out):
+    """``out[m, n] = sum_k x[m, k] w[n, k]``."""
+    M, K = x.shape
+    N = w.shape[0]
+    call("fl_gemm_plain", _check(x, "gemm.x", w.dtype, (M, K)), _check(w, "gemm.w", None, (N, K)),
+         _check(out, "gemm.out", None, (M, N)), dtype_code(x.dtype), dtype_code(out.dtype), M, N, K,
+         stream_handle())
+    return out
+
+
+def rope_kv_write(qkv, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads,
+                  rotated_dims, theta, write_cache=True):
+    n, ld = qkv.shape
+    nkv, hd = cache.n_kv_heads, cache.head_dim
+    if ld != (n_heads + 2 * nkv) * hd:
+        raise KernelError(f"rope_kv_write: row of {ld} values, expected {(n_heads + 2 * nkv) * hd}")
+    call("fl_rope_kv_write", _check(qkv, "rope.qkv"), dtype_code(qkv.dtype), ld,
+         _check(positions, "rope.positions", torch.int32, (n,)),
+         _check(tok_seq, "rope.tok_seq", torch.int32, (n,)),
+         _check(block_table, "rope.block_table", torch.int32, (None, None)), block_table.shape[1],
+         _check(q_out, "rope.q_out", cache.pool.dtype, (n, n_heads * hd)),
+         _check(cache.pool, "rope.cache"), dtype_code(cache.pool.dtype), n, n_heads, nkv, hd,
+         cache.page_size, cache.n_pages, int(rotated_dims), float(theta), int(bool(write_cache)),
+         stream_handle())
+    return q_out
+
+
+def attn_plain(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, n_heads, scale, window):
+    n = q.shape[0]
+    hd = cache.head_dim
+    dt = cache.pool.dtype
+    call("fl_attn_plain", _check(q, "attn.q", dt, (n, n_heads * hd)),
+         _check(out, "attn.out", dt, (n, n_heads * hd)), _check(cache.pool, "attn.cache"),
+         dtype_code(dt), _check(positions, "attn.positions", torch.int32, (n,)),
+         _check(tok_seq, "attn.tok_seq", torch.int32, (n,)),
+         _check(block_table, "attn.block_table", torch.int32, (None, None)), block_table.shape[1],
+         n, n_heads, cache.n_kv_heads, hd, cache.page_size, cache.n_pages, float(scale), int(window),
+         stream_handle())
+    return out
+
+
+def silu_mul(gu, out):
+    n, two_i = gu.shape
+    I = two_i // 2
+    call("fl_silu_mul", _check(gu, "silu_mul.gu"), dtype_code(gu.dtype),
+         _check(out, "silu_mul.out", None, (n, I)), dtype_code(out.dtype), n, I, stream_handle())
+    return out
+
+
+def argmax(logits, out):
+    R, V = logits.shape
+    call("fl_argmax", _check(logits, "argmax.logits", torch.float32), _check(out, "argmax.out", torch.int32, (R,)),
+         R, V, stream_handle())
+    return out
+
+
+def sample(logits, inv_temp, uniform, out):
+    R, V = logits.shape
+    call("fl_sample", _check(logits, "sample.logits", torch.float32),
+         _check(inv_temp, "sample.inv_temp", torch.float32, (R,)),
+         _check(uniform, "sample.uniform", torch.float32, (R,)),
+         _check(out, "sample.out", torch.int32, (R,)), R, V, stream_handle())
+    return out

@@ -1,0 +1,124 @@
+"""A decoder described as data, and the model built from the description.
+
+``ModelSpec`` lists the layers (each a block ``PartSpec`` plus the file names of its tensors)
+and, separately, the order in which they run: a list of ``RunEntry`` that may name a layer
+twice (shared weights) or let an entry read the cache an earlier entry wrote.  Caches belong
+to run-order entries, not to layers.  ``DecoderModel`` turns the description into parts,
+says which tensors it needs (``manifest``), takes them (``bind``) and runs a batch
+(``forward``).  The reference's counterpart is the ``Arch`` trait and the layer loop of a
+model crate (crates/forward/src/runtime/mod.rs:59-136, crates/models/qwen35-v2/src/model.rs:11-51).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..parts import BLOCKS, NORMS, OutputHead, PartSpec, ResidualStream, TokenEmbedding
+
+
+@dataclass
+class LayerSpec:
+    block: PartSpec
+    names: dict                       # the block's local tensor name -> name in the weight files
+
+
+@dataclass
+class RunEntry:
+    layer: int                        # index into ModelSpec.layers
+    cache_of: int | None = None       # index of an earlier run-order entry whose cache is read
+
+
+@dataclass
+class ModelSpec:
+    architecture: str
+    hidden_size: int
+    vocab_size: int
+    max_position: int
+    layers: list
+    run_order: list
+    final_norm: PartSpec
+    names: dict                       # "embedding.weight", "final_norm.weight", "head.weight" -> file names
+    tied_head: bool = False
+    eos_token_id: int | None = None
+    bos_token_id: int | None = None
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, rt):
+        self.spec = spec
+        self.rt = rt
+        self.embedding = TokenEmbedding(spec.vocab_size, spec.hidden_size)
+        self.blocks = [BLOCKS.create(ls.block) for ls in spec.layers]
+        self.final_norm = NORMS.create(spec.final_norm)
+        self.head = OutputHead(spec.vocab_size, spec.hidden_size, tied=spec.tied_head)
+        for i, e in enumerate(spec.run_order):
+            if not 0 <= e.layer < len(self.blocks):
+                raise ValueError(f"run-order entry {i} names layer {e.layer}, the model has {len(self.blocks)}")
+
+    # ------------------------------------------------------------ tensors
+    def manifest(self) -> dict:
+        """``{file tensor name: (owner, local name, TensorSpec)}`` of everything the model loads."""
+        out = {}
+
+        def put(file_name, owner, local, tspec):
+            if file_name in out:
+                raise ValueError(f"tensor '{file_name}' is asked for twice")
+            out[file_name] = (owner, local, tspec)
+
+        for local, ts in self.embedding.tensors().items():
+            put(self.spec.names["embedding." + local], "embedding", local, ts)
+        for li, (ls, block) in enumerate(zip(self.spec.layers, self.blocks)):
+            for local, ts in block.tensors().items():
+                if local not in ls.names:
+                    raise KeyError(f"layer {li}: no file name given for the tensor '{local}'")
+                put(ls.names[local], li, local, ts)
+        for local, ts in self.final_norm.tensors().items():
+            put(self.spec.names["final_norm." + local], "final_norm", local, ts)
+        for local, ts in self.head.tensors().items():
+            put(self.spec.names["head." + local], "head", local, ts)
+        return out
+
+    def bind(self, tensors: dict) -> None:
+        """``tensors``: file name -> device tensor, as ``manifest`` asked for them."""
+        per_owner: dict = {}
+        for file_name, (owner, local, _) in self.manifest().items():
+            per_owner.setdefault(owner, {})[local] = tensors[file_name]
+        self.embedding.bind(per_owner.get("embedding", {}), self.rt)
+        for li, block in enumerate(self.blocks):
+            block.bind(per_owner.get(li, {}), self.rt)
+        self.final_norm.bind(per_owner.get("final_norm", {}), self.rt)
+        self.head.bind(per_owner.get("head", {}), self.rt, embedding_table=self.embedding.weight)
+
+    # ------------------------------------------------------------ cache needs
+    def cache_entries(self):
+        """Per run-order entry: (cache spec or None, index of the entry it shares with or None)."""
+        specs, shares = [], []
+        for e in self.spec.run_order:
+            specs.append(self.blocks[e.layer].cache_spec())
+            shares.append(e.cache_of)
+        return specs, shares
+
+    def mixer_classes(self):
+        seen = []
+        for b in self.blocks:
+            for m in getattr(b, "mixers", lambda: [])():
+                if type(m) not in seen:
+                    seen.append(type(m))
+        return seen
+
+    # ------------------------------------------------------------ the forward pass of one batch
+    def forward(self, step, caches, max_logit_rows: int):
+        """Logits ``[R, vocab]`` (float32) at ``step.logit_rows``; ``caches[i]`` belongs to
+        run-order entry ``i``."""
+        rt = self.rt
+        resid = rt.buffer("residual", step.n_tokens, self.spec.hidden_size, torch.float32)
+        self.embedding.forward(step.tokens, resid)
+        stream = ResidualStream(resid, rt)
+        for i, e in enumerate(self.spec.run_order):
+            self.blocks[e.layer].forward(stream, step, caches[i])
+        if step.logit_rows.shape[0] == 0:
+            stream.flush()
+            return None
+        x = stream.normed(self.final_norm, rows=step.logit_rows, name="final")
+        return self.head.forward(x, max_logit_rows)

@@ -1,0 +1,77 @@
+"""Grouped-query attention over the paged cache.
+
+x -> Q, K, V (one joined matrix product) -> position encoding on Q and K -> K, V stored at
+the tokens' positions -> softmax(Q K^T / sqrt(hd)) V over the keys
+[max(0, p - window + 1), p] of the same request -> output projection.
+(crates/forward/src/core/composites/standard_attn.rs:198-286 projections, :356-397
+rotation, :485-500 paged store, :509-533 attention, :1289-1301 output projection; head map
+kv_head = q_head / (n_heads / n_kv_heads), crates/kernels-hip/src/kernels/attention_prefill_f16.cu:50-51.)
+
+This step's keys are stored before attention runs, so every query reads all its keys from the
+cache and the same code serves whole prompts, portions and single decoded tokens.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..kernels import ops
+from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, TensorSpec
+
+
+@MIXERS.register("paged_gqa_attention")
+class PagedGQAAttention(Mixer):
+    def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                 position: PartSpec, window: int = 0, scale: float | None = None):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} query heads are not a multiple of {n_kv_heads} key/value heads")
+        self.hidden_size = hidden_size
+        self.n_heads = n_heads
+        self.n_kv_heads = n_kv_heads
+        self.head_dim = head_dim
+        self.window = int(window or 0)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.position = POSITION_ENCODINGS.create(position)
+
+    def cache_spec(self):
+        return PagedKVSpec(self.n_kv_heads, self.head_dim, self.window)
+
+    def tensors(self):
+        H, qw, kvw = self.hidden_size, self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
+        return {"q.weight": TensorSpec((qw, H)), "k.weight": TensorSpec((kvw, H)),
+                "v.weight": TensorSpec((kvw, H)), "o.weight": TensorSpec((H, qw))}
+
+    @classmethod
+    def step_metadata(cls, batch):
+        from ..kernels import tuned
+        return tuned.attention_metadata(batch)
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.w_qkv = torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0).contiguous()
+        self.w_o = weights["o.weight"]
+        self.position.bind({}, rt)
+
+    def forward(self, x, step, cache):
+        rt, n = self.rt, x.shape[0]
+        nh, nkv, hd = self.n_heads, self.n_kv_heads, self.head_dim
+        table = step.block_tables[cache.group]
+        qkv = rt.buffer("attn_qkv", n, (nh + 2 * nkv) * hd, torch.float32)
+        rt.gemm(x, self.w_qkv, qkv)
+        rotary = self.position.rotary_parameters()
+        if rotary is None:
+            self.position.apply(qkv, step.positions, nh, nkv, hd)
+            rotary = (0, 1.0)
+        q = rt.buffer("attn_q", n, nh * hd)
+        ops.rope_kv_write(qkv, step.positions, step.tok_seq, table, q, cache.kv, nh, rotary[0], rotary[1],
+                          write_cache=cache.writes)
+        out = rt.buffer("attn_out", n, nh * hd)
+        if rt.tuned:
+            from ..kernels import tuned
+            tuned.attention(q, out, cache.kv, step, table, nh, self.scale, self.window)
+        else:
+            ops.attn_plain(q, out, cache.kv, step.positions, step.tok_seq, table, nh, self.scale, self.window)
+        delta = rt.buffer("delta", n, self.hidden_size, torch.float32)
+        rt.gemm(out, self.w_o, delta)
+        return delta

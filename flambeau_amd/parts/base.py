@@ -1,0 +1,200 @@
+"""What a model is built from: the interfaces of the parts and the records they exchange.
+
+A decoder layer is an arrangement (``Block``) of a ``Mixer`` (attention here), a
+``FeedForward``, ``Norm``s and, inside the mixer, a ``PositionEncoding``.  Each part
+is created from a ``PartSpec`` (a registry key plus its sizes and constants), says
+which tensors it needs, is given them, and is then run on a batch.  No part knows
+which model it is in: everything it needs arrives through its parameters, the
+``StepState`` and its ``LayerCache``.
+
+The reference's counterpart is the composite-op vocabulary a model writes against
+(crates/forward/src/ctx.rs:14-206) with per-kind weight bundles
+(ctx.rs:316-496) and the per-layer cache shape (crates/forward/src/core/scratch.rs:137-165).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable
+
+import torch
+
+
+# ---------------------------------------------------------------- descriptions
+@dataclass(frozen=True)
+class PartSpec:
+    """A part chosen by the configuration: registry key and parameters."""
+    kind: str
+    params: dict = field(default_factory=dict)
+
+    def __hash__(self):
+        return hash((self.kind, tuple(sorted((k, repr(v)) for k, v in self.params.items()))))
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """A tensor a part needs.  ``role``: ``matrix``/``table`` are stored in the compute
+    dtype; ``vector32`` (norm gains) is always held in float32; ``int32`` integer tables."""
+    shape: tuple
+    role: str = "matrix"
+
+
+@dataclass(frozen=True)
+class PagedKVSpec:
+    """Per-token rows that grow with the request: keys and values in pages.
+    ``window`` = number of newest keys still needed (0: all)."""
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Per-request state of fixed size, one record per slot, zeroed when a slot is claimed."""
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerCache:
+    """What one run-order entry sees of the cache."""
+    kv: Any = None                 # kernels.ops.PagedLayerCache or None
+    group: int = -1                # index of the block table in StepState.block_tables
+    state: torch.Tensor | None = None   # [max_slots, *StateSpec.shape]
+    writes: bool = True            # False: the entry reads another layer's cache
+
+
+@dataclass
+class StepState:
+    """One batch on the device.  Tokens of all requests lie one after another;
+    ``tok_seq[i]`` is the index (within this step) of the request token ``i`` belongs to."""
+    n_tokens: int
+    n_seqs: int
+    tokens: torch.Tensor           # int32 [n]
+    positions: torch.Tensor        # int32 [n] absolute position of each token
+    tok_seq: torch.Tensor          # int32 [n]
+    seq_slots: torch.Tensor        # int32 [S] state slot of each request
+    seq_q_start: torch.Tensor      # int32 [S] first row of the request in this batch
+    seq_q_len: torch.Tensor        # int32 [S]
+    seq_ctx_len: torch.Tensor      # int32 [S] tokens in the cache after this step
+    block_tables: list             # per cache group: int32 [S, max_blocks], -1 = no page
+    logit_rows: torch.Tensor       # int32 [R] rows whose logits are wanted
+    host: "HostBatch"              # the same numbers on the host, for choosing kernels
+    extra: dict = field(default_factory=dict)   # metadata parts asked for (step_metadata)
+
+
+@dataclass
+class HostBatch:
+    """Host-side description of a batch, before upload."""
+    q_starts: list
+    q_lens: list
+    start_pos: list                # position of each request's first token in this step
+    slots: list
+    n_tokens: int
+    n_logit_rows: int
+    fixed_shape: bool = False      # padded to a fixed size for graph replay
+
+    @property
+    def n_seqs(self): return len(self.q_lens)
+    @property
+    def all_single(self): return all(q == 1 for q in self.q_lens)
+    @property
+    def max_q_len(self): return max(self.q_lens) if self.q_lens else 0
+    @property
+    def max_ctx_len(self): return max((s + q for s, q in zip(self.start_pos, self.q_lens)), default=0)
+
+
+# ---------------------------------------------------------------- interfaces
+class Part:
+    """Base of all parts.  Subclasses take their sizes and constants as keyword
+    parameters, list their tensors, and receive them in ``bind``."""
+
+    def tensors(self) -> dict:
+        """``{local name: TensorSpec}``."""
+        return {}
+
+    def bind(self, weights: dict, rt) -> None:
+        """Take the loaded tensors (already on the device, in the dtype their role asks for)."""
+        self.rt = rt
+
+
+class Norm(Part):
+    def forward(self, x, out, delta=None, store_sum=False, rows=None):
+        """``out = norm(x (+ delta))``; ``x`` is the 32-bit residual stream; with
+        ``store_sum`` the sum is written back to ``x``; ``rows`` selects rows."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary_parameters(self):
+        """``(rotated_dims, theta)`` if this encoding is the split-half rotation the fused
+        rotate-and-store kernel implements, else ``None`` (then ``apply`` is called)."""
+        return None
+
+    def apply(self, q, k, positions, n_heads, n_kv_heads, head_dim):
+        """Encode positions into ``q`` and ``k`` in place (rows of the fused projection)."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self):
+        """``PagedKVSpec``, ``StateSpec`` or ``None``."""
+        return None
+
+    @classmethod
+    def step_metadata(cls, batch: HostBatch) -> dict:
+        """Integer arrays (numpy int32) this kind of mixer wants on the device for the batch,
+        uploaded with the rest of the step's metadata and found in ``StepState.extra``."""
+        return {}
+
+    def forward(self, x, step: StepState, cache: LayerCache):
+        """``x``: normed activations [n, hidden] in the compute dtype.  Returns the
+        32-bit delta [n, hidden] that is added to the residual stream."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, step: StepState):
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of parts.  ``forward`` advances the residual stream by one layer."""
+
+    def cache_spec(self):
+        return None
+
+    def forward(self, stream, step: StepState, cache: LayerCache) -> None:
+        raise NotImplementedError
+
+
+# ---------------------------------------------------------------- registries
+class PartRegistry:
+    """Registry key -> constructor, one registry per family of parts."""
+
+    def __init__(self, family: str):
+        self.family = family
+        self._makers: dict[str, Callable] = {}
+
+    def register(self, kind: str, maker: Callable | None = None):
+        def deco(m):
+            self._makers[kind] = m
+            return m
+        return deco(maker) if maker is not None else deco
+
+    def create(self, spec: PartSpec, **more):
+        try:
+            maker = self._makers[spec.kind]
+        except KeyError:
+            known = ", ".join(sorted(self._makers)) or "(none)"
+            raise KeyError(f"unknown {self.family} '{spec.kind}'; known: {known}") from None
+        return maker(**spec.params, **more)
+
+    def known(self):
+        return sorted(self._makers)
+
+
+MIXERS = PartRegistry("mixer")
+FEED_FORWARDS = PartRegistry("feed-forward")
+NORMS = PartRegistry("norm")
+POSITION_ENCODINGS = PartRegistry("position encoding")
+BLOCKS = PartRegistry("block")

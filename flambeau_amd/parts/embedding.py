@@ -1,0 +1,49 @@
+"""Token embedding and output head.
+
+h0[i,:] = E[token[i],:], no scaling (crates/forward/src/core/composites/embed.rs:26-62);
+logits = norm_f(x) Wlm^T in 32-bit, a tied head being the embedding table again
+(crates/forward/src/core/composites/output_head.rs:41-100,
+crates/models/qwen35-v2/src/loader.rs:218-223)."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import Part, TensorSpec
+
+
+class TokenEmbedding(Part):
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+
+    def tensors(self):
+        return {"weight": TensorSpec((self.vocab_size, self.hidden_size), "table")}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.weight = weights["weight"]
+
+    def forward(self, tokens, out):
+        return ops.embed(self.weight, tokens, out)
+
+
+class OutputHead(Part):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.tied = tied
+
+    def tensors(self):
+        return {} if self.tied else {"weight": TensorSpec((self.vocab_size, self.hidden_size))}
+
+    def bind(self, weights, rt, embedding_table=None):
+        self.rt = rt
+        self.weight = embedding_table if self.tied else weights["weight"]
+        if self.weight is None:
+            raise ValueError("a tied output head needs the embedding table")
+
+    def forward(self, x, max_rows):
+        logits = self.rt.buffer("logits", x.shape[0], self.vocab_size, torch.float32, max_rows=max_rows)
+        self.rt.gemm(x, self.weight, logits)
+        return logits

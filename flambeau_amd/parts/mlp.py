@@ -1,0 +1,36 @@
+"""Dense SwiGLU feed-forward: d = (silu(x Wg^T) * (x Wu^T)) Wd^T
+(crates/forward/src/core/composites/dense_ffn.rs:116-186).  Gate and up matrices are
+joined at load so that one matrix product feeds both."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import FEED_FORWARDS, FeedForward, TensorSpec
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+
+    def tensors(self):
+        H, I = self.hidden_size, self.intermediate_size
+        return {"gate.weight": TensorSpec((I, H)), "up.weight": TensorSpec((I, H)),
+                "down.weight": TensorSpec((H, I))}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.w_gate_up = torch.cat([weights["gate.weight"], weights["up.weight"]], dim=0).contiguous()
+        self.w_down = weights["down.weight"]
+
+    def forward(self, x, step):
+        rt, n, I = self.rt, x.shape[0], self.intermediate_size
+        gu = rt.buffer("ffn_gate_up", n, 2 * I, torch.float32)
+        rt.gemm(x, self.w_gate_up, gu)
+        act = rt.buffer("ffn_act", n, I)
+        ops.silu_mul(gu, act)
+        delta = rt.buffer("delta", n, self.hidden_size, torch.float32)
+        rt.gemm(act, self.w_down, delta)
+        return delta

@@ -1,0 +1,42 @@
+"""Tiny configurations of the architecture for the tests.  They differ in every size and
+option: layers, width, head counts and groups (GQA, MQA, MHA), head size (derived, explicit
+and not width/heads), intermediate size, vocabulary (none a power of two but A's), theta,
+window (16, none, 24 = no multiple of a page), eps, tied or untied head, weight scale."""
+import torch
+
+from flambeau_amd.weights import write_random_model
+
+
+def _cfg(**kw):
+    base = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "hidden_act": "silu"}
+    base.update(kw)
+    return base
+
+
+TINY = {
+    "A": dict(
+        config=_cfg(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
+                    intermediate_size=160, vocab_size=256, rope_theta=10000.0, sliding_window=16,
+                    rms_norm_eps=1e-5, max_position_embeddings=128, tie_word_embeddings=False),
+        seed=0, std=0.02, gain_std=0.01, page_size=8),
+    "B": dict(
+        config=_cfg(num_hidden_layers=3, hidden_size=96, num_attention_heads=6, num_key_value_heads=1,
+                    head_dim=24, intermediate_size=224, vocab_size=384, rope_theta=1e6,
+                    sliding_window=None, rms_norm_eps=1e-6, max_position_embeddings=256,
+                    tie_word_embeddings=False),
+        seed=2, std=0.05, gain_std=0.01, page_size=16),
+    "C": dict(
+        config=_cfg(num_hidden_layers=2, hidden_size=80, num_attention_heads=5, num_key_value_heads=5,
+                    head_dim=32, intermediate_size=136, vocab_size=300, rope_theta=5e5,
+                    sliding_window=24, rms_norm_eps=1e-4, max_position_embeddings=640,
+                    tie_word_embeddings=True),
+        seed=5, std=0.04, gain_std=0.02, page_size=16),
+}
+
+STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def write_tiny(name, out_dir, store="float32"):
+    t = TINY[name]
+    return write_random_model(t["config"], out_dir, seed=t["seed"], std=t["std"], gain_std=t["gain_std"],
+                              store_dtype=STORE[store])
