@@ -1,0 +1,215 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, in every way of
+cutting the work.  A difference that appears in one way of cutting only is a fault of the cache
+or of the batch; the failure message names the first wrong position."""
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+import replay_helpers as rh
+from tiny_configs import TINY, write_sharpened
+
+pytestmark = pytest.mark.gpu
+
+STORE = {"float32": "float32", "bfloat16": "bfloat16"}
+LENGTHS = {"A": [5, 12, 23, 40, 70, 97], "B": [1, 31, 97, 64, 129], "C": [3, 50, 33, 150, 81]}
+
+
+def make_runner(model_dir, dtype, name, n_tokens, max_slots=8, page_size=None, tuned=True):
+    from flambeau_amd.engine import ModelRunner, load_model
+    ps = page_size or TINY[name]["page_size"]
+    model, _ = load_model(model_dir, dtype=dtype, max_batch_tokens=512, tuned=tuned)
+    return ModelRunner(model, n_pages=-(-n_tokens // ps), page_size=ps, max_slots=max_slots, max_logit_rows=512)
+
+
+def requests_for(name, seed=1):
+    return rh.make_requests(TINY[name]["config"]["vocab_size"], LENGTHS[name], seed)
+
+
+@pytest.fixture(scope="module")
+def runners(model_dirs):
+    """One runner per (configuration, dtype), with a pool so small that pages are used again."""
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            cache[(name, dtype)] = make_runner(model_dirs[(name, STORE[dtype])], dtype, name, n_tokens=448)
+        return cache[(name, dtype)]
+    return get
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_cutting(model_dirs, runners, name, dtype, mode):
+    d = model_dirs[(name, STORE[dtype])]
+    reqs = requests_for(name)
+    steps = {"whole": rh.trace_whole, "tail": rh.trace_tail, "portions": rh.trace_portions,
+             "mixed": lambda r: rh.trace_mixed(r, seed=7)}[mode](reqs)
+    runner = runners(name, dtype)
+    got = rh.run_in_process(runner, steps)
+    assert not runner.manager.live and runner.manager.free_pages() == [p.n_pages for p in runner.manager.pools]
+    rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, f"{name} {mode}")
+    if mode != "mixed":
+        assert len(got) == sum(len(t) for t in reqs.values())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_peaked_attention_in_every_cutting(tmp_path_factory, name, dtype):
+    """Queries and keys scaled up: single keys matter, so a key lost at a window's edge, at a
+    page's edge or in a page that is used again moves the logits far beyond the tolerance.
+    In bfloat16 the factor is smaller: scores of size 20 to 30 would turn the 8-bit rounding of
+    queries and keys into errors of several percent in the softmax weights, whatever the engine
+    does."""
+    factor = 12.0 if dtype == "float32" else 4.0
+    d = write_sharpened(name, tmp_path_factory.mktemp("sharp") / name, STORE[dtype], factor)
+    reqs = rh.make_requests(TINY[name]["config"]["vocab_size"], [90, 41, 120, 66], seed=11)
+    ref = rh.plain_logits(d, reqs)
+    runner = make_runner(d, dtype, name, n_tokens=320)
+    for mode, steps in [("whole", rh.trace_whole(reqs)), ("tail", rh.trace_tail(reqs)),
+                        ("portions", rh.trace_portions(reqs, sizes=(3, 2, 9, 8, 2, 25, 7))),
+                        ("mixed", rh.trace_mixed(reqs, seed=5, max_portion=19))]:
+        got = rh.run_in_process(runner, steps)
+        rh.compare(got, reqs, ref, dtype, f"peaked {name} {mode}")
+
+
+def test_few_pages_are_used_again(model_dirs):
+    """With room for little more than the live requests, later requests get the pages of earlier
+    ones; their logits must not see what was there."""
+    name, dtype = "B", "float32"
+    d = model_dirs[(name, "float32")]
+    reqs = rh.make_requests(384, [40, 40, 40, 40, 40, 40, 40, 40], seed=3)
+    steps = rh.trace_mixed(reqs, seed=2, max_live=2, max_portion=16)
+    runner = make_runner(d, dtype, name, n_tokens=rh.peak_tokens(steps, rounding=16))
+    seen_pages = set()
+    got = rh.run_in_process(runner, steps)
+    rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, "reuse")
+    assert runner.manager.pools[0].n_pages * 16 < sum(len(t) for t in reqs.values())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_dirs, dtype):
+    """A short prompt and 400 tokens one by one, past the window and over many pages."""
+    name = "C"
+    d = model_dirs[(name, STORE[dtype])]
+    reqs = rh.make_requests(300, [420], seed=9)
+    steps = rh.trace_tail(reqs, tail=400)
+    runner = make_runner(d, dtype, name, n_tokens=448)
+    got = rh.run_in_process(runner, steps)
+    rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, "long decoding")
+    # the window let pages go while the request was alive
+    assert len(got) == 420
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens(model_dirs, runners, name, dtype):
+    """Prompts of one, two and three tokens: position 0 sees itself only."""
+    d = model_dirs[(name, STORE[dtype])]
+    reqs = rh.make_requests(TINY[name]["config"]["vocab_size"], [1, 2, 3], seed=21)
+    runner = runners(name, dtype)
+    ref = rh.plain_logits(d, reqs)
+    rh.compare(rh.run_in_process(runner, rh.trace_whole(reqs)), reqs, ref, dtype, "first tokens whole")
+    rh.compare(rh.run_in_process(runner, rh.trace_tail(reqs, tail=2)), reqs, ref, dtype, "first tokens one by one")
+
+
+def test_logits_do_not_depend_on_neighbours(model_dirs, runners):
+    """The same request alone and beside three others: bit for bit the same with the plain
+    kernels of the 32-bit path (every row is reduced in a fixed order)."""
+    name = "A"
+    reqs = requests_for(name)
+    runner = runners(name, "float32")
+    alone = rh.run_in_process(runner, rh.trace_whole({"r3": reqs["r3"]}))
+    steps = [dict(entries=[dict(id=r, tokens=reqs[r], want=list(range(len(reqs[r])))) for r in ("r1", "r3", "r0", "r4")],
+                  end=["r1", "r3", "r0", "r4"])]
+    together = rh.run_in_process(runner, steps)
+    for p in range(len(reqs["r3"])):
+        assert np.array_equal(alone[("r3", p)], together[("r3", p)])
+
+
+def test_step_refuses_bad_batches(model_dirs, runners):
+    from flambeau_amd.cache import CacheError
+    from flambeau_amd.engine import StepEntry, StepError
+    runner = runners("A", "float32")
+    with pytest.raises(StepError, match="not live"):
+        runner.step([StepEntry("x", [1])])
+    assert runner.begin("x")
+    with pytest.raises(StepError, match="twice"):
+        runner.step([StepEntry("x", [1]), StepEntry("x", [2])])
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        runner.step([StepEntry("x", [256])])
+    with pytest.raises(StepError, match="wanted place"):
+        runner.step([StepEntry("x", [1, 2], [2])])
+    with pytest.raises(StepError, match="no tokens"):
+        runner.step([StepEntry("x", [])])
+    with pytest.raises(CacheError):
+        runner.step([StepEntry("x", [1] * 129)])          # beyond max_position_embeddings = 128
+    assert runner.cached_tokens("x") == 0                 # refused steps changed nothing
+    runner.end("x")
+    runner.manager.check_invariants()
+
+
+# ---------------------------------------------------------------- generation through the entry point
+def _plain_generate(d, prompt, n_new, temperature=0.0, seed=0):
+    cfg, w = pm.read_model_dir(d)
+    rng = pm.Xoshiro(seed)
+    toks, margins = list(prompt), []
+    for _ in range(n_new):
+        logits = pm.forward(cfg, w, toks)[-1].astype(np.float32)
+        s = np.sort(logits)
+        margins.append(float(s[-1] - s[-2]))
+        toks.append(pm.sample(logits, rng, temperature=temperature))
+    return toks[len(prompt):], margins
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(model_dirs, dtype):
+    """Workload of the first tiny configuration: prompts of 5, 12, 23 and 40 tokens, 16 greedy
+    tokens each, pages of 8, all four requests in flight with portions of 16."""
+    from flambeau_amd import generate
+    name = "A"
+    d = model_dirs[(name, STORE[dtype])]
+    prompts = list(rh.make_requests(256, [5, 12, 23, 40], seed=1).values())
+    outs = generate(str(d), prompts, max_new_tokens=16, dtype=dtype, page_size=8, inflight_slots=4,
+                    prefill_chunk_tokens=16, paged_kv=40)
+    tie = 1e-4 if dtype == "float32" else 2e-2
+    for prompt, out in zip(prompts, outs):
+        want, margins = _plain_generate(d, prompt, 16)
+        assert len(out) == 16
+        for i, (a, b) in enumerate(zip(out, want)):
+            if a != b:
+                assert margins[i] < tie, f"token {i}: engine {a}, plain {b}, margin {margins[i]}"
+                break
+
+
+def test_temperature_generation_through_the_entry_point(model_dirs):
+    """Workload of the second tiny configuration: prompts of 1, 31 and 97 tokens, 24 tokens each,
+    one greedy and two at temperature 0.8 with seeded draws; pages of 16."""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    d = model_dirs[("B", "float32")]
+    prompts = list(rh.make_requests(384, [1, 31, 97], seed=3).values())
+    temps, seeds = [0.0, 0.8, 0.8], [100, 101, 102]
+    eng = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", page_size=16, inflight_slots=3,
+                                                   prefill_chunk_tokens=32, paged_kv=24))
+    outs = eng.generate(prompts, [SamplingParams(temperature=t, seed=s, max_tokens=24) for t, s in zip(temps, seeds)])
+    for prompt, out, t, s in zip(prompts, outs, temps, seeds):
+        want, _ = _plain_generate(d, prompt, 24, temperature=t, seed=s)
+        assert out == want
+    # the host sampler (filters) takes the same path through the scheduler
+    outs2 = eng.generate(prompts[:2], [SamplingParams(temperature=0.8, top_k=384, seed=s, max_tokens=8) for s in seeds[:2]])
+    assert all(len(o) == 8 for o in outs2)
+    assert not eng.runner.manager.live and eng.runner.manager.free_pages() == [24]
+
+
+def test_generation_survives_preemption(model_dirs):
+    """So few pages that running requests are pre-empted and recomputed: the tokens stay the same."""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    d = model_dirs[("B", "float32")]
+    prompts = list(rh.make_requests(384, [30, 30, 30], seed=4).values())
+    roomy = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", inflight_slots=3, paged_kv=24, prefill_chunk_tokens=64))
+    want = roomy.generate(prompts, SamplingParams(max_tokens=30))
+    tight = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", inflight_slots=3, paged_kv=8, prefill_chunk_tokens=64))
+    got = tight.generate(prompts, SamplingParams(max_tokens=30))
+    assert tight.scheduler.n_preemptions > 0
+    assert got == want

@@ -40,3 +40,21 @@ def write_tiny(name, out_dir, store="float32"):
     t = TINY[name]
     return write_random_model(t["config"], out_dir, seed=t["seed"], std=t["std"], gain_std=t["gain_std"],
                               store_dtype=STORE[store])
+
+
+def write_sharpened(name, out_dir, store="float32", factor=12.0):
+    """The tiny model with its query and key matrices scaled up, so that attention is peaked:
+    single keys (far ones, those at a window's edge, those at a page's edge) carry visible
+    weight and a fault in any one of them shows in the logits."""
+    from flambeau_amd.weights import SafetensorsFile, write_safetensors
+    d = write_tiny(name, out_dir, store)
+    f = SafetensorsFile(d / "model.safetensors")
+    tensors = {}
+    for n in f.names():
+        t = f.read(n)
+        if n.endswith("q_proj.weight") or n.endswith("k_proj.weight"):
+            t = (t.float() * factor).to(t.dtype)
+        tensors[n] = t
+    f.close()
+    write_safetensors(d / "model.safetensors", tensors)
+    return d
