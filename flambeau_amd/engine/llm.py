@@ -76,6 +76,9 @@ class LLMEngine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
+    def abort(self, request_id) -> bool:
+        return self.scheduler.abort(request_id)
+
     # ------------------------------------------------------------ one step
     def step(self) -> list[Request]:
         """Schedule, run, sample, commit.  Returns the requests that finished in this step."""

@@ -125,6 +125,21 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
+    def abort(self, request_id) -> bool:
+        """Drop a request wherever it is; its pages and slot are given back."""
+        for r in list(self.waiting):
+            if r.request_id == request_id:
+                self.waiting.remove(r)
+                r.status, r.finish_reason = "finished", "abort"
+                return True
+        for r in self.running:
+            if r.request_id == request_id:
+                self.running.remove(r)
+                self.manager.release(request_id)
+                r.status, r.finish_reason = "finished", "abort"
+                return True
+        return False
+
     # ------------------------------------------------------------ scheduling
     def _free_after(self, planned) -> list[int]:
         """Free pages per group once the planned entries have taken theirs."""

@@ -194,3 +194,17 @@ def test_random_workloads_finish_and_keep_the_books(seed):
     for r, n_new in reqs:
         assert r.status == "finished" and len(r.output) == n_new and r.output == [100 + i for i in range(n_new)]
     assert m.free_pages() == [10] and m.n_free_slots == 3
+
+
+def test_abort_gives_everything_back():
+    m, s = mk(slots=2)
+    s.add("a", list(range(10)), SamplingParams(max_tokens=5))
+    s.add("b", list(range(10)), SamplingParams(max_tokens=5))
+    s.add("c", [1, 2], SamplingParams(max_tokens=5))
+    run_step(m, s)
+    assert s.abort("a") and s.abort("c") and not s.abort("zz")
+    assert [r.request_id for r in s.running] == ["b"] and not s.waiting
+    m.check_invariants()
+    while s.has_work():
+        run_step(m, s)
+    assert m.free_pages() == [16] and m.n_free_slots == 2

@@ -1,0 +1,56 @@
+"""bin/trace_run as a program: the same requests whole, with the last 32 tokens one by one, in
+portions of changing size, and mixed with so few pages that they are used again; in 32-bit and
+in bfloat16; all compared with the plain implementation."""
+import json
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import replay_helpers as rh
+from tiny_configs import TINY
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_replay_in_all_cuttings(model_dirs, tmp_path, name, dtype):
+    d = model_dirs[(name, dtype)]
+    vocab = TINY[name]["config"]["vocab_size"]
+    lengths = {"A": [40, 70, 97, 33, 64, 12], "B": [97, 1, 150, 64, 31, 33]}[name]
+    reqs = rh.make_requests(vocab, lengths, seed=5)
+    ref = rh.plain_logits(d, reqs)
+    for mode, steps in [("whole", rh.trace_whole(reqs)), ("tail", rh.trace_tail(reqs)),
+                        ("portions", rh.trace_portions(reqs)), ("mixed", rh.trace_mixed(reqs, seed=13))]:
+        out = tmp_path / mode
+        got = rh.run_program(d, dtype, steps, out, rh.peak_tokens(steps), vocab)
+        assert got, mode
+        rh.compare(got, reqs, ref, dtype, f"trace_run {name} {mode}")
+
+
+def test_replay_details(model_dirs, tmp_path):
+    """A request may sit out a step; a step may want nothing (no file) or hold no entries; files
+    are little-endian float32 [wanted, vocab] in the order of entries and of want."""
+    d = model_dirs[("A", "float32")]
+    reqs = rh.make_requests(256, [10, 6], seed=8)
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [
+        dict(entries=[dict(id="r0", tokens=a[:4], want=[])], end=[]),
+        dict(entries=[dict(id="r1", tokens=b[:3], want=[2, 0])], end=[]),
+        dict(entries=[], end=[]),
+        dict(entries=[dict(id="r1", tokens=b[3:], want=[2]), dict(id="r0", tokens=a[4:], want=[5, 0])], end=["r0", "r1"]),
+    ]
+    lines = "".join(json.dumps(dict(step=10 + i, **s)) + "\n" for i, s in enumerate(steps))
+    out = tmp_path / "o"
+    r = subprocess.run([sys.executable, str(rh.ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128"], input=lines, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert r.stdout.split() == ["done", "10", "done", "11", "done", "12", "done", "13"]
+    assert sorted(p.name for p in out.iterdir()) == ["11.f32", "13.f32"]
+    ref = rh.plain_logits(d, reqs)
+    s11 = np.fromfile(out / "11.f32", dtype="<f4").reshape(2, 256)
+    s13 = np.fromfile(out / "13.f32", dtype="<f4").reshape(3, 256)
+    for row, (rid, p) in zip(list(s11) + list(s13), [("r1", 2), ("r1", 0), ("r1", 5), ("r0", 9), ("r0", 4)]):
+        assert np.abs(row - ref[rid][p]).max() < 1e-4
