@@ -35,6 +35,10 @@ int fl_argmax(const float* logits, int* out, int rows, int V, hipStream_t stream
 int fl_sample(const float* logits, const float* inv_temp, const float* uniform, int* out,
               int rows, int V, hipStream_t stream);
 
+// ---- tuned bf16 kernels ----
+int fl_gemm_skinny(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K,
+                   hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

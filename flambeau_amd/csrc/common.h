@@ -49,8 +49,11 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
     return t;
 }
 
-// Paged cache of one layer: [n_pages][2 (K,V)][n_kv_heads][page_size][head_dim].
-// Token t of a request lives in page table[t / page_size] at row t % page_size.
+// Paged cache of one layer: [n_pages][2 (K,V)][n_kv_heads][page_size * head_dim].
+// Token t of a request lives in page table[t / page_size] at row r = t % page_size.
+// Within a (page, head) block keys are stored row by row, K[r][d] at r * head_dim + d,
+// and values transposed, V[r][d] at d * page_size + r: matrix-core operands want the index
+// that is summed over (head dims for Q.K, keys for P.V) contiguous in memory.
 struct PagedCache {
     void* base;        // this layer's pool
     int n_kv_heads;
@@ -59,10 +62,14 @@ struct PagedCache {
     int n_pages;
 };
 
-__device__ __forceinline__ size_t cache_row_offset(const PagedCache& c, int page, int is_v,
-                                                   int kv_head, int row) {
-    return ((((size_t)page * 2 + is_v) * c.n_kv_heads + kv_head) * c.page_size + row) *
-           (size_t)c.head_dim;
+__device__ __forceinline__ size_t cache_block_offset(const PagedCache& c, int page, int is_v, int kv_head) {
+    return (((size_t)page * 2 + is_v) * c.n_kv_heads + kv_head) * (size_t)c.page_size * c.head_dim;
+}
+__device__ __forceinline__ size_t cache_k_offset(const PagedCache& c, int page, int kv_head, int row, int d) {
+    return cache_block_offset(c, page, 0, kv_head) + (size_t)row * c.head_dim + d;
+}
+__device__ __forceinline__ size_t cache_v_offset(const PagedCache& c, int page, int kv_head, int row, int d) {
+    return cache_block_offset(c, page, 1, kv_head) + (size_t)d * c.page_size + row;
 }
 
 // ---- host side -----------------------------------------------------------

@@ -1,0 +1,148 @@
+// Skinny bf16 matrix product for decode: out[m, n] = sum_k x[m, k] w[n, k] with few rows m
+// (up to 64) and a large weight matrix that is read exactly once.  The product is bound by the
+// stream of w out of HBM, so the kernel is built around that stream:
+//
+//  * a block owns 16 consecutive output features (rows of w); its NW waves split K between
+//    them and add their partial sums through LDS in a fixed order (no atomics: the result
+//    does not depend on timing);
+//  * a wave keeps 8 (or 16) 16-byte loads of w in flight per lane before it consumes them;
+//    within an iteration over 256 values of k, lane (i, g) reads the 128 contiguous bytes
+//    w[row i][k0 + 64 g .. k0 + 64 g + 63]; w is loaded with the non-temporal hint so that it
+//    does not push x out of the caches;
+//  * the arithmetic is v_mfma_f32_16x16x32_bf16 with w as the A operand (16 features x 32 k)
+//    and x as the B operand (32 k x 16 tokens): C[feature][token] leaves each lane with four
+//    consecutive features of one token, i.e. one 16-byte store.  Rows of x beyond M are not
+//    loaded.  With MT > 1 the same w registers feed MT token tiles.
+//
+// The reference's nearest kernels are its float GEMV, one block per output row
+// (crates/kernels-hip/src/kernels/dense_gemv_f16_f16.cu:27-71, ..._batched.cu:17-63).
+#include "common.h"
+#include "api.h"
+
+__device__ __forceinline__ void store4(float* p, f32x4 v) { *(f32x4*)p = v; }
+__device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
+    bf16x4 o = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+    *(bf16x4*)p = o;
+}
+
+template <int MT, typename TOut>
+__global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
+                                                           const bf16_t* __restrict__ w,
+                                                           TOut* __restrict__ out, int M, int N, int K,
+                                                           int vec_out) {
+    extern __shared__ float red[];               // [NW][MT][64][4]
+    const int nw = blockDim.x >> 6;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int li = lane & 15, g = lane >> 4;
+    const int row = min(blockIdx.x * 16 + li, N - 1);
+    const bf16_t* wrow = w + (size_t)row * K;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // K in steps of 32; this wave's steps [s0, s1)
+    const int n_steps = (K + 31) >> 5;
+    const int per = (n_steps + nw - 1) / nw;
+    const int s0 = wave * per, s1 = min(n_steps, s0 + per);
+
+    const bf16_t* xrow[MT];
+    bool xok[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int tok = mt * 16 + li;
+        xok[mt] = tok < M;
+        xrow[mt] = x + (size_t)min(tok, M - 1) * K;
+    }
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    int s = s0;
+    // full iterations: 8 steps = 256 values of k, all inside K
+    for (; s + 8 <= s1 && (s + 8) * 32 <= K; s += 8) {
+        const int kb = s * 32 + 64 * g;
+        bf16x8 a[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] = __builtin_nontemporal_load((const bf16x8*)(wrow + kb + 8 * j));
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            bf16x8 b[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) b[j] = xok[mt] ? *(const bf16x8*)(xrow[mt] + kb + 8 * j) : zero;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);
+        }
+    }
+    // remaining steps one by one; a chunk of 8 values that reaches beyond K counts as zero
+    for (; s < s1; ++s) {
+        const int k = s * 32 + 8 * g;
+        const bool in = k + 8 <= K;
+        const bf16x8 a = in ? __builtin_nontemporal_load((const bf16x8*)(wrow + k)) : zero;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const bf16x8 b = (in && xok[mt]) ? *(const bf16x8*)(xrow[mt] + k) : zero;
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+        }
+    }
+
+    // add the waves' partial sums in wave order
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *(f32x4*)(red + (((size_t)wave * MT + mt) * 64 + lane) * 4) = acc[mt];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            f32x4 sum = *(f32x4*)(red + ((size_t)mt * 64 + lane) * 4);
+            for (int ww = 1; ww < nw; ++ww) {
+                const f32x4 v = *(f32x4*)(red + (((size_t)ww * MT + mt) * 64 + lane) * 4);
+                sum += v;
+            }
+            // lane (token li, group g) holds features 16*block + 4g .. 4g+3 of token mt*16 + li
+            const int tok = mt * 16 + li;
+            const int f0 = blockIdx.x * 16 + 4 * g;
+            if (tok < M && f0 < N) {
+                TOut* p = out + (size_t)tok * N + f0;
+                if (vec_out && f0 + 4 <= N) {
+                    store4(p, sum);
+                } else {
+                    for (int r = 0; r < 4 && f0 + r < N; ++r) p[r] = from_f32<TOut>(sum[r]);
+                }
+            }
+        }
+    }
+}
+
+template <int MT, typename TOut>
+static int launch_skinny(const bf16_t* x, const bf16_t* w, TOut* out, int M, int N, int K, hipStream_t stream) {
+    const int groups = ceil_div(N, 16);
+    // enough waves in flight to cover the memory latency: about 2048 and more over the chip
+    int nw = 4;
+    while (nw < 16 && groups * nw < 2048) nw *= 2;
+    while (nw > 1 && ceil_div(K, 32) < nw * 2) nw /= 2;
+    const size_t lds = (size_t)nw * MT * 64 * 4 * sizeof(float);
+    const int vec_out = (N % 4 == 0) ? 1 : 0;      // 16-byte stores need aligned rows
+    gemm_skinny_kernel<MT, TOut><<<groups, nw * 64, lds, stream>>>(x, w, out, M, N, K, vec_out);
+    return 0;
+}
+
+extern "C" int fl_gemm_skinny(const void* x, const void* w, void* out, int out_dtype, int M, int N,
+                              int K, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+    FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
+    FL_CHECK(K % 8 == 0, "gemm_skinny: K=%d is no multiple of 8 (16-byte loads)", K);
+    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0),
+             "gemm_skinny: operands must be 16-byte aligned");
+    if (M == 0) return 0;
+    const int mt = ceil_div(M, 16);
+#define FL_SK(MT_)                                                                                         \
+    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w, (float*)out, M, N, K, stream); \
+    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)out, M, N, K, stream)
+    FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
+    switch (mt) {
+        case 1: FL_SK(1); break;
+        case 2: FL_SK(2); break;
+        case 3: FL_SK(3); break;
+        default: FL_SK(4); break;
+    }
+#undef FL_SK
+    FL_LAUNCH_CHECK();
+    return 0;
+}

@@ -187,6 +187,7 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const int pos = positions[token];
     const TIn* src = qkv + (size_t)token * ld + (size_t)head * hd;
     T* dst;
+    size_t stride = 1;      // distance between consecutive head dims at the destination
     bool rotate;
     if (head < nh) {
         dst = q_out + ((size_t)token * nh + head) * hd;
@@ -197,7 +198,13 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
         const int is_v = (head - nh) / nkv;
         const int page = block_table[(size_t)tok_seq[token] * max_blocks + pos / cache.page_size];
         if (page < 0 || page >= cache.n_pages) return;  // padding rows of a fixed-size batch
-        dst = (T*)cache.base + cache_row_offset(cache, page, is_v, kvh, pos % cache.page_size);
+        const int row = pos % cache.page_size;
+        if (is_v) {
+            dst = (T*)cache.base + cache_v_offset(cache, page, kvh, row, 0);
+            stride = cache.page_size;
+        } else {
+            dst = (T*)cache.base + cache_k_offset(cache, page, kvh, row, 0);
+        }
         rotate = !is_v;
     }
     const int half = rot >> 1;
@@ -213,7 +220,7 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
         }
         for (int i = rot + threadIdx.x; i < hd; i += 64) dst[i] = from_f32<T>(to_f32(src[i]));
     } else {
-        for (int i = threadIdx.x; i < hd; i += 64) dst[i] = from_f32<T>(to_f32(src[i]));
+        for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * stride] = from_f32<T>(to_f32(src[i]));
     }
 }
 
@@ -274,8 +281,9 @@ __global__ __launch_bounds__(256) void attn_plain_kernel(
         const int page = table[t / cache.page_size];
         if (page < 0 || page >= cache.n_pages) continue;
         const int row = t % cache.page_size;
-        const T* kr = (const T*)cache.base + cache_row_offset(cache, page, 0, kvh, row);
-        const T* vr = (const T*)cache.base + cache_row_offset(cache, page, 1, kvh, row);
+        const T* kr = (const T*)cache.base + cache_k_offset(cache, page, kvh, row, 0);
+        const T* vr = (const T*)cache.base + cache_v_offset(cache, page, kvh, row, 0);
+        const int vs = cache.page_size;
         float part = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -289,7 +297,7 @@ __global__ __launch_bounds__(256) void attn_plain_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int d = lane + 64 * j;
-            if (d < hd) acc[j] = acc[j] * corr + pe * to_f32(vr[d]);
+            if (d < hd) acc[j] = acc[j] * corr + pe * to_f32(vr[(size_t)d * vs]);
         }
         l = l * corr + pe;
         m = m_new;

@@ -1,0 +1,325 @@
+"""Each kernel alone against a plain torch reference of the same op, at other sizes than the
+engine tests use (among them the 7B model's).  The tuned bf16 kernels are also compared with
+their plain kernels."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def ops():
+    from flambeau_amd.kernels import ops as o
+    return o
+
+
+def tuned():
+    from flambeau_amd.kernels import tuned as t
+    return t
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+# ---------------------------------------------------------------- element-wise and norm kernels
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V,H,n", [(300, 80, 7), (32768, 4096, 33), (5, 3, 1)])
+def test_embed(dtype, V, H, n):
+    table = rnd(V, H, dtype=dtype)
+    tokens = torch.randint(0, V, (n,), dtype=torch.int32, device=DEV)
+    out = torch.empty(n, H, dtype=torch.float32, device=DEV)
+    ops().embed(table, tokens, out)
+    assert torch.equal(out, table[tokens.long()].float())
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,H,eps", [(5, 96, 1e-6), (3, 4096, 1e-5), (17, 250, 1e-2), (2, 5120, 1e-5)])
+def test_rmsnorm_variants(out_dtype, n, H, eps):
+    x = rnd(n, H, seed=1)
+    d = rnd(n, H, seed=2, scale=0.3)
+    w = 1 + 0.1 * rnd(H, seed=3)
+    tol = 1e-5 if out_dtype == torch.float32 else 1e-2
+
+    def ref(v):
+        v = v.double()
+        return (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * w.double())
+
+    out = torch.empty(n, H, dtype=out_dtype, device=DEV)
+    ops().rmsnorm(x, w, out, eps)
+    assert (out.double() - ref(x)).abs().max() < tol * ref(x).abs().max()
+    # with the pending delta added and stored back
+    x2 = x.clone()
+    ops().rmsnorm(x2, w, out, eps, delta=d, store_sum=True)
+    assert torch.equal(x2, x + d)
+    assert (out.double() - ref(x + d)).abs().max() < tol * ref(x + d).abs().max()
+    # gathered rows, nothing stored
+    rows = torch.tensor([n - 1, 0, n // 2], dtype=torch.int32, device=DEV)
+    out3 = torch.empty(3, H, dtype=out_dtype, device=DEV)
+    x3 = x.clone()
+    ops().rmsnorm(x3, w, out3, eps, delta=d, rows=rows)
+    assert torch.equal(x3, x)
+    assert (out3.double() - ref(x + d)[rows.long()]).abs().max() < tol * ref(x + d).abs().max()
+
+
+def test_add_and_silu_mul():
+    x, d = rnd(37, 1000, seed=4), rnd(37, 1000, seed=5)
+    want = x + d
+    ops().add_inplace(x, d)
+    assert torch.equal(x, want)
+    for n, I in [(3, 224), (9, 14336), (1, 5)]:
+        gu = rnd(n, 2 * I, seed=6, scale=3.0)
+        ref = (gu[:, :I].double() / (1 + torch.exp(-gu[:, :I].double()))) * gu[:, I:].double()
+        o32 = torch.empty(n, I, dtype=torch.float32, device=DEV)
+        ops().silu_mul(gu, o32)
+        assert torch.allclose(o32.double(), ref, rtol=2e-6, atol=1e-6)     # float32 rounding of values up to 100
+        o16 = torch.empty(n, I, dtype=torch.bfloat16, device=DEV)
+        ops().silu_mul(gu, o16)
+        assert (o16.double() - ref).abs().max() < 1e-2 * ref.abs().max()
+
+
+# ---------------------------------------------------------------- matrix products
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (7, 100, 36), (65, 130, 250), (33, 384, 96), (2, 6144, 4096)])
+def test_gemm_plain_float32(M, N, K):
+    x, w = rnd(M, K, seed=7), rnd(N, K, seed=8)
+    out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops().gemm_plain(x, w, out)
+    ref = x.double() @ w.double().T
+    assert (out.double() - ref).abs().max() < 2e-6 * math.sqrt(K) * ref.abs().max().clamp(min=1)
+
+
+def test_gemm_plain_rows_do_not_depend_on_the_batch():
+    x, w = rnd(70, 300, seed=9), rnd(200, 300, seed=10)
+    full = torch.empty(70, 200, dtype=torch.float32, device=DEV)
+    ops().gemm_plain(x, w, full)
+    one = torch.empty(1, 200, dtype=torch.float32, device=DEV)
+    ops().gemm_plain(x[41:42].contiguous(), w, one)
+    assert torch.equal(one[0], full[41])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 6144, 4096), (1, 4096, 14336), (64, 1024, 512),
+                                   (3, 100, 72), (17, 250, 40), (5, 16, 8), (33, 28672, 4096), (1, 32768, 4096),
+                                   (16, 37, 264), (49, 300, 80)])
+def test_gemm_skinny_against_plain(out_dtype, M, N, K):
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=11), rnd(N, K, dtype=torch.bfloat16, seed=12, scale=0.05)
+    got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+    tuned().gemm_skinny(x, w, got)
+    ref = x.double() @ w.double().T
+    plain = torch.empty(M, N, dtype=out_dtype, device=DEV)
+    ops().gemm_plain(x, w, plain)
+    scale = ref.abs().max()
+    tol = 1e-5 if out_dtype == torch.float32 else 5e-3
+    assert (got.double() - ref).abs().max() < tol * scale
+    assert (got.double() - plain.double()).abs().max() < 2 * tol * scale
+
+
+def test_gemm_skinny_refuses_what_it_cannot_do():
+    from flambeau_amd.kernels import KernelError
+    x, w = rnd(2, 36, dtype=torch.bfloat16), rnd(5, 36, dtype=torch.bfloat16)
+    out = torch.empty(2, 5, dtype=torch.float32, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 8"):
+        tuned().gemm_skinny(x, w, out)
+    tuned().gemm(x, w, out)            # the dispatcher takes the plain kernel instead
+    assert (out.double() - x.double() @ w.double().T).abs().max() < 1e-4
+    with pytest.raises(KernelError, match="at most 64"):
+        tuned().gemm_skinny(rnd(65, 64, dtype=torch.bfloat16), rnd(8, 64, dtype=torch.bfloat16),
+                            torch.empty(65, 8, dtype=torch.float32, device=DEV))
+    with pytest.raises(KernelError, match="shape"):
+        tuned().gemm_skinny(rnd(2, 64, dtype=torch.bfloat16), rnd(8, 32, dtype=torch.bfloat16), out)
+
+
+# ---------------------------------------------------------------- cache, rotation, attention
+def make_cache(n_pages, nkv, ps, hd, dtype):
+    from flambeau_amd.kernels.ops import PagedLayerCache
+    return PagedLayerCache(torch.zeros(n_pages, 2, nkv, ps, hd, dtype=dtype, device=DEV))
+
+
+def read_cache(cache, table_row, t, kvh):
+    """Key and value rows of token t through the block table (V is stored transposed in a page)."""
+    ps, hd = cache.page_size, cache.head_dim
+    page, r = int(table_row[t // ps]), t % ps
+    k = cache.pool[page, 0, kvh].reshape(ps, hd)[r]
+    v = cache.pool[page, 1, kvh].reshape(hd, ps)[:, r]
+    return k, v
+
+
+def rope_ref(x, pos, theta, rot):
+    """x [n, heads, hd] double."""
+    half = rot // 2
+    inv = theta ** (-2.0 * torch.arange(half, dtype=torch.float64, device=x.device) / rot)
+    ang = pos.double()[:, None] * inv[None]
+    c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
+    out = x.clone()
+    lo, hi = x[..., :half], x[..., half:rot]
+    out[..., :half] = lo * c - hi * s
+    out[..., half:rot] = lo * s + hi * c
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,ps,rot,theta", [(4, 2, 16, 8, 16, 1e4), (6, 1, 24, 16, 24, 1e6),
+                                                   (32, 8, 128, 16, 128, 1e6), (3, 3, 40, 4, 20, 5e5),
+                                                   (2, 1, 64, 32, 0, 1.0)])
+def test_rope_kv_write(dtype, nh, nkv, hd, ps, rot, theta):
+    seqs = [(0, 5), (37, 3), (ps - 1, 2), (100, 1)]          # (start position, tokens)
+    n = sum(q for _, q in seqs)
+    n_pages = 96
+    cache = make_cache(n_pages, nkv, ps, hd, dtype)
+    perm = torch.randperm(n_pages)
+    table = torch.full((len(seqs), 56), -1, dtype=torch.int32)
+    used = 0
+    pos, tok_seq = [], []
+    for s, (st, q) in enumerate(seqs):
+        nb = -(-(st + q) // ps)
+        table[s, :nb] = perm[used:used + nb].int()
+        used += nb
+        pos += list(range(st, st + q))
+        tok_seq += [s] * q
+    pos_d = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    seq_d = torch.tensor(tok_seq, dtype=torch.int32, device=DEV)
+    qkv = rnd(n, (nh + 2 * nkv) * hd, seed=13)
+    q_out = torch.empty(n, nh * hd, dtype=dtype, device=DEV)
+    ops().rope_kv_write(qkv, pos_d, seq_d, table.to(DEV), q_out, cache, nh, rot, theta)
+    x = qkv.double()
+    q_ref = x[:, :nh * hd].reshape(n, nh, hd)
+    k_ref = x[:, nh * hd:(nh + nkv) * hd].reshape(n, nkv, hd)
+    v_ref = x[:, (nh + nkv) * hd:].reshape(n, nkv, hd)
+    if rot:
+        q_ref, k_ref = rope_ref(q_ref, pos_d, theta, rot), rope_ref(k_ref, pos_d, theta, rot)
+    tol = 2e-5 if dtype == torch.float32 else 1e-2
+    assert (q_out.double().reshape(n, nh, hd) - q_ref).abs().max() < tol * 4
+    for i in range(n):
+        for h in range(nkv):
+            k, v = read_cache(cache, table[tok_seq[i]], pos[i], h)
+            assert (k.double() - k_ref[i, h]).abs().max() < tol * 4
+            assert (v.double() - v_ref[i, h]).abs().max() < tol * 4
+    # nothing else was touched: untouched pages are still zero
+    touched = set(int(p) for p in table[table >= 0])
+    for p in range(n_pages):
+        if p not in touched:
+            assert not cache.pool[p].any()
+
+
+def attention_ref(q, keys, vals, pos, scale, window):
+    """One query row per call site: q [nh, hd], keys/vals [T, nkv, hd] double, query at ``pos``."""
+    nh, nkv = q.shape[0], keys.shape[1]
+    lo = max(0, pos - window + 1) if window else 0
+    out = torch.zeros_like(q)
+    for h in range(nh):
+        g = h // (nh // nkv)
+        s = (keys[lo:pos + 1, g] @ q[h]) * scale
+        p = torch.softmax(s, 0)
+        out[h] = p @ vals[lo:pos + 1, g]
+    return out
+
+
+def build_attention_case(dtype, nh, nkv, hd, ps, seqs, seed=0):
+    """Random cache contents for requests ``seqs`` = (context length, query length); the queries
+    are the last ``q`` positions of each.  Returns what the kernels take and the reference."""
+    torch.manual_seed(seed)
+    n_pages = sum(-(-c // ps) for c, _ in seqs) + 3
+    cache = make_cache(n_pages, nkv, ps, hd, dtype)
+    perm = torch.randperm(n_pages)
+    width = max(-(-c // ps) for c, _ in seqs) + 1
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    used = 0
+    K, V = [], []
+    for s, (c, _) in enumerate(seqs):
+        nb = -(-c // ps)
+        table[s, :nb] = perm[used:used + nb].int()
+        used += nb
+        k = (torch.randn(c, nkv, hd) * 0.8).to(dtype)
+        v = torch.randn(c, nkv, hd).to(dtype)
+        K.append(k.double().to(DEV))
+        V.append(v.double().to(DEV))
+        for t in range(c):
+            page, r = int(table[s, t // ps]), t % ps
+            cache.pool[page, 0].reshape(nkv, ps, hd)[:, r] = k[t].to(DEV)
+            cache.pool[page, 1].reshape(nkv, hd, ps)[:, :, r] = v[t].to(DEV)
+    pos, tok_seq = [], []
+    for s, (c, ql) in enumerate(seqs):
+        pos += list(range(c - ql, c))
+        tok_seq += [s] * ql
+    n = len(pos)
+    q = (torch.randn(n, nh, hd) * 0.8).to(dtype).to(DEV)
+    return dict(cache=cache, table=table.to(DEV), K=K, V=V, pos=pos, tok_seq=tok_seq, q=q, n=n,
+                pos_d=torch.tensor(pos, dtype=torch.int32, device=DEV),
+                seq_d=torch.tensor(tok_seq, dtype=torch.int32, device=DEV))
+
+
+def attention_case_ref(case, scale, window):
+    outs = []
+    for i in range(case["n"]):
+        s = case["tok_seq"][i]
+        outs.append(attention_ref(case["q"][i].double(), case["K"][s], case["V"][s], case["pos"][i], scale, window))
+    return torch.stack(outs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,ps,window", [(4, 2, 16, 8, 0), (6, 1, 24, 16, 11), (8, 2, 128, 16, 0),
+                                                (5, 5, 72, 4, 30), (2, 2, 256, 32, 0), (3, 1, 10, 2, 5)])
+def test_attn_plain(dtype, nh, nkv, hd, ps, window):
+    seqs = [(70, 70), (33, 1), (ps * 3, 2), (1, 1), (50, 9)]
+    case = build_attention_case(dtype, nh, nkv, hd, ps, seqs)
+    scale = 1 / math.sqrt(hd)
+    out = torch.empty(case["n"], nh * hd, dtype=dtype, device=DEV)
+    ops().attn_plain(case["q"].reshape(case["n"], nh * hd), out, case["cache"], case["pos_d"], case["seq_d"],
+                     case["table"], nh, scale, window)
+    ref = attention_case_ref(case, scale, window)
+    tol = 2e-6 if dtype == torch.float32 else 1e-2
+    assert (out.double().reshape(case["n"], nh, hd) - ref).abs().max() < tol * ref.abs().max()
+
+
+def test_attn_plain_refuses_large_heads():
+    from flambeau_amd.kernels import KernelError
+    case = build_attention_case(torch.float32, 1, 1, 8, 4, [(4, 1)])
+    big = make_cache(2, 1, 4, 264, torch.float32)
+    with pytest.raises(KernelError, match="head size 264"):
+        ops().attn_plain(torch.zeros(1, 264, device=DEV), torch.zeros(1, 264, device=DEV), big, case["pos_d"],
+                         case["seq_d"], case["table"], 1, 1.0, 0)
+
+
+# ---------------------------------------------------------------- sampling
+@pytest.mark.parametrize("R,V", [(1, 10), (5, 384), (3, 32768), (8, 131072), (2, 257)])
+def test_argmax_first_maximum_wins(R, V):
+    logits = rnd(R, V, seed=14)
+    logits[0, V // 3] = 50.0
+    logits[0, V - 1] = 50.0            # a later tie loses
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops().argmax(logits, out)
+    want = [int(np.argmax(row)) for row in logits.cpu().numpy()]
+    assert out.tolist() == want and out[0] == V // 3
+
+
+@pytest.mark.parametrize("V", [97, 384, 32768])
+def test_sample_is_the_inverse_cdf_in_index_order(V):
+    import plain_model as pm
+    R = 64
+    logits = rnd(R, V, seed=15, scale=2.0)
+    u = torch.rand(R, generator=torch.Generator().manual_seed(1)).to(DEV)
+    u[0], u[1] = 0.0, 0.999999
+    inv_t = torch.full((R,), 1 / 0.8, device=DEV)
+    inv_t[2] = 0.0                                       # greedy row among the others
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops().sample(logits, inv_t, u, out)
+    l, uu = logits.cpu().double().numpy(), u.cpu().double().numpy()
+    assert out[2] == int(np.argmax(l[2]))
+    bad = 0
+    for r in range(R):
+        if r == 2:
+            continue
+        p = np.exp((l[r] - l[r].max()) / 0.8)
+        cdf = np.cumsum(p) / p.sum()
+        want = int(np.searchsorted(cdf, uu[r], side="left"))
+        got = int(out[r])
+        if got != want:
+            # a draw within rounding of a boundary may fall to the neighbour
+            assert abs(got - want) == 1 and abs(cdf[min(got, want)] - uu[r]) < 1e-5
+            bad += 1
+    assert bad <= 2
