@@ -1,0 +1,271 @@
+// Split-K grouped-query attention over the paged cache for single query rows (decode rows, and
+// the rows of short prompt portions): bf16 storage, float arithmetic, matrix cores.
+//
+// Work item = (query row, kv head, split).  A block of four waves handles the (up to 16) query
+// heads that share one kv head over the keys of its split, 32 keys per wave at a time:
+//
+//   S^T[key][head] = K[key][:] . Q[head][:]     v_mfma_f32_16x16x32_bf16, A = K rows read
+//                                               straight from the cache pages (head dims are
+//                                               contiguous), B = Q (kept in registers)
+//   per head (one lane column): running max and sum; scores and their exponentials never leave
+//   the lane that owns the column, so no broadcast is needed to rescale
+//   O^T[d][head]  += V^T[d][key] . P^T[key][head]   A = values, which the cache stores transposed
+//                                               inside a page (keys contiguous), B = P from the
+//                                               S^T accumulator without any data movement
+//
+// The four waves' states are merged through LDS; with more than one split the block writes a
+// partial (max, sum, O) and a second kernel merges the splits (same rule: exp(m_c - m_max)).
+// Which keys a row sees depends on its own position only: [max(0, p - window + 1), p].
+//
+// Reference: crates/kernels-hip/src/kernels/attention_decode_f16_paged.cu:49-158 (paged decode),
+// attention_decode_f16_splitk.cu:31-256 (partials and merge).
+#include "common.h"
+#include "api.h"
+
+#define DEC_WAVES 4
+#define DEC_CHUNK 32
+
+template <int HDP>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, PagedCache cache, const int* __restrict__ items,
+    const int* __restrict__ positions, const int* __restrict__ tok_seq,
+    const int* __restrict__ block_table, int max_blocks, int nh, float scale, int window,
+    int n_split, int q_tiles) {
+    constexpr int QS = HDP / 32;     // k-steps of the score product
+    constexpr int DT = HDP / 16;     // 16-wide tiles of head dims in the output
+    __shared__ float s_m[DEC_WAVES][16], s_l[DEC_WAVES][16];
+    __shared__ f32x4 s_o[DEC_WAVES - 1][DT][64];     // wave 0 keeps its own in registers
+
+    const int item = blockIdx.x;
+    const int kvh = blockIdx.y / q_tiles, qt = blockIdx.y % q_tiles;
+    const int split = blockIdx.z;
+    const int token = items[item];
+    const int hd = cache.head_dim, ps = cache.page_size;
+    const int G = nh / cache.n_kv_heads;
+    const int p = positions[token];
+    const int* table = block_table + (size_t)tok_seq[token] * max_blocks;
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int li = lane & 15, g = lane >> 4;
+    const bf16_t* kv = (const bf16_t*)cache.base;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // this split's chunks of 32 keys
+    const int c_lo = lo / DEC_CHUNK, c_hi = p / DEC_CHUNK;
+    const int per = (c_hi - c_lo + n_split) / n_split;
+    const int c0 = c_lo + split * per, c1 = min(c_hi + 1, c0 + per);
+
+    // Q as B operand: lane (head li, group g) holds Q[head][32 s + 8 g .. +7]
+    const int head = kvh * G + qt * 16 + li;
+    const bool head_ok = qt * 16 + li < G;
+    bf16x8 qreg[QS];
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+        const int d = 32 * s + 8 * g;
+        qreg[s] = (head_ok && d + 8 <= hd) ? *(const bf16x8*)(q + ((size_t)token * nh + head) * hd + d) : zero8;
+    }
+
+    f32x4 o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int c = c0 + wave; c < c1; c += DEC_WAVES) {
+        const int t0 = c * DEC_CHUNK;
+        // ---- scores of two 16-key tiles
+        f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+        {
+            const int ka = t0 + li, kb = t0 + 16 + li;
+            const int pa = (ka <= p && ka >= lo) ? table[ka / ps] : -1;
+            const int pb = (kb <= p && kb >= lo) ? table[kb / ps] : -1;
+            const bool oka = pa >= 0 && pa < cache.n_pages, okb = pb >= 0 && pb < cache.n_pages;
+            const bf16_t* rowa = kv + cache_k_offset(cache, oka ? pa : 0, kvh, ka % ps, 0);
+            const bf16_t* rowb = kv + cache_k_offset(cache, okb ? pb : 0, kvh, kb % ps, 0);
+            bf16x8 xa[QS], xb[QS];
+#pragma unroll
+            for (int s = 0; s < QS; ++s) {
+                const int d = 32 * s + 8 * g;
+                const bool din = d + 8 <= hd;
+                xa[s] = (oka && din) ? *(const bf16x8*)(rowa + d) : zero8;
+                xb[s] = (okb && din) ? *(const bf16x8*)(rowb + d) : zero8;
+            }
+#pragma unroll
+            for (int s = 0; s < QS; ++s) {
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[s], qreg[s], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[s], sb, 0, 0, 0);
+            }
+        }
+        // ---- values: lane (dim li of tile t, group g) reads keys 4g..4g+3 of either tile
+        const int va = t0 + 4 * g, vb = t0 + 16 + 4 * g;
+        const int pva = (va <= p) ? table[va / ps] : -1;
+        const int pvb = (vb <= p) ? table[vb / ps] : -1;
+        const bool okva = pva >= 0 && pva < cache.n_pages, okvb = pvb >= 0 && pvb < cache.n_pages;
+        bf16x4 wa[DT], wb[DT];
+        const bf16x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            const int d = 16 * t + li;
+            wa[t] = (okva && d < hd) ? *(const bf16x4*)(kv + cache_v_offset(cache, pva, kvh, va % ps, d)) : zero4;
+            wb[t] = (okvb && d < hd) ? *(const bf16x4*)(kv + cache_v_offset(cache, pvb, kvh, vb % ps, d)) : zero4;
+        }
+        // ---- online softmax; this lane holds keys 4g + r of both tiles for head li
+        float mt = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int ka = t0 + 4 * g + r, kb = ka + 16;
+            sa[r] = (ka >= lo && ka <= p) ? sa[r] * scale : -INFINITY;
+            sb[r] = (kb >= lo && kb <= p) ? sb[r] * scale : -INFINITY;
+            mt = fmaxf(mt, fmaxf(sa[r], sb[r]));
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m, mt);          // finite: every chunk holds a visible key
+        const float corr = expf(m - m_new);
+        bf16x8 pb8;
+        float ls = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float ea = expf(sa[r] - m_new), eb = expf(sb[r] - m_new);
+            ls += ea + eb;
+            pb8[r] = (bf16_t)ea;
+            pb8[4 + r] = (bf16_t)eb;
+        }
+        l = l * corr + ls;
+        m = m_new;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            bf16x8 v8;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { v8[r] = wa[t][r]; v8[4 + r] = wb[t][r]; }
+            o[t] *= corr;
+            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v8, pb8, o[t], 0, 0, 0);
+        }
+    }
+    // sum over the four key groups of a head
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+
+    // ---- merge the waves
+    if (g == 0) { s_m[wave][li] = m; s_l[wave][li] = l; }
+    if (wave > 0) {
+#pragma unroll
+        for (int t = 0; t < DT; ++t) s_o[wave - 1][t][lane] = o[t];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) mm = fmaxf(mm, s_m[w][li]);
+    float f[DEC_WAVES], ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+        f[w] = s_m[w][li] == -INFINITY ? 0.f : expf(s_m[w][li] - mm);
+        ll += s_l[w][li] * f[w];
+    }
+    if (!head_ok) return;
+    // lane (head li, group g) holds dims 16 t + 4 g + r
+    if (n_split == 1) {
+        const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+        bf16_t* orow = out + ((size_t)token * nh + head) * hd;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            f32x4 acc = o[t] * f[0];
+#pragma unroll
+            for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w - 1][t][lane] * f[w];
+            const int d = 16 * t + 4 * g;
+            if (d + 4 <= hd) {
+                bf16x4 ov = {(bf16_t)(acc[0] * inv), (bf16_t)(acc[1] * inv), (bf16_t)(acc[2] * inv), (bf16_t)(acc[3] * inv)};
+                *(bf16x4*)(orow + d) = ov;
+            }
+        }
+    } else {
+        const size_t slot = ((size_t)item * nh + head) * n_split + split;
+        if (g == 0) { part_ml[slot * 2] = mm; part_ml[slot * 2 + 1] = ll; }
+        float* prow = part_o + slot * HDP;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            f32x4 acc = o[t] * f[0];
+#pragma unroll
+            for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w - 1][t][lane] * f[w];
+            *(f32x4*)(prow + 16 * t + 4 * g) = acc;
+        }
+    }
+}
+
+// Merge of the splits: one block per (item, head), one thread per head dim.
+__global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                bf16_t* __restrict__ out,
+                                                                const int* __restrict__ items, int nh,
+                                                                int hd, int hdp, int n_split) {
+    const int item = blockIdx.x, head = blockIdx.y;
+    const int token = items[item];
+    const size_t base = ((size_t)item * nh + head) * n_split;
+    float mm = -INFINITY;
+    for (int s = 0; s < n_split; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+    float ll = 0.f;
+    for (int s = 0; s < n_split; ++s) {
+        const float ms = part_ml[(base + s) * 2];
+        ll += ms == -INFINITY ? 0.f : part_ml[(base + s) * 2 + 1] * expf(ms - mm);
+    }
+    const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < n_split; ++s) {
+            const float ms = part_ml[(base + s) * 2];
+            if (ms != -INFINITY) acc += part_o[(base + s) * hdp + d] * expf(ms - mm);
+        }
+        out[((size_t)token * nh + head) * hd + d] = (bf16_t)(acc * inv);
+    }
+}
+
+extern "C" int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats,
+                                        long* ml_floats) {
+    const int hdp = ceil_div(hd, 32) * 32;
+    *o_floats = (long)n_items * nh * n_split * hdp;
+    *ml_floats = (long)n_items * nh * n_split * 2;
+    return 0;
+}
+
+extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml,
+                              const void* cache_base, const int* items, int n_items,
+                              const int* positions, const int* tok_seq, const int* block_table,
+                              int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
+                              float scale, int window, int n_split, hipStream_t stream) {
+    FL_CHECK(n_items >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_decode: bad head counts %d/%d", nh, nkv);
+    FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "attn_decode: head size %d must be a multiple of 8 up to 256", hd);
+    FL_CHECK(page_size % 4 == 0, "attn_decode: page size %d must be a multiple of 4", page_size);
+    FL_CHECK(n_split >= 1 && n_split <= 256, "attn_decode: %d splits", n_split);
+    FL_CHECK(n_split == 1 || (part_o && part_ml), "attn_decode: splits need a workspace");
+    FL_CHECK(window >= 0, "attn_decode: negative window");
+    if (n_items == 0) return 0;
+    PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
+    const int G = nh / nkv;
+    const int q_tiles = ceil_div(G, 16);
+    dim3 grid(n_items, nkv * q_tiles, n_split);
+    const int hdp = ceil_div(hd, 32) * 32;
+#define FL_DEC(HDP_)                                                                                  \
+    attn_decode_kernel<HDP_><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, part_ml, c, items, \
+                                                       positions, tok_seq, block_table, max_blocks, nh, scale,   \
+                                                       window, n_split, q_tiles)
+    switch (hdp) {
+        case 32: FL_DEC(32); break;
+        case 64: FL_DEC(64); break;
+        case 96: FL_DEC(96); break;
+        case 128: FL_DEC(128); break;
+        case 160: FL_DEC(160); break;
+        case 192: FL_DEC(192); break;
+        case 224: FL_DEC(224); break;
+        default: FL_DEC(256); break;
+    }
+#undef FL_DEC
+    FL_LAUNCH_CHECK();
+    if (n_split > 1) {
+        dim3 mg(n_items, nh);
+        attn_decode_merge_kernel<<<mg, hd <= 64 ? 64 : (hd <= 128 ? 128 : 256), 0, stream>>>(
+            part_o, part_ml, (bf16_t*)out, items, nh, hd, hdp, n_split);
+        FL_LAUNCH_CHECK();
+    }
+    return 0;
+}

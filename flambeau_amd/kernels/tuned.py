@@ -8,11 +8,12 @@ from __future__ import annotations
 import torch
 
 from . import ops
-from .library import P, I, F, call, register_signatures
+from .library import F, I, KernelError, P, call, register_signatures
 from .ops import _check, dtype_code, stream_handle
 
 register_signatures({
     "fl_gemm_skinny": [P, P, P, I, I, I, I, P],
+    "fl_attn_decode": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
 })
 
 SKINNY_MAX_ROWS = 64
@@ -34,9 +35,76 @@ def gemm(x, w, out):
     return ops.gemm_plain(x, w, out)
 
 
+# Rows of portions up to this length are treated as single query rows by the split-K kernel;
+# longer portions go to the tiled prefill kernel.
+SHORT_PORTION = 8
+DECODE_TARGET_BLOCKS = 1024
+DECODE_MIN_KEYS_PER_SPLIT = 128
+
+
 def attention_metadata(batch) -> dict:
-    return {}
+    """Work lists for the attention kernels of one batch: ``attn_rows`` = the rows that run as
+    single queries (decode rows and rows of short portions)."""
+    import numpy as np
+    rows = []
+    for q0, ql in zip(batch.q_starts, batch.q_lens):
+        if ql <= SHORT_PORTION:
+            rows += range(q0, q0 + ql)
+    return {"attn_rows": np.asarray(rows, dtype=np.int32)}
 
 
-def attention(q, out, cache, step, table, n_heads, scale, window):
+def decode_splits(n_items: int, n_kv_heads: int, group: int, max_ctx: int) -> int:
+    """How many splits of the keys give the chip enough blocks without making a split shorter
+    than a few chunks.  Depends on the batch's shape only (fixed for a captured graph)."""
+    base = max(1, n_items * n_kv_heads * -(-group // 16))
+    by_blocks = max(1, DECODE_TARGET_BLOCKS // base)
+    by_keys = max(1, -(-max_ctx // DECODE_MIN_KEYS_PER_SPLIT))
+    return int(min(by_blocks, by_keys, 64))
+
+
+def attn_decode(q, out, cache, rows, positions, tok_seq, table, n_heads, scale, window, n_split, part_o=None,
+                part_ml=None):
+    n = q.shape[0]
+    hd = cache.head_dim
+    n_items = rows.shape[0]
+    if n_split > 1:
+        hdp = -(-hd // 32) * 32
+        need_o, need_ml = n_items * n_heads * n_split * hdp, n_items * n_heads * n_split * 2
+        if part_o is None or part_o.numel() < need_o or part_ml is None or part_ml.numel() < need_ml:
+            raise KernelError("attn_decode: workspace too small for the splits")
+    call("fl_attn_decode", _check(q, "attn.q", torch.bfloat16, (n, n_heads * hd)),
+         _check(out, "attn.out", torch.bfloat16, (n, n_heads * hd)),
+         _check(part_o, "attn.part_o", torch.float32) if part_o is not None else None,
+         _check(part_ml, "attn.part_ml", torch.float32) if part_ml is not None else None,
+         _check(cache.pool, "attn.cache", torch.bfloat16), _check(rows, "attn.rows", torch.int32, (n_items,)), n_items,
+         _check(positions, "attn.positions", torch.int32, (n,)), _check(tok_seq, "attn.tok_seq", torch.int32, (n,)),
+         _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads,
+         hd, cache.page_size, cache.n_pages, float(scale), int(window), int(n_split), stream_handle())
+    return out
+
+
+def decode_supported(cache) -> bool:
+    return cache.pool.dtype == torch.bfloat16 and cache.head_dim % 8 == 0 and cache.head_dim <= 256 \
+        and cache.page_size % 4 == 0
+
+
+def attention(rt, q, out, cache, step, table, n_heads, scale, window):
+    """Attention of one batch with the tuned kernels: rows of short portions through the
+    split-K kernel; a batch with longer portions falls to the plain kernel as a whole."""
+    rows = step.extra.get("attn_rows")
+    batch = step.host
+    if rows is not None and rows.shape[0] == step.n_tokens and decode_supported(cache):
+        group = n_heads // cache.n_kv_heads
+        max_ctx = batch.ctx_bound or batch.max_ctx_len
+        if window:
+            max_ctx = min(max_ctx, window + 32)
+        n_split = decode_splits(rows.shape[0], cache.n_kv_heads, group, max_ctx)
+        part_o = part_ml = None
+        if n_split > 1:
+            hdp = -(-cache.head_dim // 32) * 32
+            slots = rows.shape[0] * n_heads * n_split
+            part_o = rt.buffer("attn_part_o", slots, hdp, torch.float32, max_rows=max(slots, 4096 * n_heads))
+            part_ml = rt.buffer("attn_part_ml", slots, 2, torch.float32, max_rows=max(slots, 4096 * n_heads))
+        return attn_decode(q, out, cache, rows, step.positions, step.tok_seq, table, n_heads, scale, window,
+                           n_split, part_o, part_ml)
     return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)

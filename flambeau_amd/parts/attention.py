@@ -69,7 +69,7 @@ class PagedGQAAttention(Mixer):
         out = rt.buffer("attn_out", n, nh * hd)
         if rt.tuned:
             from ..kernels import tuned
-            tuned.attention(q, out, cache.kv, step, table, nh, self.scale, self.window)
+            tuned.attention(rt, q, out, cache.kv, step, table, nh, self.scale, self.window)
         else:
             ops.attn_plain(q, out, cache.kv, step.positions, step.tok_seq, table, nh, self.scale, self.window)
         delta = rt.buffer("delta", n, self.hidden_size, torch.float32)

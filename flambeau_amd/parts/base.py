@@ -91,7 +91,7 @@ class HostBatch:
     slots: list
     n_tokens: int
     n_logit_rows: int
-    fixed_shape: bool = False      # padded to a fixed size for graph replay
+    ctx_bound: int | None = None   # set for a fixed-shape batch (graph replay): longest context it may ever hold
 
     @property
     def n_seqs(self): return len(self.q_lens)

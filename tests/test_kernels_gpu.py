@@ -323,3 +323,42 @@ def test_sample_is_the_inverse_cdf_in_index_order(V):
             assert abs(got - want) == 1 and abs(cdf[min(got, want)] - uu[r]) < 1e-5
             bad += 1
     assert bad <= 2
+
+
+# ---------------------------------------------------------------- tuned attention for single rows
+@pytest.mark.parametrize("n_split", [1, 2, 5])
+@pytest.mark.parametrize("nh,nkv,hd,ps,window", [(32, 8, 128, 16, 0), (4, 2, 16, 8, 16), (6, 1, 24, 16, 0),
+                                                (5, 5, 32, 16, 24), (20, 1, 64, 4, 0), (8, 4, 256, 32, 100),
+                                                (3, 1, 40, 64, 0)])
+def test_attn_decode_against_plain_and_reference(nh, nkv, hd, ps, window, n_split):
+    seqs = [(700, 1), (33, 1), (ps * 3, 1), (1, 1), (257, 3), (64, 2), (32, 1), (31, 1)]
+    case = build_attention_case(torch.bfloat16, nh, nkv, hd, ps, seqs, seed=3)
+    n = case["n"]
+    scale = 1 / math.sqrt(hd)
+    q2 = case["q"].reshape(n, nh * hd)
+    rows = torch.arange(n, dtype=torch.int32, device=DEV).flip(0).contiguous()      # any order of rows
+    out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hdp = -(-hd // 32) * 32
+    part_o = torch.empty(n * nh * n_split * hdp, dtype=torch.float32, device=DEV)
+    part_ml = torch.empty(n * nh * n_split * 2, dtype=torch.float32, device=DEV)
+    tuned().attn_decode(q2, out, case["cache"], rows, case["pos_d"], case["seq_d"], case["table"], nh, scale,
+                        window, n_split, part_o, part_ml)
+    plain = torch.empty_like(out)
+    ops().attn_plain(q2, plain, case["cache"], case["pos_d"], case["seq_d"], case["table"], nh, scale, window)
+    ref = attention_case_ref(case, scale, window)
+    top = ref.abs().max()
+    assert (out.double().reshape(n, nh, hd) - ref).abs().max() < 1e-2 * top
+    assert (out.double() - plain.double()).abs().max() < 1.5e-2 * top
+
+
+def test_attn_decode_subset_of_rows_leaves_the_others_alone():
+    nh, nkv, hd, ps = 8, 2, 64, 16
+    case = build_attention_case(torch.bfloat16, nh, nkv, hd, ps, [(40, 4), (90, 1)], seed=4)
+    n = case["n"]
+    q2 = case["q"].reshape(n, nh * hd)
+    out = torch.full((n, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    tuned().attn_decode(q2, out, case["cache"], rows, case["pos_d"], case["seq_d"], case["table"], nh, 0.125, 0, 1)
+    ref = attention_case_ref(case, 0.125, 0)
+    assert (out[[0, 2, 3]] == 7.0).all()
+    assert (out[[1, 4]].double().reshape(2, nh, hd) - ref[[1, 4]]).abs().max() < 1e-2 * ref.abs().max()
