@@ -46,7 +46,8 @@ class LLMEngine:
         ctx = min(opt.ctx_cap or spec.max_position, spec.max_position)
         n_pages = opt.paged_kv or opt.inflight_slots * -(-ctx // opt.page_size)
         self.runner = ModelRunner(model, n_pages=n_pages, page_size=opt.page_size, max_slots=opt.inflight_slots,
-                                  max_seq_len=ctx, max_logit_rows=max(opt.inflight_slots, 1))
+                                  max_seq_len=ctx, max_logit_rows=max(opt.inflight_slots, 1),
+                                  decode_graphs=opt.decode_graphs)
         self.scheduler = Scheduler(self.runner.manager, max_batch_tokens=model.rt.max_batch_tokens,
                                    prefill_chunk_tokens=opt.prefill_chunk_tokens,
                                    max_queue_depth=opt.max_queue_depth, eos_token_id=spec.eos_token_id,

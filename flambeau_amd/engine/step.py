@@ -39,7 +39,7 @@ class ModelRunner:
     """Owns the model, the cache and the step function."""
 
     def __init__(self, model, *, n_pages: int, page_size: int, max_slots: int, max_seq_len: int | None = None,
-                 max_logit_rows: int | None = None):
+                 max_logit_rows: int | None = None, decode_graphs: bool = True, max_graph_batch: int = 256):
         self.model = model
         self.rt = model.rt
         spec = model.spec
@@ -53,6 +53,11 @@ class ModelRunner:
         self._meta_host = None
         self._meta_dev = None
         self._meta_copied = None     # event: the last metadata copy has left the pinned buffer
+        # steps of single tokens replay a captured graph per batch-size bucket, if every mixer
+        # of the model says that running a step twice leaves the same cache (graph_safe)
+        self.decode_graphs = bool(decode_graphs) and all(getattr(c, "graph_safe", False) for c in self._mixer_classes)
+        self.max_graph_batch = min(max_graph_batch, max_slots)
+        self._graphs: dict[int, "_GraphedStep"] = {}
 
     # ------------------------------------------------------------ requests
     def begin(self, request_id) -> bool:
@@ -74,10 +79,8 @@ class ModelRunner:
             self._meta_capacity = cap
         return self._meta_host, self._meta_dev
 
-    def build_step(self, entries, table_width: int | None = None) -> StepState:
-        """Validate the entries, reserve their pages and put the batch's metadata on the device."""
+    def _validate(self, entries):
         mgr = self.manager
-        V = self.model.spec.vocab_size
         seen = set()
         n = 0
         for e in entries:
@@ -97,13 +100,26 @@ class ModelRunner:
         n_rows = sum(len(e.want) for e in entries)
         if n_rows > self.max_logit_rows:
             raise StepError(f"logits wanted at {n_rows} places, at most {self.max_logit_rows} per step")
+        V = self.model.spec.vocab_size
+        for e in entries:
+            if min(e.tokens) < 0 or max(e.tokens) >= V:
+                bad = next(t for t in e.tokens if not 0 <= t < V)
+                raise StepError(f"token id {bad} is outside the vocabulary of {V}")
         if not mgr.can_cover((e.request_id, mgr.live[e.request_id].n_cached + len(e.tokens)) for e in entries):
             raise CacheError("not enough free pages (or a request beyond the maximum length) for this step")
+        return n
 
-        tokens = np.empty(n, dtype=np.int32)
-        positions = np.empty(n, dtype=np.int32)
-        tok_seq = np.empty(n, dtype=np.int32)
+    def _assemble(self, entries, pad_to: int | None = None):
+        """Reserve the entries' pages and lay out the batch's metadata as integer arrays.
+        ``pad_to``: fixed number of single-token requests (graph replay); the padding rows have
+        no pages, write nothing and are never read."""
+        mgr = self.manager
+        n = sum(len(e.tokens) for e in entries)
         S = len(entries)
+        n_pad = (pad_to - S) if pad_to is not None else 0
+        tokens = np.zeros(n + n_pad, dtype=np.int32)
+        positions = np.zeros(n + n_pad, dtype=np.int32)
+        tok_seq = np.empty(n + n_pad, dtype=np.int32)
         q_starts, q_lens, starts, slots, rows = [], [], [], [], []
         at = 0
         for s, e in enumerate(entries):
@@ -119,21 +135,29 @@ class ModelRunner:
             slots.append(rc.slot)
             rows += [at + w for w in e.want]
             at += k
-        if n and (tokens.min() < 0 or tokens.max() >= V):
-            bad = int(tokens[(tokens < 0) | (tokens >= V)][0])
-            raise StepError(f"token id {bad} is outside the vocabulary of {V}")
-        batch = HostBatch(q_starts, q_lens, starts, slots, n, len(rows))
-
-        need_blocks = max((-(-(st + q) // mgr.page_size) for st, q in zip(starts, q_lens)), default=1)
-        width = table_width or max(8, -(-need_blocks // 8) * 8)
+        for s in range(S, S + n_pad):
+            tok_seq[at] = s
+            q_starts.append(at)
+            q_lens.append(1)
+            starts.append(0)
+            slots.append(0)
+            at += 1
+        if pad_to is not None:
+            rows = list(range(pad_to))          # a fixed-shape step computes every row's logits
+        batch = HostBatch(q_starts, q_lens, starts, slots, n + n_pad, len(rows),
+                          ctx_bound=self.max_seq_len if pad_to is not None else None)
+        if pad_to is not None:
+            width = mgr.max_blocks
+        else:
+            need_blocks = max((-(-(st + q) // mgr.page_size) for st, q in zip(starts, q_lens)), default=1)
+            width = max(8, -(-need_blocks // 8) * 8)
         tables = []
         for g in range(len(mgr.groups)):
-            t = np.full((S, width), -1, dtype=np.int32)
+            t = np.full((S + n_pad, width), -1, dtype=np.int32)
             for s, e in enumerate(entries):
                 row = mgr.table_row(e.request_id, g)
                 t[s, :len(row)] = row
             tables.append(t)
-
         parts = [("tokens", tokens), ("positions", positions), ("tok_seq", tok_seq),
                  ("seq_slots", np.asarray(slots, dtype=np.int32)),
                  ("seq_q_start", np.asarray(q_starts, dtype=np.int32)),
@@ -141,27 +165,46 @@ class ModelRunner:
                  ("seq_ctx_len", np.asarray([st + q for st, q in zip(starts, q_lens)], dtype=np.int32)),
                  ("logit_rows", np.asarray(rows, dtype=np.int32))]
         parts += [(f"table{g}", t) for g, t in enumerate(tables)]
-        extra_names = []
         for cls in self._mixer_classes:
             for name, arr in cls.step_metadata(batch).items():
                 parts.append(("extra:" + name, np.ascontiguousarray(arr, dtype=np.int32)))
-                extra_names.append(name)
-        dev = self._upload(parts)
-        return StepState(
-            n_tokens=n, n_seqs=S, tokens=dev["tokens"], positions=dev["positions"], tok_seq=dev["tok_seq"],
-            seq_slots=dev["seq_slots"], seq_q_start=dev["seq_q_start"], seq_q_len=dev["seq_q_len"],
-            seq_ctx_len=dev["seq_ctx_len"], block_tables=[dev[f"table{g}"] for g in range(len(tables))],
-            logit_rows=dev["logit_rows"], host=batch, extra={k: dev["extra:" + k] for k in extra_names})
+        return batch, parts
 
-    def _upload(self, parts) -> dict:
-        """One host-to-device copy for all integer arrays; returns device views by name."""
+    def _state_from(self, batch, parts, dev) -> StepState:
+        extra = {name[6:]: dev[name] for name, _ in parts if name.startswith("extra:")}
+        n_groups = len(self.manager.groups)
+        return StepState(
+            n_tokens=batch.n_tokens, n_seqs=batch.n_seqs, tokens=dev["tokens"], positions=dev["positions"],
+            tok_seq=dev["tok_seq"], seq_slots=dev["seq_slots"], seq_q_start=dev["seq_q_start"],
+            seq_q_len=dev["seq_q_len"], seq_ctx_len=dev["seq_ctx_len"],
+            block_tables=[dev[f"table{g}"] for g in range(n_groups)], logit_rows=dev["logit_rows"],
+            host=batch, extra=extra)
+
+    def build_step(self, entries) -> StepState:
+        """Validate the entries, reserve their pages and put the batch's metadata on the device."""
+        self._validate(entries)
+        batch, parts = self._assemble(entries)
+        return self._state_from(batch, parts, self._upload(parts))
+
+    @staticmethod
+    def _layout(parts):
         offsets, total = [], 0
         for _, arr in parts:
             offsets.append(total)
             total += -(-arr.size // 4) * 4 if arr.size else 0   # 16-byte alignment of every array
+        return offsets, total
+
+    def _upload(self, parts, dev=None) -> dict:
+        """One host-to-device copy for all integer arrays; returns device views by name.
+        ``dev``: a fixed device buffer (a captured graph's own) instead of the shared one."""
+        offsets, total = self._layout(parts)
         if self._meta_copied is not None:
             self._meta_copied.synchronize()
-        host, dev = self._meta_buffers(max(total, 1))
+        host, shared = self._meta_buffers(max(total, 1))
+        if dev is None:
+            dev = shared
+        elif dev.numel() < total:
+            raise StepError("metadata of a fixed-shape step outgrew its buffer")
         hnp = host.numpy()
         for (name, arr), off in zip(parts, offsets):
             if arr.size:
@@ -184,9 +227,59 @@ class ModelRunner:
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if not entries:
             return None
-        step = self.build_step(entries)
-        self.storage.zero_slots(self.manager.take_fresh_slots())
-        logits = self.model.forward(step, self.storage.entries, self.max_logit_rows)
+        self._validate(entries)
+        fresh = self.manager.take_fresh_slots()
+        self.storage.zero_slots(fresh)
+        if self.decode_graphs and self._bucket(len(entries)) <= min(self.max_graph_batch, self.rt.max_batch_tokens) \
+                and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries):
+            logits = self._step_graphed(entries)
+        else:
+            batch, parts = self._assemble(entries)
+            step = self._state_from(batch, parts, self._upload(parts))
+            logits = self.model.forward(step, self.storage.entries, self.max_logit_rows)
         for e in entries:
             self.manager.advance(e.request_id, len(e.tokens))
         return logits
+
+    # ------------------------------------------------------------ captured decode steps
+    def _bucket(self, n: int) -> int:
+        b = 1
+        while b < n:
+            b *= 2
+        return b if b <= self.max_graph_batch else max(n, self.max_graph_batch)
+
+    def _step_graphed(self, entries):
+        """A step of single tokens: pad to the bucket's size, copy the metadata into the graph's
+        own buffer, replay.  The first step of a bucket runs eagerly once (buffers are made),
+        is captured, and replayed; a step leaves the same cache however often it runs."""
+        bk = self._bucket(len(entries))
+        batch, parts = self._assemble(entries, pad_to=bk)
+        gs = self._graphs.get(bk)
+        if gs is None:
+            _, total = self._layout(parts)
+            gs = _GraphedStep(torch.empty(max(total, 1), dtype=torch.int32, device=self.rt.device))
+            self._graphs[bk] = gs
+        dev = self._upload(parts, gs.meta)
+        if gs.graph is None:
+            step = self._state_from(batch, parts, dev)
+            with self.rt.scope(f"graph{bk}"):
+                self.model.forward(step, self.storage.entries, bk)          # makes the buffers
+                torch.cuda.current_stream().synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    gs.logits = self.model.forward(step, self.storage.entries, bk)
+            gs.graph = graph
+        gs.graph.replay()
+        wanted = [i for i, e in enumerate(entries) if e.want]
+        if not wanted:
+            return None
+        if wanted == list(range(len(wanted))):
+            return gs.logits[:len(wanted)]
+        return gs.logits[torch.tensor(wanted, device=self.rt.device)]
+
+
+class _GraphedStep:
+    def __init__(self, meta):
+        self.meta = meta
+        self.graph = None
+        self.logits = None

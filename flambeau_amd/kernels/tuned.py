@@ -103,8 +103,9 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
         if n_split > 1:
             hdp = -(-cache.head_dim // 32) * 32
             slots = rows.shape[0] * n_heads * n_split
-            part_o = rt.buffer("attn_part_o", slots, hdp, torch.float32, max_rows=max(slots, 4096 * n_heads))
-            part_ml = rt.buffer("attn_part_ml", slots, 2, torch.float32, max_rows=max(slots, 4096 * n_heads))
+            cap = slots if batch.ctx_bound else max(slots, 4096 * n_heads)     # a fixed-shape step never grows
+            part_o = rt.buffer("attn_part_o", slots, hdp, torch.float32, max_rows=cap)
+            part_ml = rt.buffer("attn_part_ml", slots, 2, torch.float32, max_rows=cap)
         return attn_decode(q, out, cache, rows, step.positions, step.tok_seq, table, n_heads, scale, window,
                            n_split, part_o, part_ml)
     return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)

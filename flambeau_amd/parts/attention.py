@@ -22,6 +22,8 @@ from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, Tens
 
 @MIXERS.register("paged_gqa_attention")
 class PagedGQAAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, window: int = 0, scale: float | None = None):
         if n_heads % n_kv_heads:

@@ -136,6 +136,11 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True if running the same step twice leaves the cache as running it once does (keys and
+    # values are written by position).  A mixer that advances a state of its own is not, and a
+    # model with such a mixer never replays captured steps.
+    graph_safe = False
+
     def cache_spec(self):
         """``PagedKVSpec``, ``StateSpec`` or ``None``."""
         return None

@@ -213,3 +213,39 @@ def test_generation_survives_preemption(model_dirs):
     got = tight.generate(prompts, SamplingParams(max_tokens=30))
     assert tight.scheduler.n_preemptions > 0
     assert got == want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_equal_eager_ones(model_dirs, dtype):
+    """Steps of single tokens replay a captured graph per batch-size bucket.  Every replay, with
+    eager steps and synchronisations between them, gives the logits of the eager step."""
+    name = "A"
+    d = model_dirs[(name, STORE[dtype])]
+    reqs = rh.make_requests(256, [30, 45, 37], seed=17)
+    from flambeau_amd.engine import ModelRunner, load_model
+    model, _ = load_model(d, dtype=dtype, max_batch_tokens=256)
+    results = []
+    for graphs in (False, True):
+        runner = ModelRunner(model, n_pages=32, page_size=8, max_slots=4, max_logit_rows=256, decode_graphs=graphs)
+        assert runner.decode_graphs == graphs
+        steps = []
+        # prompts in portions, then decode rows of 3, 2 and 1 requests (buckets 4, 2, 1), with a
+        # portion of another request between replays
+        steps.append(dict(entries=[dict(id=r, tokens=reqs[r][:20], want=[19]) for r in reqs], end=[]))
+        for i in range(20, 30):
+            steps.append(dict(entries=[dict(id=r, tokens=[reqs[r][i]], want=[0]) for r in reqs], end=["r0"] if i == 29 else []))
+        steps.append(dict(entries=[dict(id="r1", tokens=reqs["r1"][30:34], want=[0, 3])], end=[]))
+        for i in range(30, 37):
+            e = [dict(id="r2", tokens=[reqs["r2"][i]], want=[0])]
+            if i + 4 < 45:
+                e.append(dict(id="r1", tokens=[reqs["r1"][i + 4]], want=[] if i % 2 else [0]))
+            steps.append(dict(entries=e, end=[]))
+        steps.append(dict(entries=[dict(id="r1", tokens=[reqs["r1"][41]], want=[0])], end=["r1", "r2"]))
+        results.append(rh.run_in_process(runner, steps))
+        if graphs:
+            assert sorted(runner._graphs) == [1, 2, 4]
+    eager, graphed = results
+    assert eager.keys() == graphed.keys() and len(eager) > 30
+    for k in eager:
+        assert np.array_equal(eager[k], graphed[k]), k
+    rh.compare(graphed, reqs, rh.plain_logits(d, reqs), dtype, "captured steps")
