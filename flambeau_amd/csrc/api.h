@@ -36,8 +36,9 @@ int fl_sample(const float* logits, const float* inv_temp, const float* uniform, 
               int rows, int V, hipStream_t stream);
 
 // ---- tuned bf16 kernels ----
+// nw_hint: waves per block that split K (0: chosen from the sizes)
 int fl_gemm_skinny(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K,
-                   hipStream_t stream);
+                   int nw_hint, hipStream_t stream);
 
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                    const int* items, int n_items, const int* positions, const int* tok_seq,

@@ -2,13 +2,16 @@
 // (up to 64) and a large weight matrix that is read exactly once.  The product is bound by the
 // stream of w out of HBM, so the kernel is built around that stream:
 //
-//  * a block owns 16 consecutive output features (rows of w); its NW waves split K between
+//  * w is stored packed (see pack_weight in kernels/packing.py): the 16 rows x 32 k that one
+//    matrix-core instruction takes as its A operand are 1 KB of contiguous memory in lane
+//    order, tiles of one row group following each other along k.  A wave's load instruction
+//    then reads one whole kilobyte, and its 8 loads per iteration 8 KB in a row (measured:
+//    6.2 TB/s against 5.3 TB/s for 16 row pieces of 64 B per instruction);
+//  * a block owns 16 consecutive output features (a row group); its NW waves split K between
 //    them and add their partial sums through LDS in a fixed order (no atomics: the result
 //    does not depend on timing);
-//  * a wave keeps 8 (or 16) 16-byte loads of w in flight per lane before it consumes them;
-//    within an iteration over 256 values of k, lane (i, g) reads the 128 contiguous bytes
-//    w[row i][k0 + 64 g .. k0 + 64 g + 63]; w is loaded with the non-temporal hint so that it
-//    does not push x out of the caches;
+//  * a wave keeps 8 16-byte loads of w in flight per lane before it consumes them; w is loaded
+//    with the non-temporal hint so that it does not push x out of the caches;
 //  * the arithmetic is v_mfma_f32_16x16x32_bf16 with w as the A operand (16 features x 32 k)
 //    and x as the B operand (32 k x 16 tokens): C[feature][token] leaves each lane with four
 //    consecutive features of one token, i.e. one 16-byte store.  Rows of x beyond M are not
@@ -27,19 +30,18 @@ __device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
 
 template <int MT, typename TOut>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
-                                                           const bf16_t* __restrict__ w,
+                                                           const bf16_t* __restrict__ wp,
                                                            TOut* __restrict__ out, int M, int N, int K,
-                                                           int vec_out) {
+                                                           int n_steps, int vec_out) {
     extern __shared__ float red[];               // [NW][MT][64][4]
     const int nw = blockDim.x >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int li = lane & 15, g = lane >> 4;
-    const int row = min(blockIdx.x * 16 + li, N - 1);
-    const bf16_t* wrow = w + (size_t)row * K;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    // tiles of this row group: [n_steps][64 lanes][8 values]
+    const bf16_t* wt = wp + ((size_t)blockIdx.x * n_steps * 64 + lane) * 8;
 
     // K in steps of 32; this wave's steps [s0, s1)
-    const int n_steps = (K + 31) >> 5;
     const int per = (n_steps + nw - 1) / nw;
     const int s0 = wave * per, s1 = min(n_steps, s0 + per);
 
@@ -49,39 +51,34 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     for (int mt = 0; mt < MT; ++mt) {
         const int tok = mt * 16 + li;
         xok[mt] = tok < M;
-        xrow[mt] = x + (size_t)min(tok, M - 1) * K;
+        xrow[mt] = x + (size_t)min(tok, M - 1) * K + 8 * g;
     }
     f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     int s = s0;
-    // full iterations: 8 steps = 256 values of k, all inside K
-    for (; s + 8 <= s1 && (s + 8) * 32 <= K; s += 8) {
-        const int kb = s * 32 + 64 * g;
-        bf16x8 a[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) a[j] = __builtin_nontemporal_load((const bf16x8*)(wrow + kb + 8 * j));
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            bf16x8 b[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) b[j] = xok[mt] ? *(const bf16x8*)(xrow[mt] + kb + 8 * j) : zero;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);
-        }
+    // iterations of U steps: every load of the iteration is issued before the first product needs
+    // its data.  x beyond K does not exist (w is zero there): such chunks count as zero.
+#define FL_SKINNY_ITER(U)                                                                              \
+    for (; s + U <= s1; s += U) {                                                                      \
+        bf16x8 a[U];                                                                                   \
+        _Pragma("unroll") for (int j = 0; j < U; ++j)                                                  \
+            a[j] = __builtin_nontemporal_load((const bf16x8*)(wt + (size_t)(s + j) * 512));            \
+        _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                            \
+            bf16x8 b[U];                                                                               \
+            _Pragma("unroll") for (int j = 0; j < U; ++j)                                              \
+                b[j] = (xok[mt] && (s + j) * 32 + 8 * g + 8 <= K)                                      \
+                           ? *(const bf16x8*)(xrow[mt] + (s + j) * 32) : zero;                         \
+            _Pragma("unroll") for (int j = 0; j < U; ++j)                                              \
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);       \
+        }                                                                                              \
     }
-    // remaining steps one by one; a chunk of 8 values that reaches beyond K counts as zero
-    for (; s < s1; ++s) {
-        const int k = s * 32 + 8 * g;
-        const bool in = k + 8 <= K;
-        const bf16x8 a = in ? __builtin_nontemporal_load((const bf16x8*)(wrow + k)) : zero;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const bf16x8 b = (in && xok[mt]) ? *(const bf16x8*)(xrow[mt] + k) : zero;
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
-        }
-    }
+    FL_SKINNY_ITER(8)
+    FL_SKINNY_ITER(4)
+    FL_SKINNY_ITER(2)
+    FL_SKINNY_ITER(1)
+#undef FL_SKINNY_ITER
 
     // add the waves' partial sums in wave order
 #pragma unroll
@@ -111,30 +108,34 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 }
 
 template <int MT, typename TOut>
-static int launch_skinny(const bf16_t* x, const bf16_t* w, TOut* out, int M, int N, int K, hipStream_t stream) {
+static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
+                         hipStream_t stream) {
     const int groups = ceil_div(N, 16);
+    const int n_steps = ceil_div(K, 32);
     // enough waves in flight to cover the memory latency: about 2048 and more over the chip
     int nw = 4;
     while (nw < 16 && groups * nw < 2048) nw *= 2;
-    while (nw > 1 && ceil_div(K, 32) < nw * 2) nw /= 2;
+    if (nw_hint > 0) nw = nw_hint;
+    while (nw > 1 && n_steps < nw * 2) nw /= 2;
     const size_t lds = (size_t)nw * MT * 64 * 4 * sizeof(float);
     const int vec_out = (N % 4 == 0) ? 1 : 0;      // 16-byte stores need aligned rows
-    gemm_skinny_kernel<MT, TOut><<<groups, nw * 64, lds, stream>>>(x, w, out, M, N, K, vec_out);
+    gemm_skinny_kernel<MT, TOut><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, vec_out);
     return 0;
 }
 
-extern "C" int fl_gemm_skinny(const void* x, const void* w, void* out, int out_dtype, int M, int N,
-                              int K, hipStream_t stream) {
+extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N,
+                              int K, int nw_hint, hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
+    FL_CHECK(nw_hint >= 0 && nw_hint <= 16, "gemm_skinny: %d waves per block, at most 16", nw_hint);
     FL_CHECK(K % 8 == 0, "gemm_skinny: K=%d is no multiple of 8 (16-byte loads)", K);
-    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0),
+    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
              "gemm_skinny: operands must be 16-byte aligned");
     if (M == 0) return 0;
     const int mt = ceil_div(M, 16);
 #define FL_SK(MT_)                                                                                         \
-    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w, (float*)out, M, N, K, stream); \
-    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)out, M, N, K, stream)
+    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N, K, nw_hint, stream); \
+    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M, N, K, nw_hint, stream)
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
     switch (mt) {
         case 1: FL_SK(1); break;

@@ -73,9 +73,18 @@ class Runtime:
         return t.to(device=self.device, dtype=want).contiguous()
 
     # ------------------------------------------------------------ matrix products
+    def prepare_weight(self, w: torch.Tensor):
+        """A loaded matrix ``[out_features, in_features]`` in the form(s) the kernels of this
+        runtime read: row-major for the plain kernels, packed tiles for the tuned ones."""
+        if self.tuned:
+            from ..kernels import tuned
+            return tuned.prepare_weight(w)
+        from ..kernels.packing import Weight
+        return Weight(w.shape[0], w.shape[1], rowmajor=w)
+
     def gemm(self, x, w, out):
-        """``out = x @ w.T``; ``w`` is ``[out_features, in_features]``."""
+        """``out = x @ w.T``; ``w`` comes from ``prepare_weight``."""
         if self.tuned:
             from ..kernels import tuned
             return tuned.gemm(x, w, out)
-        return ops.gemm_plain(x, w, out)
+        return ops.gemm_plain(x, w.rowmajor, out)

@@ -10,29 +10,45 @@ import torch
 from . import ops
 from .library import F, I, KernelError, P, call, register_signatures
 from .ops import _check, dtype_code, stream_handle
+from .packing import Weight, pack_weight
 
 register_signatures({
-    "fl_gemm_skinny": [P, P, P, I, I, I, I, P],
+    "fl_gemm_skinny": [P, P, P, I, I, I, I, I, P],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
 })
 
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny(x, w, out):
+def gemm_skinny(x, w_packed, out, waves_per_block: int = 0):
+    """``out = x @ w.T`` for up to 64 rows of x; ``w_packed`` = ``pack_weight(w)``, N rows taken
+    from ``out``."""
     M, K = x.shape
-    N = w.shape[0]
-    call("fl_gemm_skinny", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w, "gemm.w", torch.bfloat16, (N, K)),
-         _check(out, "gemm.out", None, (M, N)), dtype_code(out.dtype), M, N, K, stream_handle())
+    N = out.shape[1]
+    need = (-(-N // 16) * 16) * (-(-K // 32) * 32)
+    if w_packed.numel() != need:
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {need}")
+    call("fl_gemm_skinny", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(out, "gemm.out", None, (M, N)), dtype_code(out.dtype), M, N, K, int(waves_per_block), stream_handle())
     return out
 
 
-def gemm(x, w, out):
+def gemm(x, w: Weight, out):
+    """``out = x @ w.T`` with the best kernel that takes the shape."""
     M, K = x.shape
-    if x.dtype == torch.bfloat16 and K % 8 == 0:
-        if M <= SKINNY_MAX_ROWS:
-            return gemm_skinny(x, w, out)
-    return ops.gemm_plain(x, w, out)
+    if w.packed is not None and x.dtype == torch.bfloat16 and K % 8 == 0 and M <= SKINNY_MAX_ROWS:
+        return gemm_skinny(x, w.packed, out)
+    if w.rowmajor is None:
+        raise KernelError(f"gemm: no kernel for {M} rows of a packed [{w.rows}, {w.cols}] matrix")
+    return ops.gemm_plain(x, w.rowmajor, out)
+
+
+def prepare_weight(w: torch.Tensor) -> Weight:
+    """The forms of a weight matrix the tuned path wants."""
+    N, K = w.shape
+    if w.dtype == torch.bfloat16 and K % 8 == 0:
+        return Weight(N, K, rowmajor=w, packed=pack_weight(w))
+    return Weight(N, K, rowmajor=w)
 
 
 # Rows of portions up to this length are treated as single query rows by the split-K kernel;

@@ -51,8 +51,9 @@ class PagedGQAAttention(Mixer):
 
     def bind(self, weights, rt):
         self.rt = rt
-        self.w_qkv = torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0).contiguous()
-        self.w_o = weights["o.weight"]
+        self.w_qkv = rt.prepare_weight(
+            torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0).contiguous())
+        self.w_o = rt.prepare_weight(weights["o.weight"])
         self.position.bind({}, rt)
 
     def forward(self, x, step, cache):

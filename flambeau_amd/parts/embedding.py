@@ -39,9 +39,10 @@ class OutputHead(Part):
 
     def bind(self, weights, rt, embedding_table=None):
         self.rt = rt
-        self.weight = embedding_table if self.tied else weights["weight"]
-        if self.weight is None:
+        table = embedding_table if self.tied else weights["weight"]
+        if table is None:
             raise ValueError("a tied output head needs the embedding table")
+        self.weight = rt.prepare_weight(table)
 
     def forward(self, x, max_rows):
         logits = self.rt.buffer("logits", x.shape[0], self.vocab_size, torch.float32, max_rows=max_rows)

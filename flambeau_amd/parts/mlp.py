@@ -22,8 +22,8 @@ class SwiGLU(FeedForward):
 
     def bind(self, weights, rt):
         self.rt = rt
-        self.w_gate_up = torch.cat([weights["gate.weight"], weights["up.weight"]], dim=0).contiguous()
-        self.w_down = weights["down.weight"]
+        self.w_gate_up = rt.prepare_weight(torch.cat([weights["gate.weight"], weights["up.weight"]], dim=0).contiguous())
+        self.w_down = rt.prepare_weight(weights["down.weight"])
 
     def forward(self, x, step):
         rt, n, I = self.rt, x.shape[0], self.intermediate_size

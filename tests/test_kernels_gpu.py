@@ -108,8 +108,11 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch():
                                    (16, 37, 264), (49, 300, 80)])
 def test_gemm_skinny_against_plain(out_dtype, M, N, K):
     x, w = rnd(M, K, dtype=torch.bfloat16, seed=11), rnd(N, K, dtype=torch.bfloat16, seed=12, scale=0.05)
+    from flambeau_amd.kernels.packing import pack_weight, unpack_weight
+    packed = pack_weight(w)
+    assert torch.equal(unpack_weight(packed, N, K), w)
     got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-    tuned().gemm_skinny(x, w, got)
+    tuned().gemm_skinny(x, packed, got)
     ref = x.double() @ w.double().T
     plain = torch.empty(M, N, dtype=out_dtype, device=DEV)
     ops().gemm_plain(x, w, plain)
@@ -121,17 +124,20 @@ def test_gemm_skinny_against_plain(out_dtype, M, N, K):
 
 def test_gemm_skinny_refuses_what_it_cannot_do():
     from flambeau_amd.kernels import KernelError
+    from flambeau_amd.kernels.packing import pack_weight
     x, w = rnd(2, 36, dtype=torch.bfloat16), rnd(5, 36, dtype=torch.bfloat16)
     out = torch.empty(2, 5, dtype=torch.float32, device=DEV)
     with pytest.raises(KernelError, match="multiple of 8"):
-        tuned().gemm_skinny(x, w, out)
-    tuned().gemm(x, w, out)            # the dispatcher takes the plain kernel instead
+        tuned().gemm_skinny(x, pack_weight(w), out)
+    prepared = tuned().prepare_weight(w)
+    assert prepared.packed is None                 # the dispatcher takes the plain kernel instead
+    tuned().gemm(x, prepared, out)
     assert (out.double() - x.double() @ w.double().T).abs().max() < 1e-4
     with pytest.raises(KernelError, match="at most 64"):
-        tuned().gemm_skinny(rnd(65, 64, dtype=torch.bfloat16), rnd(8, 64, dtype=torch.bfloat16),
+        tuned().gemm_skinny(rnd(65, 64, dtype=torch.bfloat16), pack_weight(rnd(8, 64, dtype=torch.bfloat16)),
                             torch.empty(65, 8, dtype=torch.float32, device=DEV))
-    with pytest.raises(KernelError, match="shape"):
-        tuned().gemm_skinny(rnd(2, 64, dtype=torch.bfloat16), rnd(8, 32, dtype=torch.bfloat16), out)
+    with pytest.raises(KernelError, match="packs to"):
+        tuned().gemm_skinny(rnd(2, 64, dtype=torch.bfloat16), pack_weight(rnd(8, 32, dtype=torch.bfloat16)), out)
 
 
 # ---------------------------------------------------------------- cache, rotation, attention
