@@ -86,5 +86,5 @@ class Runtime:
         """``out = x @ w.T``; ``w`` comes from ``prepare_weight``."""
         if self.tuned:
             from ..kernels import tuned
-            return tuned.gemm(x, w, out)
+            return tuned.gemm(x, w, out, rt=self)
         return ops.gemm_plain(x, w.rowmajor, out)

@@ -14,6 +14,8 @@ from .packing import Weight, pack_weight
 
 register_signatures({
     "fl_gemm_skinny": [P, P, P, I, I, I, I, I, P],
+    "fl_gemm_tiled": [P, P, P, P, I, I, I, I, P],
+    "fl_gemm_tiled_splits": [I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
 })
 
@@ -33,11 +35,44 @@ def gemm_skinny(x, w_packed, out, waves_per_block: int = 0):
     return out
 
 
-def gemm(x, w: Weight, out):
+def gemm_tiled_splits(M: int, N: int, K: int) -> int:
+    from .library import load
+    return load().fl_gemm_tiled_splits(M, N, K)
+
+
+def gemm_tiled(x, w_packed, out, workspace=None):
+    """``out = x @ w.T`` for many rows of x.  A shape whose grid would not fill the chip splits K
+    and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values)."""
+    M, K = x.shape
+    N = out.shape[1]
+    need = (-(-N // 16) * 16) * (-(-K // 32) * 32)
+    if w_packed.numel() != need:
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {need}")
+    splits = gemm_tiled_splits(M, N, K)
+    if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
+        raise KernelError(f"gemm_tiled: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
+    call("fl_gemm_tiled", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(out, "gemm.out", None, (M, N)),
+         _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
+         dtype_code(out.dtype), M, N, K, stream_handle())
+    return out
+
+
+def gemm(x, w: Weight, out, rt=None):
     """``out = x @ w.T`` with the best kernel that takes the shape."""
     M, K = x.shape
-    if w.packed is not None and x.dtype == torch.bfloat16 and K % 8 == 0 and M <= SKINNY_MAX_ROWS:
-        return gemm_skinny(x, w.packed, out)
+    if w.packed is not None and x.dtype == torch.bfloat16 and K % 8 == 0:
+        if M <= SKINNY_MAX_ROWS:
+            return gemm_skinny(x, w.packed, out)
+        N = w.rows
+        splits = gemm_tiled_splits(M, N, K)
+        workspace = None
+        if splits > 1:
+            if rt is None:
+                workspace = torch.empty(splits * M * N, dtype=torch.float32, device=x.device)
+            else:
+                workspace = rt.buffer("gemm_splitk", 1, splits * M * N, torch.float32, max_rows=1)
+        return gemm_tiled(x, w.packed, out, workspace)
     if w.rowmajor is None:
         raise KernelError(f"gemm: no kernel for {M} rows of a packed [{w.rows}, {w.cols}] matrix")
     return ops.gemm_plain(x, w.rowmajor, out)

@@ -368,3 +368,42 @@ def test_attn_decode_subset_of_rows_leaves_the_others_alone():
     ref = attention_case_ref(case, 0.125, 0)
     assert (out[[0, 2, 3]] == 7.0).all()
     assert (out[[1, 4]].double().reshape(2, nh, hd) - ref[[1, 4]]).abs().max() < 1e-2 * ref.abs().max()
+
+
+# ---------------------------------------------------------------- tiled matrix product
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (65, 100, 72), (300, 250, 40), (2048, 512, 256), (129, 37, 264),
+                                   (70, 4096, 4096), (200, 6144, 512), (513, 384, 96), (1000, 130, 1000)])
+def test_gemm_tiled_against_plain(out_dtype, M, N, K):
+    from flambeau_amd.kernels.packing import pack_weight
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=21), rnd(N, K, dtype=torch.bfloat16, seed=22, scale=0.05)
+    got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+    splits = tuned().gemm_tiled_splits(M, N, K)
+    ws = torch.empty(splits * M * N, dtype=torch.float32, device=DEV) if splits > 1 else None
+    tuned().gemm_tiled(x, pack_weight(w), got, ws)
+    ref = x.double() @ w.double().T
+    scale = ref.abs().max()
+    tol = 1e-5 if out_dtype == torch.float32 else 5e-3
+    assert (got.double() - ref).abs().max() < tol * scale
+
+
+def test_gemm_tiled_splits_k_for_small_grids():
+    assert tuned().gemm_tiled_splits(2048, 4096, 4096) == 1
+    assert tuned().gemm_tiled_splits(128, 4096, 4096) > 1
+    from flambeau_amd.kernels import KernelError
+    from flambeau_amd.kernels.packing import pack_weight
+    x, w = rnd(128, 4096, dtype=torch.bfloat16), rnd(256, 4096, dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="workspace"):
+        tuned().gemm_tiled(x, pack_weight(w), torch.empty(128, 256, dtype=torch.float32, device=DEV))
+
+
+def test_gemm_dispatch_rows_agree_across_kernels():
+    """The same row through the skinny and the tiled kernel: equal up to float rounding of sums."""
+    w = rnd(512, 1024, dtype=torch.bfloat16, seed=23, scale=0.05)
+    x = rnd(200, 1024, dtype=torch.bfloat16, seed=24)
+    W = tuned().prepare_weight(w)
+    big = torch.empty(200, 512, dtype=torch.float32, device=DEV)
+    tuned().gemm(x, W, big)
+    small = torch.empty(3, 512, dtype=torch.float32, device=DEV)
+    tuned().gemm(x[17:20].contiguous(), W, small)
+    assert (big[17:20] - small).abs().max() < 1e-5 * big.abs().max()
