@@ -16,6 +16,7 @@ register_signatures({
     "fl_gemm_skinny": [P, P, P, I, I, I, I, I, P],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
+    "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
 })
 
@@ -93,15 +94,23 @@ DECODE_TARGET_BLOCKS = 1024
 DECODE_MIN_KEYS_PER_SPLIT = 128
 
 
+PREFILL_TILE = 64        # query tokens per block of the tiled kernel
+
+
 def attention_metadata(batch) -> dict:
     """Work lists for the attention kernels of one batch: ``attn_rows`` = the rows that run as
-    single queries (decode rows and rows of short portions)."""
+    single queries (decode rows and rows of short portions); ``attn_tiles`` = (request, first
+    row, rows) for every 64 rows of the longer portions."""
     import numpy as np
-    rows = []
-    for q0, ql in zip(batch.q_starts, batch.q_lens):
+    rows, tiles = [], []
+    for s, (q0, ql) in enumerate(zip(batch.q_starts, batch.q_lens)):
         if ql <= SHORT_PORTION:
             rows += range(q0, q0 + ql)
-    return {"attn_rows": np.asarray(rows, dtype=np.int32)}
+        else:
+            for off in range(0, ql, PREFILL_TILE):
+                tiles.append((s, q0 + off, min(PREFILL_TILE, ql - off)))
+    return {"attn_rows": np.asarray(rows, dtype=np.int32),
+            "attn_tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 3)}
 
 
 def decode_splits(n_items: int, n_kv_heads: int, group: int, max_ctx: int) -> int:
@@ -134,17 +143,40 @@ def attn_decode(q, out, cache, rows, positions, tok_seq, table, n_heads, scale, 
     return out
 
 
+def attn_prefill(q, out, cache, tiles, positions, table, n_heads, scale, window, heads_per_wave: int = 0):
+    n = q.shape[0]
+    hd = cache.head_dim
+    n_tiles = tiles.shape[0]
+    call("fl_attn_prefill", _check(q, "attn.q", torch.bfloat16, (n, n_heads * hd)),
+         _check(out, "attn.out", torch.bfloat16, (n, n_heads * hd)), _check(cache.pool, "attn.cache", torch.bfloat16),
+         _check(tiles, "attn.tiles", torch.int32, (n_tiles, 3)), n_tiles,
+         _check(positions, "attn.positions", torch.int32, (n,)),
+         _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads, hd,
+         cache.page_size, cache.n_pages, float(scale), int(window), int(heads_per_wave), stream_handle())
+    return out
+
+
 def decode_supported(cache) -> bool:
     return cache.pool.dtype == torch.bfloat16 and cache.head_dim % 8 == 0 and cache.head_dim <= 256 \
         and cache.page_size % 4 == 0
 
 
+def prefill_supported(cache) -> bool:
+    ps = cache.page_size
+    return decode_supported(cache) and ps >= 4 and (64 % ps == 0 or ps % 64 == 0)
+
+
 def attention(rt, q, out, cache, step, table, n_heads, scale, window):
-    """Attention of one batch with the tuned kernels: rows of short portions through the
-    split-K kernel; a batch with longer portions falls to the plain kernel as a whole."""
-    rows = step.extra.get("attn_rows")
+    """Attention of one batch with the tuned kernels: rows of short portions through the split-K
+    kernel, longer portions through the tiled kernel.  A cache shape one of them does not take
+    sends the whole batch to the plain kernel."""
+    rows, tiles = step.extra.get("attn_rows"), step.extra.get("attn_tiles")
     batch = step.host
-    if rows is not None and rows.shape[0] == step.n_tokens and decode_supported(cache):
+    if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache)):
+        return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
+    if tiles.shape[0]:
+        attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window)
+    if rows.shape[0]:
         group = n_heads // cache.n_kv_heads
         max_ctx = batch.ctx_bound or batch.max_ctx_len
         if window:
@@ -157,6 +189,6 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
             cap = slots if batch.ctx_bound else max(slots, 4096 * n_heads)     # a fixed-shape step never grows
             part_o = rt.buffer("attn_part_o", slots, hdp, torch.float32, max_rows=cap)
             part_ml = rt.buffer("attn_part_ml", slots, 2, torch.float32, max_rows=cap)
-        return attn_decode(q, out, cache, rows, step.positions, step.tok_seq, table, n_heads, scale, window,
-                           n_split, part_o, part_ml)
-    return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
+        attn_decode(q, out, cache, rows, step.positions, step.tok_seq, table, n_heads, scale, window,
+                    n_split, part_o, part_ml)
+    return out

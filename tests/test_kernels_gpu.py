@@ -407,3 +407,65 @@ def test_gemm_dispatch_rows_agree_across_kernels():
     small = torch.empty(3, 512, dtype=torch.float32, device=DEV)
     tuned().gemm(x[17:20].contiguous(), W, small)
     assert (big[17:20] - small).abs().max() < 1e-5 * big.abs().max()
+
+
+# ---------------------------------------------------------------- tiled attention for portions
+def tiles_for(seqs, tile=64):
+    rows, at = [], 0
+    for s, (_, ql) in enumerate(seqs):
+        for off in range(0, ql, tile):
+            rows.append((s, at + off, min(tile, ql - off)))
+        at += ql
+    return torch.tensor(rows, dtype=torch.int32, device=DEV).reshape(-1, 3)
+
+
+@pytest.mark.parametrize("heads_per_wave", [0, 1])
+@pytest.mark.parametrize("nh,nkv,hd,ps,window", [(32, 8, 128, 16, 0), (4, 2, 16, 8, 16), (6, 1, 24, 16, 0),
+                                                (5, 5, 32, 16, 24), (8, 4, 64, 4, 0), (4, 2, 256, 32, 100),
+                                                (6, 3, 40, 64, 37), (2, 1, 160, 128, 0), (8, 2, 96, 16, 70)])
+def test_attn_prefill_against_plain_and_reference(nh, nkv, hd, ps, window, heads_per_wave):
+    # (context, queries): a whole prompt, a portion deep in a context, one that starts mid-page,
+    # a portion that is no multiple of the tile, a short one
+    seqs = [(200, 200), (300, 70), (ps * 5 + 3, 9), (131, 130), (64, 64), (17, 16)]
+    case = build_attention_case(torch.bfloat16, nh, nkv, hd, ps, seqs, seed=5)
+    n = case["n"]
+    scale = 1 / math.sqrt(hd)
+    q2 = case["q"].reshape(n, nh * hd)
+    out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    tuned().attn_prefill(q2, out, case["cache"], tiles_for(seqs), case["pos_d"], case["table"], nh, scale, window,
+                         heads_per_wave)
+    plain = torch.empty_like(out)
+    ops().attn_plain(q2, plain, case["cache"], case["pos_d"], case["seq_d"], case["table"], nh, scale, window)
+    ref = attention_case_ref(case, scale, window)
+    top = ref.abs().max()
+    err = (out.double().reshape(n, nh, hd) - ref).abs()
+    assert not torch.isnan(out).any()
+    assert err.max() < 1e-2 * top, f"worst at {np.unravel_index(int(err.argmax()), err.shape)}"
+    assert (out.double() - plain.double()).abs().max() < 1.5e-2 * top
+
+
+def test_attn_prefill_peaked_scores_find_single_keys():
+    """One key per query is made to stand out (large q.k): the output must be that key's value
+    row, wherever the key lies: first key, a page's edge, the window's first key, the query itself."""
+    nh, nkv, hd, ps, window = 4, 1, 64, 16, 48
+    seqs = [(160, 160)]
+    case = build_attention_case(torch.bfloat16, nh, nkv, hd, ps, seqs, seed=6)
+    n = 160
+    q = torch.zeros(n, nh, hd, dtype=torch.bfloat16, device=DEV)
+    targets = []
+    K = case["K"][0]
+    for i in range(n):
+        lo = max(0, i - window + 1)
+        t = [lo, i, (i // ps) * ps if (i // ps) * ps >= lo else lo, min(i, lo + 15)][i % 4]
+        targets.append(t)
+        q[i] = (K[t, 0] / K[t, 0].norm() * 60.0).to(torch.bfloat16)          # all heads alike
+    out = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
+    tuned().attn_prefill(q.reshape(n, nh * hd), out, case["cache"], tiles_for(seqs), case["pos_d"], case["table"], nh,
+                         1.0, window)
+    case["q"] = q
+    ref = attention_case_ref(case, 1.0, window)
+    assert (out.double().reshape(n, nh, hd) - ref).abs().max() < 2e-2 * ref.abs().max()
+    # and the reference indeed picks single keys
+    V = case["V"][0]
+    hits = sum(float((ref[i, 0] - V[targets[i], 0]).abs().max()) < 0.05 for i in range(n))
+    assert hits > 0.9 * n
