@@ -125,6 +125,8 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="run only the first layers (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="run one part only and print its numbers (for profiling)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
@@ -138,6 +140,14 @@ def main():
     model, _ = random_model(CONFIG_7B, seed=0, dtype=dtype_name, max_batch_tokens=PROMPT_LEN + 64,
                             std=0.02, gain_std=0.0, n_layers=n_layers)
     sz = sizes(CONFIG_7B, n_layers)
+
+    if a.only == "prefill":
+        t = run_prefill(model, dtype_name)
+        print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": PROMPT_LEN, "tok_s": round(PROMPT_LEN / t, 1),
+                          "frac": round(prefill_flops(sz, PROMPT_LEN) / t / PEAK_FLOPS[a.dtype], 4)}))
+        return 0
+    if a.only == "decode":
+        a.no_points = True
 
     dt, mean_ctx = run_decode(model, a.batch, a.steps, a.warmup, dtype_name)
     tok_s = a.batch * a.steps / dt

@@ -37,11 +37,12 @@ int fl_sample(const float* logits, const float* inv_temp, const float* uniform, 
 
 // ---- tuned bf16 kernels ----
 // nw_hint: waves per block that split K (0: chosen from the sizes)
-int fl_gemm_skinny(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K,
-                   int nw_hint, hipStream_t stream);
+// epilogue: 0 = plain product; 1 = SwiGLU over interleaved gate/up rows, out_cols <= N / 2
+int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
+                   int nw_hint, int epilogue, int out_cols, hipStream_t stream);
 
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
-                  int M, int N, int K, hipStream_t stream);
+                  int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_tiled_splits(int M, int N, int K);
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                    const int* items, int n_items, const int* positions, const int* tok_seq,

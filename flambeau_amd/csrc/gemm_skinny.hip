@@ -28,11 +28,14 @@ __device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
     *(bf16x4*)p = o;
 }
 
-template <int MT, typename TOut>
+// SWIGLU: the rows of w are gate and up rows interleaved in fours ([g0-3 | u0-3 | g4-7 | u4-7] per
+// group of 16, see interleave_gate_up in kernels/packing.py); the kernel then writes
+// silu(gate) * up, N / 2 values per token, instead of the N products.
+template <int MT, typename TOut, bool SWIGLU>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ wp,
                                                            TOut* __restrict__ out, int M, int N, int K,
-                                                           int n_steps, int vec_out) {
+                                                           int n_steps, int out_cols) {
     extern __shared__ float red[];               // [NW][MT][64][4]
     const int nw = blockDim.x >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -92,15 +95,33 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
                 const f32x4 v = *(f32x4*)(red + (((size_t)ww * MT + mt) * 64 + lane) * 4);
                 sum += v;
             }
-            // lane (token li, group g) holds features 16*block + 4g .. 4g+3 of token mt*16 + li
+            // lane (token li, group g) holds rows 16*block + 4g .. 4g+3 of token mt*16 + li
             const int tok = mt * 16 + li;
-            const int f0 = blockIdx.x * 16 + 4 * g;
-            if (tok < M && f0 < N) {
-                TOut* p = out + (size_t)tok * N + f0;
-                if (vec_out && f0 + 4 <= N) {
-                    store4(p, sum);
-                } else {
-                    for (int r = 0; r < 4 && f0 + r < N; ++r) p[r] = from_f32<TOut>(sum[r]);
+            if (SWIGLU) {
+                f32x4 up;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) up[r] = __shfl_down(sum[r], 16, 64);      // lane g+1 holds the up rows
+                const int f0 = blockIdx.x * 8 + 2 * g;                                 // g even: features 8 b + 4 (g / 2)
+                if ((g & 1) == 0 && tok < M && f0 < out_cols) {
+                    f32x4 act;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) act[r] = sum[r] / (1.0f + expf(-sum[r])) * up[r];
+                    TOut* p = out + (size_t)tok * out_cols + f0;
+                    if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
+                        store4(p, act);
+                    } else {
+                        for (int r = 0; r < 4 && f0 + r < out_cols; ++r) p[r] = from_f32<TOut>(act[r]);
+                    }
+                }
+            } else {
+                const int f0 = blockIdx.x * 16 + 4 * g;
+                if (tok < M && f0 < N) {
+                    TOut* p = out + (size_t)tok * N + f0;
+                    if (N % 4 == 0 && f0 + 4 <= N) {
+                        store4(p, sum);
+                    } else {
+                        for (int r = 0; r < 4 && f0 + r < N; ++r) p[r] = from_f32<TOut>(sum[r]);
+                    }
                 }
             }
         }
@@ -109,7 +130,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 
 template <int MT, typename TOut>
 static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
-                         hipStream_t stream) {
+                         int swiglu, int out_cols, hipStream_t stream) {
     const int groups = ceil_div(N, 16);
     const int n_steps = ceil_div(K, 32);
     // enough waves in flight to cover the memory latency: about 2048 and more over the chip
@@ -118,24 +139,31 @@ static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, in
     if (nw_hint > 0) nw = nw_hint;
     while (nw > 1 && n_steps < nw * 2) nw /= 2;
     const size_t lds = (size_t)nw * MT * 64 * 4 * sizeof(float);
-    const int vec_out = (N % 4 == 0) ? 1 : 0;      // 16-byte stores need aligned rows
-    gemm_skinny_kernel<MT, TOut><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, vec_out);
+    if (swiglu)
+        gemm_skinny_kernel<MT, TOut, true><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols);
+    else
+        gemm_skinny_kernel<MT, TOut, false><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols);
     return 0;
 }
 
+// epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): w holds N interleaved gate/up rows and
+// out[M, out_cols] = silu(gate) * up with out_cols <= N / 2.
 extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N,
-                              int K, int nw_hint, hipStream_t stream) {
+                              int K, int nw_hint, int epilogue, int out_cols, hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
     FL_CHECK(nw_hint >= 0 && nw_hint <= 16, "gemm_skinny: %d waves per block, at most 16", nw_hint);
     FL_CHECK(K % 8 == 0, "gemm_skinny: K=%d is no multiple of 8 (16-byte loads)", K);
+    FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_skinny: unknown epilogue %d", epilogue);
+    FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
+             "gemm_skinny: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
              "gemm_skinny: operands must be 16-byte aligned");
     if (M == 0) return 0;
     const int mt = ceil_div(M, 16);
 #define FL_SK(MT_)                                                                                         \
-    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N, K, nw_hint, stream); \
-    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M, N, K, nw_hint, stream)
+    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N, K, nw_hint, epilogue, out_cols, stream); \
+    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M, N, K, nw_hint, epilogue, out_cols, stream)
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
     switch (mt) {
         case 1: FL_SK(1); break;

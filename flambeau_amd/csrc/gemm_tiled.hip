@@ -36,11 +36,13 @@ template <> __device__ __forceinline__ void tg_store4<bf16_t>(bf16_t* p, f32x4 v
     *(bf16x4*)p = o;
 }
 
-template <typename TOut>
+// SWIGLU: w holds gate and up rows interleaved in fours; the block writes silu(gate) * up,
+// out_cols <= N / 2 values per token (never together with a split of K).
+template <typename TOut, bool SWIGLU>
 __global__ __launch_bounds__(256, 2) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
                                                             const bf16_t* __restrict__ wp,
                                                             TOut* __restrict__ out, int M, int N, int K,
-                                                            int n_steps, int steps_per_split, int vec_out) {
+                                                            int n_steps, int steps_per_split, int out_cols) {
     // [buffer][operand tile row (8)][k-step in slice (2)][512 values]
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][TG_BM / 16][2][TG_TILE];
     __shared__ __attribute__((aligned(16))) bf16_t ws[2][TG_BN / 16][2][TG_TILE];
@@ -118,9 +120,38 @@ __global__ __launch_bounds__(256, 2) void gemm_tiled_kernel(const bf16_t* __rest
         buf ^= 1;
     }
 
-    // ---- store: lane (token j = lane % 16, g) holds features 4 g .. 4 g + 3 of tile (ta, tb)
-    TOut* obase = out + (size_t)blockIdx.z * M * N;
+    // ---- store: lane (token j = lane % 16, g) holds rows 4 g .. 4 g + 3 of tile (ta, tb)
     const int j = lane & 15, g = lane >> 4;
+    if (SWIGLU) {
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) {
+            const int tok = m0 + (wm * 4 + tb) * 16 + j;
+#pragma unroll
+            for (int ta = 0; ta < 4; ++ta) {
+                f32x4 up;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) up[r] = __shfl_down(acc[ta][tb][r], 16, 64);
+                const int f0 = (n0 >> 1) + (wn * 4 + ta) * 8 + 2 * g;
+                if ((g & 1) == 0 && tok < M && f0 < out_cols) {
+                    f32x4 act;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float gv = acc[ta][tb][r];
+                        act[r] = gv / (1.0f + expf(-gv)) * up[r];
+                    }
+                    TOut* p = out + (size_t)tok * out_cols + f0;
+                    if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
+                        tg_store4<TOut>(p, act);
+                    } else {
+                        for (int r = 0; r < 4 && f0 + r < out_cols; ++r) p[r] = from_f32<TOut>(act[r]);
+                    }
+                }
+            }
+        }
+        return;
+    }
+    TOut* obase = out + (size_t)blockIdx.z * M * N;
+    const int vec_out = (N % 4 == 0) ? 1 : 0;
 #pragma unroll
     for (int tb = 0; tb < 4; ++tb) {
         const int tok = m0 + (wm * 4 + tb) * 16 + j;
@@ -159,24 +190,35 @@ extern "C" int fl_gemm_tiled_splits(int M, int N, int K) {
     return splits;
 }
 
+// epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up from the
+// N interleaved gate/up rows of w (K is not split then).
 extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace,
-                             int out_dtype, int M, int N, int K, hipStream_t stream) {
+                             int out_dtype, int M, int N, int K, int epilogue, int out_cols,
+                             hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_tiled: unknown output dtype %d", out_dtype);
+    FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_tiled: unknown epilogue %d", epilogue);
+    FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
+             "gemm_tiled: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
              "gemm_tiled: operands must be 16-byte aligned");
     if (M == 0) return 0;
     const int n_steps = ceil_div(K, 32);
-    const int splits = fl_gemm_tiled_splits(M, N, K);
+    const int splits = epilogue ? 1 : fl_gemm_tiled_splits(M, N, K);
     FL_CHECK(splits == 1 || workspace, "gemm_tiled: this shape splits K %d ways and needs a workspace", splits);
     int per = ceil_div(n_steps, splits);
     per += per & 1;                                    // whole slices of two steps
     dim3 grid(ceil_div(N, TG_BN), ceil_div(M, TG_BM), splits);
-    const int vec_out = (N % 4 == 0) ? 1 : 0;
-    if (splits > 1) {
-        gemm_tiled_kernel<float><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N,
-                                                           K, n_steps, per, vec_out);
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)w_packed;
+    if (epilogue) {
+        if (out_dtype == FL_F32)
+            gemm_tiled_kernel<float, true><<<grid, 256, 0, stream>>>(xb, wb, (float*)out, M, N, K, n_steps, per, out_cols);
+        else
+            gemm_tiled_kernel<bf16_t, true><<<grid, 256, 0, stream>>>(xb, wb, (bf16_t*)out, M, N, K, n_steps, per, out_cols);
+    } else if (splits > 1) {
+        gemm_tiled_kernel<float, false><<<grid, 256, 0, stream>>>(xb, wb, workspace, M, N, K, n_steps, per, N);
         FL_LAUNCH_CHECK();
         const size_t total = (size_t)M * N;
         const unsigned rb = (unsigned)((total + 255) / 256);
@@ -185,11 +227,9 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
         else
             gemm_splitk_reduce_kernel<bf16_t><<<rb, 256, 0, stream>>>(workspace, (bf16_t*)out, total, splits);
     } else if (out_dtype == FL_F32) {
-        gemm_tiled_kernel<float><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N,
-                                                           K, n_steps, per, vec_out);
+        gemm_tiled_kernel<float, false><<<grid, 256, 0, stream>>>(xb, wb, (float*)out, M, N, K, n_steps, per, N);
     } else {
-        gemm_tiled_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M,
-                                                            N, K, n_steps, per, vec_out);
+        gemm_tiled_kernel<bf16_t, false><<<grid, 256, 0, stream>>>(xb, wb, (bf16_t*)out, M, N, K, n_steps, per, N);
     }
     FL_LAUNCH_CHECK();
     return 0;

@@ -82,9 +82,27 @@ class Runtime:
         from ..kernels.packing import Weight
         return Weight(w.shape[0], w.shape[1], rowmajor=w)
 
+    def prepare_gate_up(self, gate: torch.Tensor, up: torch.Tensor):
+        """Gate and up matrices of a gated feed-forward as one weight for ``gemm_swiglu``."""
+        if self.tuned:
+            from ..kernels import tuned
+            return tuned.prepare_gate_up(gate, up)
+        from ..kernels.packing import Weight
+        return Weight(2 * gate.shape[0], gate.shape[1], rowmajor=torch.cat([gate, up], dim=0).contiguous())
+
     def gemm(self, x, w, out):
         """``out = x @ w.T``; ``w`` comes from ``prepare_weight``."""
         if self.tuned:
             from ..kernels import tuned
             return tuned.gemm(x, w, out, rt=self)
         return ops.gemm_plain(x, w.rowmajor, out)
+
+    def gemm_swiglu(self, x, w, out):
+        """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``.  The tuned
+        kernels apply the gate before they store; the plain path is a product and a gate kernel."""
+        if self.tuned:
+            from ..kernels import tuned
+            return tuned.gemm_swiglu(x, w, out, self)
+        gu = self.buffer("ffn_gate_up", x.shape[0], w.rows, torch.float32)
+        ops.gemm_plain(x, w.rowmajor, gu)
+        return ops.silu_mul(gu, out)

@@ -31,6 +31,20 @@ def unpack_weight(packed: torch.Tensor, N: int, K: int) -> torch.Tensor:
     return t[:N, :K].contiguous()
 
 
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """Gate and up rows interleaved in fours, ``[g0-3 | u0-3 | g4-7 | u4-7]`` per eight features
+    (I padded to a multiple of 8 with zero rows): one matrix-core tile of 16 rows then holds
+    gate and up of the same eight features, and a kernel can apply ``silu(gate) * up`` before
+    it stores."""
+    I, K = gate.shape
+    Ip = -(-I // 8) * 8
+    if Ip != I:
+        pad = torch.zeros((Ip - I, K), dtype=gate.dtype, device=gate.device)
+        gate, up = torch.cat([gate, pad]), torch.cat([up, pad])
+    g, u = gate.view(Ip // 8, 2, 4, K), up.view(Ip // 8, 2, 4, K)
+    return torch.stack([g[:, 0], u[:, 0], g[:, 1], u[:, 1]], dim=1).reshape(2 * Ip, K).contiguous()
+
+
 @dataclass
 class Weight:
     """A matrix ``[rows, cols]`` (out features, in features) as the kernels take it: row-major,
@@ -39,6 +53,8 @@ class Weight:
     cols: int
     rowmajor: torch.Tensor | None = None
     packed: torch.Tensor | None = None
+    packed_rows: int = 0          # rows the packed form was built from (with interleaving and padding)
+    swiglu_cols: int = 0          # > 0: the packed form holds interleaved gate/up rows of this many features
 
     @property
     def shape(self):

@@ -10,11 +10,11 @@ import torch
 from . import ops
 from .library import F, I, KernelError, P, call, register_signatures
 from .ops import _check, dtype_code, stream_handle
-from .packing import Weight, pack_weight
+from .packing import Weight, interleave_gate_up, pack_weight
 
 register_signatures({
-    "fl_gemm_skinny": [P, P, P, I, I, I, I, I, P],
-    "fl_gemm_tiled": [P, P, P, P, I, I, I, I, P],
+    "fl_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, P],
+    "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
@@ -23,16 +23,21 @@ register_signatures({
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny(x, w_packed, out, waves_per_block: int = 0):
+def _packed_size(n_rows: int, K: int) -> int:
+    return (-(-n_rows // 16) * 16) * (-(-K // 32) * 32)
+
+
+def gemm_skinny(x, w_packed, out, waves_per_block: int = 0, swiglu_rows: int = 0):
     """``out = x @ w.T`` for up to 64 rows of x; ``w_packed`` = ``pack_weight(w)``, N rows taken
-    from ``out``."""
+    from ``out``.  With ``swiglu_rows`` the packed matrix holds that many interleaved gate/up
+    rows and ``out`` receives ``silu(gate) * up``."""
     M, K = x.shape
-    N = out.shape[1]
-    need = (-(-N // 16) * 16) * (-(-K // 32) * 32)
-    if w_packed.numel() != need:
-        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {need}")
+    N = swiglu_rows or out.shape[1]
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
     call("fl_gemm_skinny", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         _check(out, "gemm.out", None, (M, N)), dtype_code(out.dtype), M, N, K, int(waves_per_block), stream_handle())
+         _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, int(waves_per_block),
+         1 if swiglu_rows else 0, out.shape[1], stream_handle())
     return out
 
 
@@ -41,28 +46,28 @@ def gemm_tiled_splits(M: int, N: int, K: int) -> int:
     return load().fl_gemm_tiled_splits(M, N, K)
 
 
-def gemm_tiled(x, w_packed, out, workspace=None):
+def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0):
     """``out = x @ w.T`` for many rows of x.  A shape whose grid would not fill the chip splits K
-    and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values)."""
+    and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values).  With
+    ``swiglu_rows`` see ``gemm_skinny``."""
     M, K = x.shape
-    N = out.shape[1]
-    need = (-(-N // 16) * 16) * (-(-K // 32) * 32)
-    if w_packed.numel() != need:
-        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {need}")
-    splits = gemm_tiled_splits(M, N, K)
+    N = swiglu_rows or out.shape[1]
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    splits = 1 if swiglu_rows else gemm_tiled_splits(M, N, K)
     if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
         raise KernelError(f"gemm_tiled: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
     call("fl_gemm_tiled", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         _check(out, "gemm.out", None, (M, N)),
+         _check(out, "gemm.out", None, (M, None)),
          _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-         dtype_code(out.dtype), M, N, K, stream_handle())
+         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], stream_handle())
     return out
 
 
 def gemm(x, w: Weight, out, rt=None):
     """``out = x @ w.T`` with the best kernel that takes the shape."""
     M, K = x.shape
-    if w.packed is not None and x.dtype == torch.bfloat16 and K % 8 == 0:
+    if w.packed is not None and not w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
         if M <= SKINNY_MAX_ROWS:
             return gemm_skinny(x, w.packed, out)
         N = w.rows
@@ -79,12 +84,33 @@ def gemm(x, w: Weight, out, rt=None):
     return ops.gemm_plain(x, w.rowmajor, out)
 
 
+def gemm_swiglu(x, w: Weight, out, rt):
+    """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``."""
+    M, K = x.shape
+    if w.packed is not None and w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
+        if M <= SKINNY_MAX_ROWS:
+            return gemm_skinny(x, w.packed, out, swiglu_rows=w.packed_rows)
+        return gemm_tiled(x, w.packed, out, swiglu_rows=w.packed_rows)
+    gu = rt.buffer("ffn_gate_up", M, w.rows, torch.float32)
+    ops.gemm_plain(x, w.rowmajor, gu)
+    return ops.silu_mul(gu, out)
+
+
 def prepare_weight(w: torch.Tensor) -> Weight:
-    """The forms of a weight matrix the tuned path wants."""
+    """The form of a weight matrix the tuned path wants: packed tiles when the kernels take the
+    shape (the row-major matrix is dropped then), else row-major for the plain kernel."""
     N, K = w.shape
     if w.dtype == torch.bfloat16 and K % 8 == 0:
-        return Weight(N, K, rowmajor=w, packed=pack_weight(w))
+        return Weight(N, K, packed=pack_weight(w), packed_rows=N)
     return Weight(N, K, rowmajor=w)
+
+
+def prepare_gate_up(gate: torch.Tensor, up: torch.Tensor) -> Weight:
+    I, K = gate.shape
+    if gate.dtype == torch.bfloat16 and K % 8 == 0:
+        inter = interleave_gate_up(gate, up)
+        return Weight(2 * I, K, packed=pack_weight(inter), packed_rows=inter.shape[0], swiglu_cols=I)
+    return Weight(2 * I, K, rowmajor=torch.cat([gate, up], dim=0).contiguous())
 
 
 # Rows of portions up to this length are treated as single query rows by the split-K kernel;

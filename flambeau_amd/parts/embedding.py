@@ -42,6 +42,7 @@ class OutputHead(Part):
         table = embedding_table if self.tied else weights["weight"]
         if table is None:
             raise ValueError("a tied output head needs the embedding table")
+        # a tied head packs its own copy: the embedding keeps the row-major table for its gather
         self.weight = rt.prepare_weight(table)
 
     def forward(self, x, max_rows):

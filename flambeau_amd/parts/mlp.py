@@ -1,11 +1,10 @@
 """Dense SwiGLU feed-forward: d = (silu(x Wg^T) * (x Wu^T)) Wd^T
 (crates/forward/src/core/composites/dense_ffn.rs:116-186).  Gate and up matrices are
-joined at load so that one matrix product feeds both."""
+joined at load so that one matrix product feeds both and applies the gate before it stores."""
 from __future__ import annotations
 
 import torch
 
-from ..kernels import ops
 from .base import FEED_FORWARDS, FeedForward, TensorSpec
 
 
@@ -22,15 +21,13 @@ class SwiGLU(FeedForward):
 
     def bind(self, weights, rt):
         self.rt = rt
-        self.w_gate_up = rt.prepare_weight(torch.cat([weights["gate.weight"], weights["up.weight"]], dim=0).contiguous())
+        self.w_gate_up = rt.prepare_gate_up(weights["gate.weight"], weights["up.weight"])
         self.w_down = rt.prepare_weight(weights["down.weight"])
 
     def forward(self, x, step):
         rt, n, I = self.rt, x.shape[0], self.intermediate_size
-        gu = rt.buffer("ffn_gate_up", n, 2 * I, torch.float32)
-        rt.gemm(x, self.w_gate_up, gu)
         act = rt.buffer("ffn_act", n, I)
-        ops.silu_mul(gu, act)
+        rt.gemm_swiglu(x, self.w_gate_up, act)
         delta = rt.buffer("delta", n, self.hidden_size, torch.float32)
         rt.gemm(act, self.w_down, delta)
         return delta

@@ -469,3 +469,24 @@ def test_attn_prefill_peaked_scores_find_single_keys():
     V = case["V"][0]
     hits = sum(float((ref[i, 0] - V[targets[i], 0]).abs().max()) < 0.05 for i in range(n))
     assert hits > 0.9 * n
+
+
+# ---------------------------------------------------------------- gated feed-forward in the product's epilogue
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,I,K", [(1, 14336, 4096), (8, 224, 96), (64, 136, 80), (5, 13, 40), (200, 14336, 512),
+                                   (65, 160, 64), (300, 52, 72), (16, 8, 8)])
+def test_gemm_swiglu_epilogue(out_dtype, M, I, K):
+    gate = rnd(I, K, dtype=torch.bfloat16, seed=31, scale=0.3)
+    up = rnd(I, K, dtype=torch.bfloat16, seed=32, scale=0.3)
+    x = rnd(M, K, dtype=torch.bfloat16, seed=33)
+    W = tuned().prepare_gate_up(gate, up)
+    assert W.packed is not None and W.swiglu_cols == I and W.packed_rows % 16 == 0
+    got = torch.full((M, I), float("nan"), dtype=out_dtype, device=DEV)
+    if M <= 64:
+        tuned().gemm_skinny(x, W.packed, got, swiglu_rows=W.packed_rows)
+    else:
+        tuned().gemm_tiled(x, W.packed, got, swiglu_rows=W.packed_rows)
+    g, u = x.double() @ gate.double().T, x.double() @ up.double().T
+    ref = g / (1 + torch.exp(-g)) * u
+    tol = 2e-5 if out_dtype == torch.float32 else 6e-3
+    assert (got.double() - ref).abs().max() < tol * ref.abs().max()
