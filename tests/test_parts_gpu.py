@@ -1,0 +1,344 @@
+"""Each part alone against the plain implementation, at sizes of its own, and the generality of
+the arrangement: a toy mixer with state of its own, a toy position encoding and a toy
+architecture are defined HERE, registered, built from a config.json and stepped, without a
+change to the framework's files."""
+import json
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def make_rt(dtype, tuned=True, max_tokens=256):
+    from flambeau_amd.engine import Runtime
+    return Runtime(DEV, dtype, max_tokens, tuned)
+
+
+def rnd(*shape, scale=1.0, seed=0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 2e-2
+
+
+def put(rt, t, role="matrix"):
+    return rt.to_device(t, role)
+
+
+def step_for(rt, seqs, page_size, n_pages, shuffle_seed=0):
+    """A StepState for requests ``seqs`` = (start position, tokens): pages handed out in a
+    shuffled order, everything a mixer reads on the device."""
+    from flambeau_amd.parts import HostBatch, StepState
+    from flambeau_amd.kernels import tuned
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(shuffle_seed)).tolist()
+    q_starts, q_lens, starts, pos, tok_seq = [], [], [], [], []
+    width = max(-(-(st + q) // page_size) for st, q in seqs) + 1
+    table = np.full((len(seqs), width), -1, dtype=np.int32)
+    at = 0
+    for s, (st, q) in enumerate(seqs):
+        nb = -(-(st + q) // page_size)
+        table[s, :nb] = [perm.pop() for _ in range(nb)]
+        q_starts.append(at); q_lens.append(q); starts.append(st)
+        pos += range(st, st + q); tok_seq += [s] * q
+        at += q
+    batch = HostBatch(q_starts, q_lens, starts, list(range(len(seqs))), at, 0)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=DEV)
+    extra = {k: i32(v) for k, v in tuned.attention_metadata(batch).items()}
+    extra["attn_tiles"] = extra["attn_tiles"].reshape(-1, 3)
+    return StepState(n_tokens=at, n_seqs=len(seqs), tokens=i32([0] * at), positions=i32(pos), tok_seq=i32(tok_seq),
+                     seq_slots=i32(range(len(seqs))), seq_q_start=i32(q_starts), seq_q_len=i32(q_lens),
+                     seq_ctx_len=i32([st + q for st, q in seqs]), block_tables=[i32(table)], logit_rows=i32([]),
+                     host=batch, extra=extra)
+
+
+# ---------------------------------------------------------------- norm, feed-forward, embedding, head
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(dtype):
+    from flambeau_amd.parts import NORMS, PartSpec
+    rt = make_rt(dtype)
+    H, eps = 200, 3e-4
+    norm = NORMS.create(PartSpec("rmsnorm", dict(hidden_size=H, eps=eps)))
+    assert norm.tensors()["weight"].shape == (H,) and norm.tensors()["weight"].role == "vector32"
+    w = 1 + rnd(H, scale=0.2, seed=1)
+    norm.bind({"weight": put(rt, w, "vector32")}, rt)
+    x, d = rnd(9, H, seed=2), rnd(9, H, scale=0.5, seed=3)
+    xd = x.to(DEV)
+    out = torch.empty(9, H, dtype=dtype, device=DEV)
+    norm.forward(xd, out, delta=d.to(DEV), store_sum=True)
+    want = pm.rmsnorm((x + d).numpy(), w.numpy(), eps)
+    assert np.abs(out.double().cpu().numpy() - want).max() < tol(dtype) * np.abs(want).max()
+    assert torch.equal(xd.cpu(), x + d)
+
+
+@pytest.mark.parametrize("tuned", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [3, 130])
+def test_swiglu_part(dtype, tuned, n):
+    from flambeau_amd.parts import FEED_FORWARDS, PartSpec
+    rt = make_rt(dtype, tuned)
+    H, I = 72, 152
+    ffn = FEED_FORWARDS.create(PartSpec("swiglu", dict(hidden_size=H, intermediate_size=I)))
+    assert {k: v.shape for k, v in ffn.tensors().items()} == {"gate.weight": (I, H), "up.weight": (I, H), "down.weight": (H, I)}
+    w = {k: rnd(*v.shape, scale=0.2, seed=i).to(dtype) for i, (k, v) in enumerate(ffn.tensors().items())}
+    ffn.bind({k: put(rt, v) for k, v in w.items()}, rt)
+    x = rnd(n, H, seed=9).to(dtype)
+    got = ffn.forward(x.to(DEV), None)
+    assert got.dtype == torch.float32
+    want = pm.swiglu_mlp(x.double().numpy(), *(w[k].double().numpy() for k in ("gate.weight", "up.weight", "down.weight")))
+    assert np.abs(got.double().cpu().numpy() - want).max() < tol(dtype) * np.abs(want).max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tied", [False, True])
+def test_embedding_and_head_parts(dtype, tied):
+    from flambeau_amd.parts import OutputHead, TokenEmbedding
+    rt = make_rt(dtype)
+    V, H = 150, 40
+    emb, head = TokenEmbedding(V, H), OutputHead(V, H, tied=tied)
+    assert ("weight" in head.tensors()) == (not tied)
+    E, W = rnd(V, H, seed=1).to(dtype), rnd(V, H, seed=2).to(dtype)
+    emb.bind({"weight": put(rt, E, "table")}, rt)
+    head.bind({} if tied else {"weight": put(rt, W)}, rt, embedding_table=emb.weight)
+    toks = torch.tensor([3, 149, 0, 77], dtype=torch.int32, device=DEV)
+    resid = torch.empty(4, H, dtype=torch.float32, device=DEV)
+    emb.forward(toks, resid)
+    assert torch.equal(resid.cpu(), E[toks.cpu().long()].float())
+    x = rnd(5, H, seed=3).to(dtype)
+    logits = head.forward(x.to(DEV), max_rows=8)
+    want = pm.linear(x.double().numpy(), (E if tied else W).double().numpy())
+    assert logits.dtype == torch.float32
+    assert np.abs(logits.double().cpu().numpy() - want).max() < tol(dtype) * np.abs(want).max()
+
+
+# ---------------------------------------------------------------- the attention mixer and the block
+def _mixer_weights(mixer, dtype, seed=0, scale=0.25):
+    return {k: rnd(*v.shape, scale=scale, seed=seed + i).to(dtype) for i, (k, v) in enumerate(mixer.tensors().items())}
+
+
+@pytest.mark.parametrize("tuned", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,window,theta,ps", [(6, 2, 24, 0, 1e4, 8), (4, 4, 16, 13, 1e6, 16), (8, 1, 64, 40, 5e5, 4)])
+def test_attention_mixer_part(dtype, tuned, nh, nkv, hd, window, theta, ps):
+    """A whole prompt in one step, then the same prompt as a portion, a short portion and single
+    tokens into a second cache: both must equal the plain mixer."""
+    from flambeau_amd.cache.storage import CacheStorage
+    from flambeau_amd.parts import MIXERS, PartSpec
+    rt = make_rt(dtype, tuned)
+    H, n = 56, 75
+    spec = PartSpec("paged_gqa_attention", dict(hidden_size=H, n_heads=nh, n_kv_heads=nkv, head_dim=hd, window=window,
+                                                position=PartSpec("rope_neox", dict(head_dim=hd, theta=theta))))
+    mixer = MIXERS.create(spec)
+    w = _mixer_weights(mixer, dtype)
+    mixer.bind({k: put(rt, v) for k, v in w.items()}, rt)
+    x = rnd(n, H, seed=7).to(dtype)
+    wd = {"a." + k.replace(".weight", "_proj.weight"): v.double().numpy() for k, v in w.items()}
+    want = pm.attention_mixer(x.double().numpy(), wd, "a.", np.arange(n), nh, nkv, hd, theta, window)
+    for cuts in ([n], [40, 5, 1, 1, 20, 2, 6]):
+        store = CacheStorage([mixer.cache_spec()], [None], rt.device, dtype, n_pages=32, page_size=ps, max_slots=2)
+        got, at = [], 0
+        for k in cuts:
+            step = step_for(rt, [(at, k)], ps, 32, shuffle_seed=1)       # same seed: the same pages every step
+            got.append(mixer.forward(x[at:at + k].to(DEV).contiguous(), step, store.entries[0]).double().cpu().numpy())
+            at += k
+        got = np.concatenate(got)
+        assert np.abs(got - want).max() < tol(dtype) * np.abs(want).max(), cuts
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_prenorm_block_part(dtype):
+    from flambeau_amd.cache.storage import CacheStorage
+    from flambeau_amd.parts import BLOCKS, PartSpec, ResidualStream
+    rt = make_rt(dtype)
+    H, nh, nkv, hd, I, eps, n = 48, 3, 1, 16, 100, 1e-5, 37
+    norm = PartSpec("rmsnorm", dict(hidden_size=H, eps=eps))
+    mixer = PartSpec("paged_gqa_attention", dict(hidden_size=H, n_heads=nh, n_kv_heads=nkv, head_dim=hd,
+                                                 position=PartSpec("rope_neox", dict(head_dim=hd, theta=1e4))))
+    ffn = PartSpec("swiglu", dict(hidden_size=H, intermediate_size=I))
+    block = BLOCKS.create(PartSpec("prenorm", dict(mixer=mixer, feed_forward=ffn, norm=norm)))
+    names = block.tensors()
+    assert set(names) == {"mixer_norm.weight", "mixer.q.weight", "mixer.k.weight", "mixer.v.weight", "mixer.o.weight",
+                          "ffn_norm.weight", "ffn.gate.weight", "ffn.up.weight", "ffn.down.weight"}
+    w = {}
+    for i, (k, ts) in enumerate(names.items()):
+        w[k] = (1 + rnd(*ts.shape, scale=0.1, seed=i)) if ts.role == "vector32" else rnd(*ts.shape, scale=0.2, seed=i).to(dtype)
+    block.bind({k: put(rt, v, names[k].role) for k, v in w.items()}, rt)
+    x = rnd(n, H, seed=50)
+    store = CacheStorage([block.cache_spec()], [None], rt.device, dtype, n_pages=8, page_size=8, max_slots=1)
+    stream = ResidualStream(x.to(DEV), rt)
+    block.forward(stream, step_for(rt, [(0, n)], 8, 8), store.entries[0])
+    got = stream.flush().double().cpu().numpy()
+    W = {k: v.double().numpy() for k, v in w.items()}
+    xs = x.double().numpy()
+    a = pm.rmsnorm(xs, W["mixer_norm.weight"], eps)
+    wd = {"a." + k[6:].replace(".weight", "_proj.weight"): v for k, v in W.items() if k.startswith("mixer.")}
+    xs = xs + pm.attention_mixer(a, wd, "a.", np.arange(n), nh, nkv, hd, 1e4, 0)
+    b = pm.rmsnorm(xs, W["ffn_norm.weight"], eps)
+    want = xs + pm.swiglu_mlp(b, W["ffn.gate.weight"], W["ffn.up.weight"], W["ffn.down.weight"])
+    assert np.abs(got - want).max() < tol(dtype) * np.abs(want).max()
+
+
+# ---------------------------------------------------------------- toy parts, defined here
+def _register_toys():
+    """A mixer with per-request state (a decaying sum of its inputs), a position encoding that is
+    not a rotation (it scales queries and keys by a function of the position), and an
+    architecture that puts them beside the built-in parts, layer by layer."""
+    from dataclasses import dataclass
+    from flambeau_amd.config.base import KeyReader
+    from flambeau_amd.kernels import ops
+    from flambeau_amd.models.decoder import LayerSpec, ModelSpec, RunEntry
+    from flambeau_amd.parts import (MIXERS, POSITION_ENCODINGS, Mixer, PartSpec, PositionEncoding, StateSpec, TensorSpec)
+    from flambeau_amd.registry import register_architecture
+
+    if "toy_decay_sum" in MIXERS.known():
+        return
+
+    @MIXERS.register("toy_decay_sum")
+    class DecaySum(Mixer):
+        """s <- decay * s + x_t (per request, in order); delta_t = s W^T."""
+        def __init__(self, hidden_size, decay):
+            self.hidden_size, self.decay = hidden_size, decay
+
+        def cache_spec(self):
+            return StateSpec((self.hidden_size,), torch.float32)
+
+        def tensors(self):
+            return {"w.weight": TensorSpec((self.hidden_size, self.hidden_size))}
+
+        def bind(self, weights, rt):
+            self.rt, self.w = rt, rt.prepare_weight(weights["w.weight"])
+
+        def forward(self, x, step, cache):
+            n, H = x.shape
+            sums = torch.empty(n, H, dtype=torch.float32, device=x.device)
+            for q0, ql, slot in zip(step.host.q_starts, step.host.q_lens, step.host.slots):
+                s = cache.state[slot]
+                for i in range(q0, q0 + ql):
+                    s = self.decay * s + x[i].float()
+                    sums[i] = s
+                cache.state[slot] = s
+            delta = self.rt.buffer("delta", n, H, torch.float32)
+            self.rt.gemm(sums.to(x.dtype), self.w, delta)
+            return delta
+
+    @POSITION_ENCODINGS.register("toy_position_scale")
+    class PositionScale(PositionEncoding):
+        """q and k of position p are multiplied by 1 + rate * cos(p): no rotation, so the mixer
+        calls ``apply`` and stores without rotating."""
+        def __init__(self, rate):
+            self.rate = rate
+
+        def apply(self, qkv, positions, n_heads, n_kv_heads, head_dim):
+            f = 1.0 + self.rate * torch.cos(positions.float())
+            qkv[:, :(n_heads + n_kv_heads) * head_dim] *= f[:, None]
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        hidden_size: int
+        vocab_size: int
+        layer_kinds: tuple
+        decay: float
+        rate: float
+        max_position_embeddings: int
+
+        @classmethod
+        def from_dict(cls, raw, where="config.json"):
+            r = KeyReader(raw, where)
+            return cls(r.integer("hidden_size"), r.integer("vocab_size"), tuple(raw["layer_kinds"]),
+                       r.number("decay"), r.number("rate"), r.integer("max_position_embeddings"))
+
+    def toy_spec(cfg):
+        H = cfg.hidden_size
+        norm = PartSpec("rmsnorm", dict(hidden_size=H, eps=1e-5))
+        ffn = PartSpec("swiglu", dict(hidden_size=H, intermediate_size=2 * H))
+        mixers = {
+            "decay": PartSpec("toy_decay_sum", dict(hidden_size=H, decay=cfg.decay)),
+            "attn": PartSpec("paged_gqa_attention", dict(hidden_size=H, n_heads=2, n_kv_heads=1, head_dim=16,
+                                                         position=PartSpec("toy_position_scale", dict(rate=cfg.rate)))),
+        }
+        layers = []
+        for l, kind in enumerate(cfg.layer_kinds):
+            block = PartSpec("prenorm", dict(mixer=mixers[kind], feed_forward=ffn, norm=norm))
+            local = ["w"] if kind == "decay" else ["q", "k", "v", "o"]
+            names = {f"mixer.{t}.weight": f"toy.{l}.mix.{t}" for t in local}
+            names.update({"mixer_norm.weight": f"toy.{l}.n1", "ffn_norm.weight": f"toy.{l}.n2",
+                          "ffn.gate.weight": f"toy.{l}.gate", "ffn.up.weight": f"toy.{l}.up", "ffn.down.weight": f"toy.{l}.down"})
+            layers.append(LayerSpec(block, names))
+        # the order layers run in is data: layer 1 runs twice, its second run reads the first's cache
+        order = [RunEntry(l) for l in range(len(layers))]
+        if cfg.layer_kinds[1] == "attn":
+            order.append(RunEntry(1, cache_of=1))
+        return ModelSpec("ToyStateLM", H, cfg.vocab_size, cfg.max_position_embeddings, layers, order, norm,
+                         {"embedding.weight": "toy.embed", "final_norm.weight": "toy.norm", "head.weight": "toy.head"})
+
+    register_architecture("ToyStateLM", ToyConfig, toy_spec)
+
+
+def _toy_plain(cfg, w, toks):
+    """The toy architecture in numpy, whole sequence."""
+    H, n = cfg["hidden_size"], len(toks)
+    x = w["toy.embed"][toks]
+    order = list(range(len(cfg["layer_kinds"])))
+    if cfg["layer_kinds"][1] == "attn":
+        order.append(1)
+    kept = {}            # keys and values a layer's first run stored
+    for l in order:
+        a = pm.rmsnorm(x, w[f"toy.{l}.n1"], 1e-5)
+        if cfg["layer_kinds"][l] == "decay":
+            s, sums = np.zeros(H), []
+            for t in range(n):
+                s = cfg["decay"] * s + a[t]
+                sums.append(s)
+            d = np.stack(sums) @ w[f"toy.{l}.mix.w"].T
+        else:
+            f = (1.0 + cfg["rate"] * np.cos(np.arange(n)))[:, None, None]
+            q = (a @ w[f"toy.{l}.mix.q"].T).reshape(n, 2, 16) * f
+            if l in kept:                      # the second run reads the cache of the first
+                k, v = kept[l]
+            else:
+                k = (a @ w[f"toy.{l}.mix.k"].T).reshape(n, 1, 16) * f
+                v = (a @ w[f"toy.{l}.mix.v"].T).reshape(n, 1, 16)
+                kept[l] = (k, v)
+            d = pm.attention(q, k, v, np.arange(n), 0.25, 0).reshape(n, 32) @ w[f"toy.{l}.mix.o"].T
+        x = x + d
+        b = pm.rmsnorm(x, w[f"toy.{l}.n2"], 1e-5)
+        x = x + pm.swiglu_mlp(b, w[f"toy.{l}.gate"], w[f"toy.{l}.up"], w[f"toy.{l}.down"])
+    return pm.rmsnorm(x, w["toy.norm"], 1e-5) @ w["toy.head"].T
+
+
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
+    import replay_helpers as rh
+    from flambeau_amd.engine import ModelRunner, load_model
+    from flambeau_amd.weights import write_random_model
+    _register_toys()
+    cfg = dict(architectures=["ToyStateLM"], hidden_size=32, vocab_size=90, layer_kinds=["decay", "attn", "decay"],
+               decay=0.8, rate=0.3, max_position_embeddings=128)
+    d = write_random_model(cfg, tmp_path / "toy", seed=4, std=0.15, gain_std=0.05, store_dtype=torch.float32)
+    model, _ = load_model(d, dtype="float32", max_batch_tokens=128)
+    assert [type(b.mixer).__name__ for b in model.blocks] == ["DecaySum", "PagedGQAAttention", "DecaySum"]
+    runner = ModelRunner(model, n_pages=16, page_size=8, max_slots=3, max_logit_rows=128)
+    assert not runner.decode_graphs                                    # a mixer with state of its own never replays
+    assert len(runner.storage.states) == 2 and len(runner.storage.pools) == 1
+    assert runner.storage.pools[0].shape[0] == 1                       # the repeated layer reads, it owns no cache
+    w = {k: v for k, v in pm.read_safetensors(d / "model.safetensors").items()}
+    reqs = rh.make_requests(90, [30, 17, 41, 9, 25], seed=2)
+    ref = {rid: _toy_plain(cfg, w, toks) for rid, toks in reqs.items()}
+    for mode, steps in [("whole", rh.trace_whole(reqs)), ("tail", rh.trace_tail(reqs, tail=8)),
+                        ("portions", rh.trace_portions(reqs, sizes=(2, 7, 3, 11))),
+                        ("mixed", rh.trace_mixed(reqs, seed=1, max_live=3, max_portion=9, decode_tail=4))]:
+        got = rh.run_in_process(runner, steps)
+        rh.compare(got, reqs, ref, "float32", f"toy {mode}")
+    # slots are zeroed when they are claimed again: a second pass over the same requests agrees
+    rh.compare(rh.run_in_process(runner, rh.trace_mixed(reqs, seed=3, max_live=3)), reqs, ref, "float32", "toy again")
+
+
+def test_unknown_part_names_the_known_ones():
+    from flambeau_amd.parts import MIXERS, PartSpec
+    with pytest.raises(KeyError, match="paged_gqa_attention"):
+        MIXERS.create(PartSpec("no_such_mixer", {}))
