@@ -1,32 +1,34 @@
 // Tiled bf16 matrix product for prompt portions: out[m, n] = sum_k x[m, k] w[n, k] with many
 // rows m, on the matrix cores (v_mfma_f32_16x16x32_bf16, float accumulation).
 //
-//  * w arrives packed (kernels/packing.py): a tile of 16 features x 32 k is 1 KB in lane order,
-//    so the block's slice of w is copied to LDS as it lies in memory, and a wave reads an
-//    operand tile from LDS with one ds_read_b128 per lane at consecutive addresses (no bank
-//    conflicts, no transposition);
-//  * x is row-major; on its way into LDS every 16-byte chunk is put where the same tile layout
-//    wants it, so the x operand is read the same way;
-//  * a block of four waves (2 x 2) computes BM x BN = 128 x 128 outputs, each wave 64 x 64
-//    (16 accumulator tiles); K is walked in slices of 64 with two LDS buffers: the next slice
-//    is fetched from memory into registers while the current one is multiplied;
+//  * w arrives packed (kernels/packing.py): a tile of 16 features x 32 k is 1 KB in lane order.
+//    Operand tiles of both matrices go from memory straight into LDS with
+//    global_load_lds_dwordx4 (no staging registers, no ds_write): for w a wave copies the tile as
+//    it lies; for the row-major x every lane reads the 16 bytes that the tile layout wants at its
+//    place.  A wave then reads an operand from LDS with one ds_read_b128 per lane at consecutive
+//    addresses (no bank conflicts, no transposition);
+//  * LDS is a ring of NS stages of one k-step (32 values of k); one bare s_barrier per stage;
 //  * the w tile is the A operand and the x tile the B operand: C[feature][token] leaves each
 //    lane with four consecutive features of one token, one 16-byte store;
-//  * with few rows and a narrow matrix the grid would not fill the chip: K is then split over
+//  * two shapes: 256 features x 128 tokens per block (a wave computes 8 x 4 tiles: 12 operand
+//    reads feed 32 products) when that grid fills the chip, else 128 x 128 (4 x 4 tiles, deeper
+//    ring);
+//  * with few rows and a narrow matrix even that grid is small: K is then split over
 //    blockIdx.z, the parts are written as float partial sums and a second kernel adds them in
-//    a fixed order.
+//    a fixed order;
+//  * optional SwiGLU epilogue over gate/up rows interleaved in fours.
+//
+// Measured on the 7B shapes at 2,048 rows: 0.73 to 0.88 PFLOP/s.  What bounds it is the delivery
+// of operand tiles into LDS (the same kernel without loads runs at 1.2 to 1.6 PFLOP/s).
 //
 // The reference's nearest kernel multiplies a 64 x 8 tile per 64-thread block without matrix
 // cores (crates/kernels-hip/src/kernels/mmq_f16_tile.cu:33-107).
 #include "common.h"
 #include "api.h"
 
-#define TG_BM 128
+#define TG_BM 128                        // block tile the split-K rule counts with
 #define TG_BN 128
-#define TG_BK 64
-#define TG_TILE 512                      // values in a 16 x 32 tile
 
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 template <typename TOut>
 __device__ __forceinline__ void tg_store4(TOut* p, f32x4 v);
@@ -36,102 +38,116 @@ template <> __device__ __forceinline__ void tg_store4<bf16_t>(bf16_t* p, f32x4 v
     *(bf16x4*)p = o;
 }
 
-// SWIGLU: w holds gate and up rows interleaved in fours; the block writes silu(gate) * up,
-// out_cols <= N / 2 values per token (never together with a split of K).
-template <typename TOut, bool SWIGLU>
-__global__ __launch_bounds__(256, 2) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
+// ---- the asynchronous variant: operand tiles go from memory straight into LDS
+// (global_load_lds_dwordx4: every lane gives its own global address, the 64 x 16 bytes of a wave
+// land side by side in LDS, which is exactly the tile layout), through a ring of NS stages of one
+// k-step (32 values of k) each.  No staging registers, no ds_write, one barrier per stage:
+//     wait for my loads of stage i; barrier; issue the loads of stage i + NS - 1 into the slot that
+//     stage i - 1 just left; read the operands of stage i from LDS; FT * TT products.
+// Nothing is zero-filled: rows beyond M and feature groups beyond N are clamped to valid ones (their
+// results are never stored), and k beyond K meets the zero padding of the packed w.
+template <int FT, int TT, int NS, int OCC, typename TOut, bool SWIGLU>
+__global__ __launch_bounds__(256, OCC) void gemm_async_kernel(const bf16_t* __restrict__ x,
                                                             const bf16_t* __restrict__ wp,
                                                             TOut* __restrict__ out, int M, int N, int K,
                                                             int n_steps, int steps_per_split, int out_cols) {
-    // [buffer][operand tile row (8)][k-step in slice (2)][512 values]
-    __shared__ __attribute__((aligned(16))) bf16_t xs[2][TG_BM / 16][2][TG_TILE];
-    __shared__ __attribute__((aligned(16))) bf16_t ws[2][TG_BN / 16][2][TG_TILE];
+    constexpr int NTF = 2 * FT, NTT = 2 * TT;         // operand tiles of the block: features, tokens
+    constexpr int TILES = NTF + NTT;                  // 1 KB tiles per stage
+    constexpr int LPS = TILES / 4;                    // load instructions per wave and stage
+    static_assert(TILES % 4 == 0, "tiles must divide among four waves");
+    extern __shared__ __attribute__((aligned(16))) bf16_t ring[];      // [NS][TILES][512]
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
-    const int wm = wave >> 1, wn = wave & 1;          // wave's place in the 2 x 2 arrangement
-    const int m0 = blockIdx.y * TG_BM, n0 = blockIdx.x * TG_BN;
-    const int n_groups = (N + 15) >> 4;               // row groups of the packed matrix
+    const int wf = wave & 1, wt = wave >> 1;
+    const int m0 = blockIdx.y * (NTT * 16), n0 = blockIdx.x * (NTF * 16);
+    const int n_groups = (N + 15) >> 4;
     const int s_begin = blockIdx.z * steps_per_split;
     const int s_end = min(n_steps, s_begin + steps_per_split);
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    const int n_iter = max(0, s_end - s_begin);
 
-    f32x4 acc[4][4];                                  // [feature tile][token tile]
+    f32x4 acc[FT][TT];
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < FT; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < TT; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // ---- what this thread fetches for one K slice (64 values of k = two steps)
-    // x: 128 rows x 8 chunks of 16 bytes; thread t takes chunks t, t+256, t+512, t+768
-    //    chunk c -> row c / 8, k-chunk c % 8 -> LDS tile (row / 16, kc / 4), lane 16 (kc % 4) + row % 16
-    // w: 8 row groups x 2 steps x 64 lanes of 16 bytes, copied as they lie
-    u32x4 xr[4], wr[4];
-    auto fetch = [&](int s) {
+    // per-lane source addresses of this wave's tiles at k-step 0 (tile t = wave + 4 u)
+    const bf16_t* src[LPS];
+    int kstride[LPS];                                 // values to advance per k-step
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int c = tid + 256 * u;
-            const int row = c >> 3, kc = c & 7;
-            const int gm = m0 + row;
-            const int k = s * 32 + kc * 8;
-            xr[u] = (gm < M && k + 8 <= K && s + (kc >> 2) < s_end) ? *(const u32x4*)(x + (size_t)gm * K + k) : zero4;
-            const int grp = c >> 7, st = (c >> 6) & 1, ln = c & 63;
-            const int gg = (n0 >> 4) + grp;
-            wr[u] = (gg < n_groups && s + st < s_end)
-                        ? *(const u32x4*)(wp + (((size_t)gg * n_steps + s + st) * 64 + ln) * 8) : zero4;
+    for (int u = 0; u < LPS; ++u) {
+        const int t = wave + 4 * u;
+        if (t < NTF) {
+            const int gg = min((n0 >> 4) + t, n_groups - 1);
+            src[u] = wp + (((size_t)gg * n_steps) * 64 + lane) * 8;
+            kstride[u] = 512;
+        } else {
+            const int row = min(m0 + (t - NTF) * 16 + (lane & 15), M - 1);
+            src[u] = x + (size_t)row * K + 8 * (lane >> 4);
+            kstride[u] = 32;
         }
-    };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int c = tid + 256 * u;
-            const int row = c >> 3, kc = c & 7;
-            *(u32x4*)&xs[buf][row >> 4][kc >> 2][(16 * (kc & 3) + (row & 15)) * 8] = xr[u];
-            const int grp = c >> 7, st = (c >> 6) & 1, ln = c & 63;
-            *(u32x4*)&ws[buf][grp][st][ln * 8] = wr[u];
-        }
-    };
-
-    int buf = 0;
-    if (s_begin < s_end) {
-        fetch(s_begin);
-        stash(0);
     }
-    __syncthreads();
-    for (int s = s_begin; s < s_end; s += 2) {
-        const bool more = s + 2 < s_end;
-        if (more) fetch(s + 2);
+    const int x_kmax = K - 8;                         // last whole 16-byte chunk of a row of x
+    auto issue = [&](int i) {                         // loads of stage i (k-step s_begin + i) into slot i % NS
+        const int s = s_begin + i;
+        bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
-            bf16x8 a[4], b[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                a[t] = *(const bf16x8*)&ws[buf][wn * 4 + t][st][lane * 8];
-                b[t] = *(const bf16x8*)&xs[buf][wm * 4 + t][st][lane * 8];
+        for (int u = 0; u < LPS; ++u) {
+            const int t = wave + 4 * u;
+            const bf16_t* g = src[u] + (size_t)s * kstride[u];
+            if (t >= NTF) {                           // x: keep the chunk inside the row
+                const int k = s * 32 + 8 * (lane >> 4);
+                if (k > x_kmax) g -= (k - x_kmax);
             }
-#pragma unroll
-            for (int ta = 0; ta < 4; ++ta)
-#pragma unroll
-                for (int tb = 0; tb < 4; ++tb)
-                    acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ta], b[tb], acc[ta][tb], 0, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                             (__attribute__((address_space(3))) void*)(slot + t * 512), 16, 0, 0);
         }
-        if (more) stash(buf ^ 1);
-        __syncthreads();
-        buf ^= 1;
-    }
+    };
 
-    // ---- store: lane (token j = lane % 16, g) holds rows 4 g .. 4 g + 3 of tile (ta, tb)
+#pragma unroll
+    for (int i = 0; i < NS - 1; ++i)
+        if (i < n_iter) issue(i);
+    for (int i = 0; i < n_iter; ++i) {
+        // my loads of stage i have landed when at most the later stages' are still in flight
+        if (i + NS - 2 < n_iter) {
+            __builtin_amdgcn_s_waitcnt(0xF70 | ((LPS * (NS - 2)) & 0xF) | ((((LPS * (NS - 2)) >> 4) & 3) << 14));
+        } else {
+            __builtin_amdgcn_s_waitcnt(0xF70);        // vmcnt(0)
+        }
+        // a bare barrier: __syncthreads() would add a fence that waits for ALL loads in flight,
+        // also those of the later stages, and the ring would be one stage deep
+        asm volatile("s_barrier" ::: "memory");
+        if (i + NS - 1 < n_iter) issue(i + NS - 1);
+        const bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
+        bf16x8 a[FT], b[TT];
+#pragma unroll
+        for (int t = 0; t < FT; ++t) a[t] = *(const bf16x8*)(slot + (wf * FT + t) * 512 + lane * 8);
+#pragma unroll
+        for (int t = 0; t < TT; ++t) b[t] = *(const bf16x8*)(slot + (NTF + wt * TT + t) * 512 + lane * 8);
+#pragma unroll
+        for (int ta = 0; ta < FT; ++ta)
+#pragma unroll
+            for (int tb = 0; tb < TT; ++tb)
+                acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ta], b[tb], acc[ta][tb], 0, 0, 0);
+        // all operand reads first, then the products (the scheduler would otherwise wait for LDS
+        // once per pair of feature tiles)
+        __builtin_amdgcn_sched_group_barrier(0x100, FT + TT, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, FT * TT, 0);
+    }
+    // the loads are done (the last stage waited for vmcnt(0)); LDS is not touched again
+
     const int j = lane & 15, g = lane >> 4;
     if (SWIGLU) {
 #pragma unroll
-        for (int tb = 0; tb < 4; ++tb) {
-            const int tok = m0 + (wm * 4 + tb) * 16 + j;
+        for (int tb = 0; tb < TT; ++tb) {
+            const int tok = m0 + (wt * TT + tb) * 16 + j;
 #pragma unroll
-            for (int ta = 0; ta < 4; ++ta) {
+            for (int ta = 0; ta < FT; ++ta) {
                 f32x4 up;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) up[r] = __shfl_down(acc[ta][tb][r], 16, 64);
-                const int f0 = (n0 >> 1) + (wn * 4 + ta) * 8 + 2 * g;
+                const int f0 = (n0 >> 1) + (wf * FT + ta) * 8 + 2 * g;
                 if ((g & 1) == 0 && tok < M && f0 < out_cols) {
                     f32x4 act;
 #pragma unroll
@@ -153,12 +169,12 @@ __global__ __launch_bounds__(256, 2) void gemm_tiled_kernel(const bf16_t* __rest
     TOut* obase = out + (size_t)blockIdx.z * M * N;
     const int vec_out = (N % 4 == 0) ? 1 : 0;
 #pragma unroll
-    for (int tb = 0; tb < 4; ++tb) {
-        const int tok = m0 + (wm * 4 + tb) * 16 + j;
+    for (int tb = 0; tb < TT; ++tb) {
+        const int tok = m0 + (wt * TT + tb) * 16 + j;
         if (tok >= M) continue;
 #pragma unroll
-        for (int ta = 0; ta < 4; ++ta) {
-            const int f0 = n0 + (wn * 4 + ta) * 16 + 4 * g;
+        for (int ta = 0; ta < FT; ++ta) {
+            const int f0 = n0 + (wf * FT + ta) * 16 + 4 * g;
             if (f0 >= N) continue;
             TOut* p = obase + (size_t)tok * N + f0;
             if (vec_out && f0 + 4 <= N) {
@@ -170,6 +186,20 @@ __global__ __launch_bounds__(256, 2) void gemm_tiled_kernel(const bf16_t* __rest
     }
 }
 
+template <int FT, int TT, int NS, int OCC, typename TOut, bool SWIGLU>
+static void launch_async(int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N,
+                         int K, int n_steps, int per, int out_cols) {
+    constexpr int LDS = NS * (2 * FT + 2 * TT) * 1024;
+    static bool configured = false;
+    auto kern = gemm_async_kernel<FT, TT, NS, OCC, TOut, SWIGLU>;
+    if (!configured) {
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        configured = true;
+    }
+    dim3 grid(ceil_div(N, 2 * FT * 16), ceil_div(M, 2 * TT * 16), splits);
+    kern<<<grid, 256, LDS, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols);
+}
+
 template <typename TOut>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part,
                                                                  TOut* __restrict__ out, size_t total,
@@ -179,6 +209,20 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     float s = part[i];
     for (int z = 1; z < splits; ++z) s += part[(size_t)z * total + i];
     out[i] = from_f32<TOut>(s);
+}
+
+// Shape of the block tile: 0 = chosen from the sizes, 1 = 128 x 128, 2 = 256 x 128 (for experiments).
+static int g_tiled_variant = 0;
+extern "C" int fl_gemm_tiled_set_variant(int v) { g_tiled_variant = v; return 0; }
+
+template <typename TOut, bool SWIGLU>
+static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out,
+                         int M, int N, int K, int n_steps, int per, int out_cols) {
+    if (variant == 0) variant = (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320) ? 2 : 1;
+    if (variant == 2)
+        launch_async<8, 4, 2, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols);
+    else
+        launch_async<4, 4, 4, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols);
 }
 
 // How many ways K is split for a product of this shape: 1 if the grid fills the chip.
@@ -207,18 +251,17 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
     const int n_steps = ceil_div(K, 32);
     const int splits = epilogue ? 1 : fl_gemm_tiled_splits(M, N, K);
     FL_CHECK(splits == 1 || workspace, "gemm_tiled: this shape splits K %d ways and needs a workspace", splits);
-    int per = ceil_div(n_steps, splits);
-    per += per & 1;                                    // whole slices of two steps
-    dim3 grid(ceil_div(N, TG_BN), ceil_div(M, TG_BM), splits);
+    const int per = ceil_div(n_steps, splits);
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
+    const int v = g_tiled_variant;
     if (epilogue) {
         if (out_dtype == FL_F32)
-            gemm_tiled_kernel<float, true><<<grid, 256, 0, stream>>>(xb, wb, (float*)out, M, N, K, n_steps, per, out_cols);
+            launch_tiled<float, true>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, out_cols);
         else
-            gemm_tiled_kernel<bf16_t, true><<<grid, 256, 0, stream>>>(xb, wb, (bf16_t*)out, M, N, K, n_steps, per, out_cols);
+            launch_tiled<bf16_t, true>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, out_cols);
     } else if (splits > 1) {
-        gemm_tiled_kernel<float, false><<<grid, 256, 0, stream>>>(xb, wb, workspace, M, N, K, n_steps, per, N);
+        launch_tiled<float, false>(v, splits, stream, xb, wb, workspace, M, N, K, n_steps, per, N);
         FL_LAUNCH_CHECK();
         const size_t total = (size_t)M * N;
         const unsigned rb = (unsigned)((total + 255) / 256);
@@ -227,9 +270,9 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
         else
             gemm_splitk_reduce_kernel<bf16_t><<<rb, 256, 0, stream>>>(workspace, (bf16_t*)out, total, splits);
     } else if (out_dtype == FL_F32) {
-        gemm_tiled_kernel<float, false><<<grid, 256, 0, stream>>>(xb, wb, (float*)out, M, N, K, n_steps, per, N);
+        launch_tiled<float, false>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, N);
     } else {
-        gemm_tiled_kernel<bf16_t, false><<<grid, 256, 0, stream>>>(xb, wb, (bf16_t*)out, M, N, K, n_steps, per, N);
+        launch_tiled<bf16_t, false>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, N);
     }
     FL_LAUNCH_CHECK();
     return 0;
