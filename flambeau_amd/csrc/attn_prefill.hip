@@ -5,8 +5,9 @@
 // one kv head, QT of the query heads that share it (QT = 4, 2 or 1, a divisor of the group size):
 // each wave holds QT query tiles and reuses every key/value operand it reads from LDS QT times.
 // Keys are walked in stages of 64 from the first key any of the block's queries may see to the
-// last; the next stage is fetched from the cache pages into registers while the current one is
-// multiplied, and put into the other LDS buffer.
+// last, through a ring of LDS stages filled straight from the cache pages
+// (global_load_lds_dwordx4: each lane names its own 16 bytes, the wave's kilobyte lands in tile
+// order), one bare barrier per stage.  The block's part of the block table sits in LDS.
 //
 // Everything is computed transposed, so that a query is a lane column:
 //   S^T[key][query] = K . Q^T        A = K tile (LDS, stored as matrix-core tiles), B = Q (registers)
@@ -24,23 +25,27 @@
 
 #define PF_TOKENS 64          // query tokens per block
 #define PF_STAGE 64           // keys per LDS stage
+#define PF_MAX_PAGES 4096     // block-table entries a block keeps in LDS
 
-typedef __attribute__((ext_vector_type(4))) unsigned int pf_u32x4;
-typedef __attribute__((ext_vector_type(2))) unsigned int pf_u32x2;
+// Which key sits in row i of the two 16-key score tiles of a 32-key chunk: tile a holds keys
+// 8 (i / 4) + i % 4, tile b the same + 4.  A lane (query, g) of the score accumulators then owns
+// the eight consecutive keys 8 g .. 8 g + 7 of the chunk (four from each tile), which is one
+// 16-byte run of a row of the transposed values: the value operand needs no gathering.
+__device__ __forceinline__ int pf_key_of_row(int i, int ab) { return 8 * (i >> 2) + 4 * ab + (i & 3); }
 
-template <int HDP, int QT, int NBUF>
+template <int HDP, int QT, int NS>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, PagedCache cache,
     const int* __restrict__ tiles, const int* __restrict__ positions,
-    const int* __restrict__ block_table, int max_blocks, int nh, float scale_log2e, int window) {
+    const int* __restrict__ block_table, int max_blocks, int nh, float scale_log2e, int window,
+    int log2_ps) {
     constexpr int QS = HDP / 32;              // k-steps of the score product
     constexpr int DT = HDP / 16;              // tiles of head dims in the output
-    constexpr int KCH = PF_STAGE * HDP / 8;   // 16-byte chunks of a K stage
-    constexpr int VPC = PF_STAGE * HDP / 4;   // 8-byte pieces of a V stage
-    constexpr int KPT = KCH / 256, VPT = VPC / 256;
-    // K stage: [key tile (4)][k-step (QS)][512]; V stage: [32-key chunk (2)][dim tile (DT)][512]
-    __shared__ __attribute__((aligned(16))) bf16_t ks[NBUF][PF_STAGE / 16][QS][512];
-    __shared__ __attribute__((aligned(16))) bf16_t vs[NBUF][PF_STAGE / 32][DT][512];
+    constexpr int KT = 4 * QS;                // 1 KB tiles of a K stage: [chunk (2)][a/b (2)][k-step]
+    constexpr int VT = 2 * DT;                // of a V stage: [chunk (2)][dim tile]
+    constexpr int LPW = (KT + VT) / 4;        // tile loads per wave and stage
+    extern __shared__ __attribute__((aligned(16))) bf16_t ring[];       // [NS][KT + VT][512]
+    __shared__ int s_pages[PF_MAX_PAGES];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int j = lane & 15, g = lane >> 4;
@@ -48,21 +53,31 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const int G = nh / cache.n_kv_heads;
     const int hgroups = G / QT;
     const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
-    const int seq = tiles[3 * blockIdx.x], row0 = tiles[3 * blockIdx.x + 1], cnt = tiles[3 * blockIdx.x + 2];
+    // tiles late in a prompt have the most keys: they are started first
+    const int tile = gridDim.x - 1 - blockIdx.x;
+    const int seq = tiles[3 * tile], row0 = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
     const int* table = block_table + (size_t)seq * max_blocks;
     const bf16_t* kv = (const bf16_t*)cache.base;
 
     const int p_first = positions[row0], p_last = p_first + cnt - 1;
     const int lo = window > 0 ? max(0, p_first - window + 1) : 0;     // first key anyone here sees
-    // this lane's query
     const int qtok = 16 * wave + j;
     const bool q_ok = qtok < cnt;
     const int p = q_ok ? p_first + qtok : -1;
     const int my_lo = window > 0 ? max(0, p - window + 1) : 0;
-    // this wave's span of positions (wave-uniform)
     const bool wave_on = 16 * wave < cnt;
     const int wp_first = p_first + 16 * wave, wp_last = min(p_last, wp_first + 15);
     const int w_lo = window > 0 ? max(0, wp_first - window + 1) : 0;
+
+    // ---- the pages of the keys [lo, p_last] go to LDS; a missing page (a hole below a window,
+    // or beyond the request) is replaced by the page of the last key: what is read from it is
+    // finite and never used (such keys are masked)
+    const int page0 = lo >> log2_ps, n_pg = (p_last >> log2_ps) - page0 + 1;
+    const int safe_page = table[p_last >> log2_ps];
+    for (int i = tid; i < n_pg; i += 256) {
+        const int pg = table[page0 + i];
+        s_pages[i] = (pg >= 0 && pg < cache.n_pages) ? pg : safe_page;
+    }
 
     // ---- Q as B operand, QT tiles: lane (query j, g) holds Q[token][head][32 s + 8 g ..]
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -86,65 +101,67 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         for (int d = 0; d < DT; ++d) o[t][d] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
 
-    // ---- staging of one 64-key stage
-    pf_u32x4 kr[KPT];
-    pf_u32x2 vr[VPT];
-    const int PP = ps < PF_STAGE ? ps : PF_STAGE;        // keys of a page that lie in one stage
-    const int v_per_part = HDP * (PP / 4);               // 8-byte pieces of one page part
-    auto fetch = [&](int t0) {
+    // ---- what this wave loads per stage: tiles tl = wave + 4 u of [K tiles | V tiles]; per lane the
+    // key offset inside the stage and the offset inside the (page, head) block are fixed
+    int key_off[LPW], blk_off[LPW];
+    const size_t head_k = (size_t)kvh * ps * hd, head_v = ((size_t)cache.n_kv_heads + kvh) * ps * hd;
+    const size_t page_stride = (size_t)2 * cache.n_kv_heads * ps * hd;
 #pragma unroll
-        for (int u = 0; u < KPT; ++u) {
-            const int c = tid + 256 * u;
-            const int kk = c / (HDP / 8), dc = c % (HDP / 8);
-            const int t = t0 + kk;
-            int page = (t >= lo && t <= p_last) ? table[t / ps] : -1;
-            if (page >= cache.n_pages) page = -1;
-            kr[u] = (page >= 0 && dc * 8 + 8 <= hd)
-                        ? *(const pf_u32x4*)(kv + cache_k_offset(cache, page, kvh, t % ps, dc * 8))
-                        : (pf_u32x4){0u, 0u, 0u, 0u};
+    for (int u = 0; u < LPW; ++u) {
+        const int tl = wave + 4 * u;
+        if (tl < KT) {                                         // K tile: chunk, a/b, k-step
+            const int c2 = tl / (2 * QS), ab = (tl / QS) & 1, s = tl % QS;
+            key_off[u] = 32 * c2 + pf_key_of_row(j, ab);
+            int d = 32 * s + 8 * g;
+            if (d + 8 > hd) d = 0;                             // padding dims: any finite data (Q is zero there)
+            blk_off[u] = d;                                    // + row * hd, row known per stage
+        } else {                                               // V tile: chunk, dim tile
+            const int tv = tl - KT;
+            const int c2 = tv / DT, dt = tv % DT;
+            key_off[u] = 32 * c2 + 8 * g;
+            int d = 16 * dt + j;
+            if (d >= hd) d = 0;                                // padding dims are never stored
+            blk_off[u] = d * ps;                               // + row
         }
+    }
+    const int n_stage = (p_last / PF_STAGE) - (lo / PF_STAGE) + 1;
+    const int t_base = (lo / PF_STAGE) * PF_STAGE;
+    auto issue = [&](int i) {
+        const int t0 = t_base + i * PF_STAGE;
+        bf16_t* slot = ring + (size_t)(i % NS) * (KT + VT) * 512;
 #pragma unroll
-        for (int u = 0; u < VPT; ++u) {
-            const int c = tid + 256 * u;
-            const int part = c / v_per_part, rem = c % v_per_part;
-            const int d = rem / (PP / 4), r4 = rem % (PP / 4);
-            const int t = t0 + part * PP + 4 * r4;
-            int page = (t + 3 >= lo && t <= p_last) ? table[t / ps] : -1;
-            if (page >= cache.n_pages) page = -1;
-            vr[u] = (page >= 0 && d < hd) ? *(const pf_u32x2*)(kv + cache_v_offset(cache, page, kvh, t % ps, d))
-                                           : (pf_u32x2){0u, 0u};
-        }
-    };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int u = 0; u < KPT; ++u) {
-            const int c = tid + 256 * u;
-            const int kk = c / (HDP / 8), dc = c % (HDP / 8);
-            *(pf_u32x4*)&ks[buf][kk >> 4][dc >> 2][(16 * (dc & 3) + (kk & 15)) * 8] = kr[u];
-        }
-#pragma unroll
-        for (int u = 0; u < VPT; ++u) {
-            const int c = tid + 256 * u;
-            const int part = c / v_per_part, rem = c % v_per_part;
-            const int d = rem / (PP / 4), r4 = rem % (PP / 4);
-            const int q4 = (part * PP) / 4 + r4;          // group of 4 keys within the stage, 0..15
-            // 32-key chunk q4 / 8; within it tile a/b = (q4 / 4) % 2, lane group g = q4 % 4
-            *(pf_u32x2*)&vs[buf][q4 >> 3][d >> 4][(16 * (q4 & 3) + (d & 15)) * 8 + 4 * ((q4 >> 2) & 1)] = vr[u];
+        for (int u = 0; u < LPW; ++u) {
+            const int tl = wave + 4 * u;
+            // keys outside [lo, p_last] are masked: read any valid one instead.  A value piece is a run
+            // of 8 keys and keeps its place if any of its keys is needed (its page is alive then)
+            int t = t0 + key_off[u];
+            if (tl < KT) t = min(max(t, lo), p_last);
+            else if (t + 7 < lo || t > p_last) t = p_last & ~7;
+            const int page = s_pages[(t >> log2_ps) - page0];
+            const int row = t & (ps - 1);
+            const bf16_t* src = kv + (size_t)page * page_stride +
+                                (tl < KT ? head_k + (size_t)row * hd + blk_off[u] : head_v + blk_off[u] + row);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)(slot + tl * 512), 16, 0, 0);
         }
     };
+    __syncthreads();                                            // s_pages is complete
+#pragma unroll
+    for (int i = 0; i < NS - 1; ++i)
+        if (i < n_stage) issue(i);
 
-    const int st_first = lo / PF_STAGE, st_last = p_last / PF_STAGE;
-    int buf = 0;
-    fetch(st_first * PF_STAGE);
-    stash(0);
-    __syncthreads();
-    for (int st = st_first; st <= st_last; ++st) {
-        const bool more = st < st_last;
-        if (more) fetch((st + 1) * PF_STAGE);
-        if (NBUF == 1) __syncthreads();       // (single buffer: computed below before it is overwritten)
+    for (int i = 0; i < n_stage; ++i) {
+        if (i + NS - 2 < n_stage) {
+            __builtin_amdgcn_s_waitcnt(0xF70 | ((LPW * (NS - 2)) & 0xF) | ((((LPW * (NS - 2)) >> 4) & 3) << 14));
+        } else {
+            __builtin_amdgcn_s_waitcnt(0xF70);
+        }
+        asm volatile("s_barrier" ::: "memory");
+        if (i + NS - 1 < n_stage) issue(i + NS - 1);
+        const bf16_t* slot = ring + (size_t)(i % NS) * (KT + VT) * 512;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            const int t0 = st * PF_STAGE + 32 * half;
+            const int t0 = t_base + i * PF_STAGE + 32 * half;
             // wave-uniform: does any query of this wave see any key of this chunk?
             if (!wave_on || t0 > wp_last || t0 + 31 < w_lo) continue;
             const bool need_mask = (t0 + 31 > wp_first) || (t0 < (window > 0 ? max(0, wp_last - window + 1) : 0));
@@ -154,45 +171,43 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             for (int t = 0; t < QT; ++t) { sa[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; sb[t] = sa[t]; }
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
-                const bf16x8 ka = *(const bf16x8*)&ks[buf][2 * half][s][lane * 8];
-                const bf16x8 kb = *(const bf16x8*)&ks[buf][2 * half + 1][s][lane * 8];
+                const bf16x8 ka = *(const bf16x8*)(slot + ((2 * half) * QS + s) * 512 + lane * 8);
+                const bf16x8 kb = *(const bf16x8*)(slot + ((2 * half + 1) * QS + s) * 512 + lane * 8);
 #pragma unroll
                 for (int t = 0; t < QT; ++t) {
                     sa[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[t][s], sa[t], 0, 0, 0);
                     sb[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[t][s], sb[t], 0, 0, 0);
                 }
             }
-            // ---- softmax per query column; this lane holds keys t0 + 4 g + r (a) and + 16 (b)
+            // ---- softmax per query column; this lane holds keys t0 + 8 g + r (a) and + 4 + r (b)
             bf16x8 pmat[QT];
             bool moved = false;
             float corr[QT];
 #pragma unroll
             for (int t = 0; t < QT; ++t) {
+                // raw scores; the scale (with log2 e folded in) enters inside the exponent: one fma per value
                 float mx = -INFINITY;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float va = sa[t][r] * scale_log2e, vb = sb[t][r] * scale_log2e;
                     if (need_mask) {
-                        const int ka = t0 + 4 * g + r, kb = ka + 16;
-                        if (ka > p || ka < my_lo) va = -INFINITY;
-                        if (kb > p || kb < my_lo) vb = -INFINITY;
+                        const int ka = t0 + 8 * g + r, kb = ka + 4;
+                        if (ka > p || ka < my_lo) sa[t][r] = -INFINITY;
+                        if (kb > p || kb < my_lo) sb[t][r] = -INFINITY;
                     }
-                    sa[t][r] = va;
-                    sb[t][r] = vb;
-                    mx = fmaxf(mx, fmaxf(va, vb));
+                    mx = fmaxf(mx, fmaxf(sa[t][r], sb[t][r]));
                 }
                 mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m[t], mx);
+                const float m_new = fmaxf(m[t], mx);            // m holds raw (unscaled) maxima; scale > 0
                 // a column that has seen no key yet keeps m = -inf: use 0 as the base then
-                const float base = m_new == -INFINITY ? 0.f : m_new;
-                corr[t] = __builtin_amdgcn_exp2f(m[t] - base);        // exp2(-inf) = 0
+                const float base = m_new == -INFINITY ? 0.f : m_new * scale_log2e;
+                corr[t] = __builtin_amdgcn_exp2f(fmaf(m[t], scale_log2e, -base));      // exp2(-inf) = 0
                 if (m_new != m[t]) moved = true;
                 float ls = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float ea = __builtin_amdgcn_exp2f(sa[t][r] - base);
-                    const float eb = __builtin_amdgcn_exp2f(sb[t][r] - base);
+                    const float ea = __builtin_amdgcn_exp2f(fmaf(sa[t][r], scale_log2e, -base));
+                    const float eb = __builtin_amdgcn_exp2f(fmaf(sb[t][r], scale_log2e, -base));
                     ls += ea + eb;
                     pmat[t][r] = (bf16_t)ea;
                     pmat[t][4 + r] = (bf16_t)eb;
@@ -210,18 +225,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             // ---- O^T += V^T P^T
 #pragma unroll
             for (int d = 0; d < DT; ++d) {
-                const bf16x8 vt = *(const bf16x8*)&vs[buf][half][d][lane * 8];
+                const bf16x8 vt = *(const bf16x8*)(slot + (KT + half * DT + d) * 512 + lane * 8);
 #pragma unroll
                 for (int t = 0; t < QT; ++t)
                     o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pmat[t], o[t][d], 0, 0, 0);
             }
         }
-        if (more) {
-            if (NBUF == 1) __syncthreads();
-            stash(NBUF == 1 ? 0 : buf ^ 1);
-        }
-        __syncthreads();
-        if (NBUF == 2) buf ^= 1;
     }
 
     // ---- normalise and store: lane (query j, g) holds dims 16 d + 4 g + r
@@ -246,16 +255,30 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     }
 }
 
-template <int HDP, int NBUF>
+template <int HDP, int QT, int NS>
+static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
+                               const int* tiles, const int* positions, const int* block_table, int max_blocks,
+                               int nh, float scale_log2e, int window, int log2_ps) {
+    constexpr int LDS = NS * (4 * (HDP / 32) + 2 * (HDP / 16)) * 1024;
+    static bool configured = false;
+    auto kern = attn_prefill_kernel<HDP, QT, NS>;
+    if (!configured) {
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        configured = true;
+    }
+    kern<<<grid, 256, LDS, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
+}
+
+template <int HDP, int NS>
 static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                            const int* tiles, const int* positions, const int* block_table, int max_blocks, int nh,
-                           float scale_log2e, int window) {
+                           float scale_log2e, int window, int log2_ps) {
     if (qt == 4)
-        attn_prefill_kernel<HDP, 4, NBUF><<<grid, 256, 0, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window);
+        launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
     else if (qt == 2)
-        attn_prefill_kernel<HDP, 2, NBUF><<<grid, 256, 0, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window);
+        launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
     else
-        attn_prefill_kernel<HDP, 1, NBUF><<<grid, 256, 0, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window);
+        launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
 }
 
 extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int* tiles,
@@ -264,33 +287,37 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
                                float scale, int window, int qt_hint, hipStream_t stream) {
     FL_CHECK(n_tiles >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_prefill: bad head counts %d/%d", nh, nkv);
     FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "attn_prefill: head size %d must be a multiple of 8 up to 256", hd);
-    FL_CHECK(page_size >= 4 && (PF_STAGE % page_size == 0 || page_size % PF_STAGE == 0),
-             "attn_prefill: page size %d must divide %d or be a multiple of it", page_size, PF_STAGE);
+    FL_CHECK(page_size >= 8 && (page_size & (page_size - 1)) == 0,
+             "attn_prefill: page size %d must be a power of two, at least 8", page_size);
+    FL_CHECK(max_blocks <= PF_MAX_PAGES, "attn_prefill: %d pages per request, at most %d", max_blocks, PF_MAX_PAGES);
     FL_CHECK(window >= 0, "attn_prefill: negative window");
+    FL_CHECK(scale > 0.f, "attn_prefill: the score scale must be positive");
     if (n_tiles == 0) return 0;
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
     const int G = nh / nkv;
     const int hdp = ceil_div(hd, 32) * 32;
+    int log2_ps = 0;
+    while ((1 << log2_ps) < page_size) ++log2_ps;
     // query heads per wave: a divisor of the group size, as many as the registers hold
     int qt = (G % 4 == 0) ? 4 : (G % 2 == 0 ? 2 : 1);
-    const int qt_max = hdp <= 128 ? 4 : (hdp <= 192 ? 2 : 1);
+    const int qt_max = hdp <= 128 ? 4 : 2;
     while (qt > qt_max) qt /= 2;
     if (qt_hint == 1 || qt_hint == 2 || qt_hint == 4)
         while (qt > qt_hint) qt /= 2;
     dim3 grid(n_tiles, nkv * (G / qt));
     const float sl = scale * 1.4426950408889634f;
-#define FL_PF(HDP_, NBUF_)                                                                                     \
-    launch_prefill<HDP_, NBUF_>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                                max_blocks, nh, sl, window)
+#define FL_PF(HDP_, NS_)                                                                                       \
+    launch_prefill<HDP_, NS_>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
+                              max_blocks, nh, sl, window, log2_ps)
     switch (hdp) {
-        case 32: FL_PF(32, 2); break;
-        case 64: FL_PF(64, 2); break;
-        case 96: FL_PF(96, 2); break;
-        case 128: FL_PF(128, 2); break;
-        case 160: FL_PF(160, 1); break;
-        case 192: FL_PF(192, 1); break;
-        case 224: FL_PF(224, 1); break;
-        default: FL_PF(256, 1); break;
+        case 32: FL_PF(32, 3); break;
+        case 64: FL_PF(64, 3); break;
+        case 96: FL_PF(96, 3); break;
+        case 128: FL_PF(128, 3); break;
+        case 160: FL_PF(160, 2); break;
+        case 192: FL_PF(192, 2); break;
+        case 224: FL_PF(224, 2); break;
+        default: FL_PF(256, 2); break;
     }
 #undef FL_PF
     FL_LAUNCH_CHECK();

@@ -187,9 +187,12 @@ def decode_supported(cache) -> bool:
         and cache.page_size % 4 == 0
 
 
-def prefill_supported(cache) -> bool:
+PREFILL_MAX_PAGES = 4096     # block-table entries per request the tiled kernel keeps in LDS
+
+
+def prefill_supported(cache, table) -> bool:
     ps = cache.page_size
-    return decode_supported(cache) and ps >= 4 and (64 % ps == 0 or ps % 64 == 0)
+    return decode_supported(cache) and ps >= 8 and ps & (ps - 1) == 0 and table.shape[1] <= PREFILL_MAX_PAGES
 
 
 def attention(rt, q, out, cache, step, table, n_heads, scale, window):
@@ -198,7 +201,7 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
     sends the whole batch to the plain kernel."""
     rows, tiles = step.extra.get("attn_rows"), step.extra.get("attn_tiles")
     batch = step.host
-    if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache)):
+    if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table)):
         return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
     if tiles.shape[0]:
         attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window)

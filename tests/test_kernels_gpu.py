@@ -421,7 +421,7 @@ def tiles_for(seqs, tile=64):
 
 @pytest.mark.parametrize("heads_per_wave", [0, 1])
 @pytest.mark.parametrize("nh,nkv,hd,ps,window", [(32, 8, 128, 16, 0), (4, 2, 16, 8, 16), (6, 1, 24, 16, 0),
-                                                (5, 5, 32, 16, 24), (8, 4, 64, 4, 0), (4, 2, 256, 32, 100),
+                                                (5, 5, 32, 16, 24), (8, 4, 64, 8, 0), (4, 2, 256, 32, 100),
                                                 (6, 3, 40, 64, 37), (2, 1, 160, 128, 0), (8, 2, 96, 16, 70)])
 def test_attn_prefill_against_plain_and_reference(nh, nkv, hd, ps, window, heads_per_wave):
     # (context, queries): a whole prompt, a portion deep in a context, one that starts mid-page,
@@ -442,6 +442,17 @@ def test_attn_prefill_against_plain_and_reference(nh, nkv, hd, ps, window, heads
     assert not torch.isnan(out).any()
     assert err.max() < 1e-2 * top, f"worst at {np.unravel_index(int(err.argmax()), err.shape)}"
     assert (out.double() - plain.double()).abs().max() < 1.5e-2 * top
+
+
+def test_attn_prefill_refuses_page_sizes_it_cannot_take():
+    from flambeau_amd.kernels import KernelError
+    for ps in (4, 12):
+        case = build_attention_case(torch.bfloat16, 2, 1, 16, ps, [(20, 20)], seed=1)
+        q2 = case["q"].reshape(20, 32)
+        with pytest.raises(KernelError, match="power of two"):
+            tuned().attn_prefill(q2, torch.empty_like(q2), case["cache"], tiles_for([(20, 20)]), case["pos_d"],
+                                 case["table"], 2, 0.25, 0)
+        assert not tuned().prefill_supported(case["cache"], case["table"])     # the engine takes the plain kernel
 
 
 def test_attn_prefill_peaked_scores_find_single_keys():
