@@ -106,7 +106,7 @@ def run_prefill(model, dtype_name, reps=3, seed=1):
         eng.add_request([int(t) for t in rng.integers(0, V, PROMPT_LEN)], SamplingParams(max_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        done = eng.step()
+        done = eng.step() + eng.flush()          # the first token has reached the host
         torch.cuda.synchronize()
         if rep:
             times.append(time.perf_counter() - t0)

@@ -31,6 +31,7 @@ int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
                   float scale, int window, hipStream_t stream);
 int fl_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n, int I,
                 hipStream_t stream);
+int fl_feed_tokens(int* tokens, const int* ids, const int* src, int n, hipStream_t stream);
 int fl_argmax(const float* logits, int* out, int rows, int V, hipStream_t stream);
 int fl_sample(const float* logits, const float* inv_temp, const float* uniform, int* out,
               int rows, int V, hipStream_t stream);

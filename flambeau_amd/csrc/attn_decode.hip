@@ -10,8 +10,9 @@
 //   per head (one lane column): running max and sum; scores and their exponentials never leave
 //   the lane that owns the column, so no broadcast is needed to rescale
 //   O^T[d][head]  += V^T[d][key] . P^T[key][head]   A = values, which the cache stores transposed
-//                                               inside a page (keys contiguous), B = P from the
-//                                               S^T accumulator without any data movement
+//                                               inside a page (keys contiguous: one 16-byte load
+//                                               per lane), B = P from the S^T accumulator without
+//                                               any data movement
 //
 // The four waves' states are merged through LDS; with more than one split the block writes a
 // partial (max, sum, O) and a second kernel merges the splits (same rule: exp(m_c - m_max)).
@@ -73,10 +74,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 
     for (int c = c0 + wave; c < c1; c += DEC_WAVES) {
         const int t0 = c * DEC_CHUNK;
-        // ---- scores of two 16-key tiles
+        // ---- scores of two 16-key tiles.  Row i of tile a is key t0 + 8 (i / 4) + i % 4, of tile b
+        // the same + 4: a lane (head, g) of the accumulators then owns the 8 consecutive keys
+        // t0 + 8 g .. + 7, one 16-byte run of a row of the transposed values
         f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
         {
-            const int ka = t0 + li, kb = t0 + 16 + li;
+            const int ka = t0 + 8 * (li >> 2) + (li & 3), kb = ka + 4;
             const int pa = (ka <= p && ka >= lo) ? table[ka / ps] : -1;
             const int pb = (kb <= p && kb >= lo) ? table[kb / ps] : -1;
             const bool oka = pa >= 0 && pa < cache.n_pages, okb = pb >= 0 && pb < cache.n_pages;
@@ -96,24 +99,21 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
                 sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[s], sb, 0, 0, 0);
             }
         }
-        // ---- values: lane (dim li of tile t, group g) reads keys 4g..4g+3 of either tile
-        const int va = t0 + 4 * g, vb = t0 + 16 + 4 * g;
-        const int pva = (va <= p) ? table[va / ps] : -1;
-        const int pvb = (vb <= p) ? table[vb / ps] : -1;
-        const bool okva = pva >= 0 && pva < cache.n_pages, okvb = pvb >= 0 && pvb < cache.n_pages;
-        bf16x4 wa[DT], wb[DT];
-        const bf16x4 zero4 = {0, 0, 0, 0};
+        // ---- values: lane (dim li of tile t, group g) reads the keys t0 + 8 g .. + 7 of its dim
+        const int vk = t0 + 8 * g;
+        const int pv = (vk <= p && vk + 7 >= lo) ? table[vk / ps] : -1;
+        const bool okv = pv >= 0 && pv < cache.n_pages;
+        bf16x8 wv[DT];
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
             const int d = 16 * t + li;
-            wa[t] = (okva && d < hd) ? *(const bf16x4*)(kv + cache_v_offset(cache, pva, kvh, va % ps, d)) : zero4;
-            wb[t] = (okvb && d < hd) ? *(const bf16x4*)(kv + cache_v_offset(cache, pvb, kvh, vb % ps, d)) : zero4;
+            wv[t] = (okv && d < hd) ? *(const bf16x8*)(kv + cache_v_offset(cache, pv, kvh, vk % ps, d)) : zero8;
         }
-        // ---- online softmax; this lane holds keys 4g + r of both tiles for head li
+        // ---- online softmax; this lane holds keys t0 + 8 g + r (tile a) and + 4 + r (tile b) for head li
         float mt = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int ka = t0 + 4 * g + r, kb = ka + 16;
+            const int ka = t0 + 8 * g + r, kb = ka + 4;
             sa[r] = (ka >= lo && ka <= p) ? sa[r] * scale : -INFINITY;
             sb[r] = (kb >= lo && kb <= p) ? sb[r] * scale : -INFINITY;
             mt = fmaxf(mt, fmaxf(sa[r], sb[r]));
@@ -135,11 +135,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         m = m_new;
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
-            bf16x8 v8;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) { v8[r] = wa[t][r]; v8[4 + r] = wb[t][r]; }
             o[t] *= corr;
-            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v8, pb8, o[t], 0, 0, 0);
+            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[t], pb8, o[t], 0, 0, 0);
         }
     }
     // sum over the four key groups of a head
@@ -260,7 +257,7 @@ extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* pa
                               float scale, int window, int n_split, hipStream_t stream) {
     FL_CHECK(n_items >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_decode: bad head counts %d/%d", nh, nkv);
     FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "attn_decode: head size %d must be a multiple of 8 up to 256", hd);
-    FL_CHECK(page_size % 4 == 0, "attn_decode: page size %d must be a multiple of 4", page_size);
+    FL_CHECK(page_size % 8 == 0, "attn_decode: page size %d must be a multiple of 8", page_size);
     FL_CHECK(n_split >= 1 && n_split <= 256, "attn_decode: %d splits", n_split);
     FL_CHECK(n_split == 1 || (part_o && part_ml), "attn_decode: splits need a workspace");
     FL_CHECK(window >= 0, "attn_decode: negative window");

@@ -549,6 +549,22 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
     }
 }
 
+// Token ids that are still on the device: tokens[i] = ids[src[i]] where src[i] >= 0 (the token a
+// request drew in the step before, fed back without a round trip through the host).
+__global__ __launch_bounds__(256) void feed_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ ids,
+                                                          const int* __restrict__ src, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n && src[i] >= 0) tokens[i] = ids[src[i]];
+}
+
+extern "C" int fl_feed_tokens(int* tokens, const int* ids, const int* src, int n, hipStream_t stream) {
+    FL_CHECK(n >= 0, "feed_tokens: bad size");
+    if (n == 0) return 0;
+    feed_tokens_kernel<<<ceil_div(n, 256), 256, 0, stream>>>(tokens, ids, src, n);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" int fl_argmax(const float* logits, int* out, int rows, int V, hipStream_t stream) {
     FL_CHECK(rows >= 0 && V > 0, "argmax: bad sizes");
     if (rows == 0) return 0;

@@ -53,6 +53,10 @@ class LLMEngine:
                                    max_queue_depth=opt.max_queue_depth, eos_token_id=spec.eos_token_id,
                                    default_seed=opt.seed)
         self.sampler = DeviceSampler(model.rt.device, max(opt.inflight_slots, 1))
+        # tokens drawn on the device are fed to the next step on the device: the host enqueues
+        # step i + 1 while step i runs and reads step i's tokens afterwards
+        self.runner.token_feedback = self.sampler.ids
+        self._in_flight = None            # (scheduled, sampler handle) of the step the host has not read yet
         self._next_id = 0
 
     @classmethod
@@ -81,29 +85,59 @@ class LLMEngine:
         return self.scheduler.abort(request_id)
 
     # ------------------------------------------------------------ one step
-    def step(self) -> list[Request]:
-        """Schedule, run, sample, commit.  Returns the requests that finished in this step."""
-        sched = self.scheduler.schedule()
-        if not sched:
+    def flush(self) -> list[Request]:
+        """Read the tokens of the step in flight, if any.  Returns the requests that finished."""
+        if self._in_flight is None:
             return []
-        entries = [StepEntry(s.request.request_id, s.tokens, [len(s.tokens) - 1] if s.sample else [])
-                   for s in sched]
-        logits = self.runner.step(entries)
-        sampled = {}
+        sched, handle = self._in_flight
+        self._in_flight = None
+        ids = self.sampler.collect(handle)
         rows = [s for s in sched if s.sample]
-        if rows:
-            on_device = self.options.gpu_sampler and all(s.request.params.device_ok for s in rows)
-            if on_device:
-                inv_t = [0.0 if s.request.params.is_greedy else 1.0 / s.request.params.temperature for s in rows]
-                us = [0.0 if s.request.params.is_greedy else s.request.rng.next_f32() for s in rows]
-                ids = self.sampler.sample(logits, inv_t, us)
+        return self.scheduler.resolve(sched, {s.request.request_id: t for s, t in zip(rows, ids)})
+
+    def step(self) -> list[Request]:
+        """Schedule, enqueue, draw, and read the tokens of the step BEFORE this one: the device is
+        always one step ahead of what the host has seen.  Returns the requests that finished."""
+        from .scheduler import PENDING
+        sched = self.scheduler.schedule()
+        finished = []
+        if any(PENDING in s.tokens and len(s.tokens) > 1 for s in sched):
+            # a re-admitted request would feed a token the host has not seen inside a portion
+            finished += self.flush()
+            sched = self.scheduler.schedule()
+        if not sched:
+            return finished + self.flush()
+        entries = []
+        for s in sched:
+            r = s.request
+            want = [len(s.tokens) - 1] if s.sample else []
+            if s.tokens[-1] == PENDING:
+                entries.append(StepEntry(r.request_id, [0], want, from_device=r.pending_row))
             else:
-                host = logits.to("cpu").numpy()
-                ids = [sample_host(host[i], s.request.params, s.request.output, s.request.rng)
-                       for i, s in enumerate(rows)]
-            for s, tok in zip(rows, ids):
-                sampled[s.request.request_id] = tok
-        return self.scheduler.commit(sched, sampled)
+                entries.append(StepEntry(r.request_id, s.tokens, want))
+        rows = [s for s in sched if s.sample]
+        on_device = self.options.gpu_sampler and all(s.request.params.device_ok for s in rows)
+        logits = self.runner.step(entries)
+        if on_device:
+            inv_t = [0.0 if s.request.params.is_greedy else 1.0 / s.request.params.temperature for s in rows]
+            us = [0.0 if s.request.params.is_greedy else s.request.rng.next_f32() for s in rows]
+            if rows:
+                handle = self.sampler.sample_async(logits, inv_t, us)
+            else:
+                handle = (0, 0)
+            self.scheduler.advance(sched)
+            finished += self.flush()                  # the step before; this one is running meanwhile
+            self._in_flight = (sched, handle) if rows else None
+            return finished
+        # penalties, bias or filters: the logits go to the host sampler, nothing stays in flight
+        finished += self.flush()
+        host = logits.to("cpu").numpy() if rows else None
+        sampled = {}
+        for i, s in enumerate(rows):
+            r = s.request
+            if r.status != "finished":            # (a stop token of the step before may just have ended it)
+                sampled[r.request_id] = sample_host(host[i], r.params, r.output, r.rng)
+        return finished + self.scheduler.commit(sched, sampled)
 
     # ------------------------------------------------------------ whole generations
     def generate(self, prompts, params=None) -> list:
@@ -116,6 +150,7 @@ class LLMEngine:
         reqs = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
         while self.has_work():
             self.step()
+        self.flush()
         return [list(r.output) for r in reqs]
 
 

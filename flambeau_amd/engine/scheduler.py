@@ -38,6 +38,9 @@ class AdmissionError(RuntimeError):
     """A request that is refused when it is added."""
 
 
+PENDING = -1     # a token that was drawn on the device and that the host has not seen yet
+
+
 @dataclass
 class Request:
     request_id: object
@@ -50,6 +53,8 @@ class Request:
     n_preempted: int = 0
     rng: Xoshiro256 | None = None
     arrival: int = 0
+    pending_row: int | None = None      # where the PENDING token lies in the sampler's output buffer
+    reported: bool = False
 
     @property
     def tokens(self) -> list:
@@ -241,23 +246,61 @@ class Scheduler:
     def commit(self, scheduled: list, sampled: dict) -> list[Request]:
         """``sampled``: request id -> token drawn after its portion (for entries with
         ``sample``).  Returns the requests that finished; their pages and slots are free."""
-        finished = []
+        self.advance(scheduled)
+        return self.resolve(scheduled, sampled)
+
+    # The commit in two halves, for an engine that enqueues the next step before it has seen the
+    # tokens of this one: ``advance`` right after the step is enqueued (what does not depend on
+    # the tokens' values), ``resolve`` when the values have arrived.
+    def advance(self, scheduled: list) -> None:
+        row = -1
         for s in scheduled:
             r = s.request
+            if s.sample:
+                row += 1
+            if r.status == "finished":
+                continue                         # a stop token ended it while this step was enqueued
             r.n_computed += len(s.tokens)
             if not s.sample:
                 continue
-            tok = int(sampled[r.request_id])
-            r.output.append(tok)
-            stop = (not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id) \
-                or tok in r.params.stop_token_ids
-            if stop:
-                r.finish_reason = "stop"
-            elif len(r.output) >= r.params.max_tokens or len(r.prompt) + len(r.output) >= self.manager.max_seq_len:
+            r.output.append(PENDING)
+            r.pending_row = row
+            if len(r.output) >= r.params.max_tokens or len(r.prompt) + len(r.output) >= self.manager.max_seq_len:
+                # the length ends it whatever the token is; pages are free for steps enqueued later
                 r.finish_reason = "length"
-            if r.finish_reason:
                 r.status = "finished"
                 self.running.remove(r)
                 self.manager.release(r.request_id)
+
+    def resolve(self, scheduled: list, sampled: dict) -> list[Request]:
+        """Fill in the drawn tokens; a stop token ends its request (a step that was enqueued for it
+        meanwhile is wasted: its token is dropped)."""
+        finished = []
+        for s in scheduled:
+            if not s.sample:
+                continue
+            r = s.request
+            if PENDING not in r.output:
+                continue                         # stopped earlier: this was a step beyond its end
+            at = r.output.index(PENDING)
+            tok = int(sampled[r.request_id])
+            r.output[at] = tok
+            if r.pending_row is not None and PENDING not in r.output:
+                r.pending_row = None
+            stop = (not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id) \
+                or tok in r.params.stop_token_ids
+            if stop:
+                del r.output[at + 1:]
+                r.pending_row = None
+                r.finish_reason = "stop"
+                if r.status != "finished":
+                    r.status = "finished"
+                    if r in self.running:
+                        self.running.remove(r)
+                        self.manager.release(r.request_id)
+                    elif r in self.waiting:
+                        self.waiting.remove(r)
+            if r.status == "finished" and PENDING not in r.output and not r.reported:
+                r.reported = True
                 finished.append(r)
         return finished

@@ -21,6 +21,7 @@ import torch
 
 from ..cache.manager import CacheError, CacheManager
 from ..cache.storage import CacheStorage
+from ..kernels import ops
 from ..parts.base import HostBatch, StepState
 
 
@@ -29,6 +30,8 @@ class StepEntry:
     request_id: object
     tokens: list
     want: list = field(default_factory=list)   # places among ``tokens`` whose logits are wanted
+    from_device: int | None = None            # a single token that is still on the device: its row in
+                                              # the runner's ``token_feedback`` buffer (``tokens`` is ignored)
 
 
 class StepError(ValueError):
@@ -58,6 +61,10 @@ class ModelRunner:
         self.decode_graphs = bool(decode_graphs) and all(getattr(c, "graph_safe", False) for c in self._mixer_classes)
         self.max_graph_batch = min(max_graph_batch, max_slots)
         self._graphs: dict[int, "_GraphedStep"] = {}
+        # ids drawn on the device in the step before (the sampler's output buffer); entries with
+        # ``from_device`` read their token from it, so a step can be enqueued before the host has
+        # seen the step before
+        self.token_feedback = None
 
     # ------------------------------------------------------------ requests
     def begin(self, request_id) -> bool:
@@ -102,6 +109,10 @@ class ModelRunner:
             raise StepError(f"logits wanted at {n_rows} places, at most {self.max_logit_rows} per step")
         V = self.model.spec.vocab_size
         for e in entries:
+            if e.from_device is not None:
+                if len(e.tokens) != 1 or self.token_feedback is None or not 0 <= e.from_device < self.token_feedback.shape[0]:
+                    raise StepError(f"request {e.request_id!r}: a token from the device needs one place and a feedback buffer")
+                continue
             if min(e.tokens) < 0 or max(e.tokens) >= V:
                 bad = next(t for t in e.tokens if not 0 <= t < V)
                 raise StepError(f"token id {bad} is outside the vocabulary of {V}")
@@ -120,13 +131,17 @@ class ModelRunner:
         tokens = np.zeros(n + n_pad, dtype=np.int32)
         positions = np.zeros(n + n_pad, dtype=np.int32)
         tok_seq = np.empty(n + n_pad, dtype=np.int32)
+        token_src = np.full(n + n_pad, -1, dtype=np.int32)
         q_starts, q_lens, starts, slots, rows = [], [], [], [], []
         at = 0
         for s, e in enumerate(entries):
             rc = mgr.live[e.request_id]
             k = len(e.tokens)
             mgr.ensure(e.request_id, rc.n_cached + k)
-            tokens[at:at + k] = e.tokens
+            if e.from_device is not None:
+                token_src[at] = e.from_device
+            else:
+                tokens[at:at + k] = e.tokens
             positions[at:at + k] = np.arange(rc.n_cached, rc.n_cached + k, dtype=np.int32)
             tok_seq[at:at + k] = s
             q_starts.append(at)
@@ -158,7 +173,7 @@ class ModelRunner:
                 row = mgr.table_row(e.request_id, g)
                 t[s, :len(row)] = row
             tables.append(t)
-        parts = [("tokens", tokens), ("positions", positions), ("tok_seq", tok_seq),
+        parts = [("tokens", tokens), ("token_src", token_src), ("positions", positions), ("tok_seq", tok_seq),
                  ("seq_slots", np.asarray(slots, dtype=np.int32)),
                  ("seq_q_start", np.asarray(q_starts, dtype=np.int32)),
                  ("seq_q_len", np.asarray(q_lens, dtype=np.int32)),
@@ -169,6 +184,11 @@ class ModelRunner:
             for name, arr in cls.step_metadata(batch).items():
                 parts.append(("extra:" + name, np.ascontiguousarray(arr, dtype=np.int32)))
         return batch, parts
+
+    def _feed(self, dev, needed: bool) -> None:
+        """Fill in the tokens that are still on the device."""
+        if needed:
+            ops.feed_tokens(dev["tokens"], self.token_feedback, dev["token_src"])
 
     def _state_from(self, batch, parts, dev) -> StepState:
         extra = {name[6:]: dev[name] for name, _ in parts if name.startswith("extra:")}
@@ -235,7 +255,9 @@ class ModelRunner:
             logits = self._step_graphed(entries)
         else:
             batch, parts = self._assemble(entries)
-            step = self._state_from(batch, parts, self._upload(parts))
+            dev = self._upload(parts)
+            self._feed(dev, any(e.from_device is not None for e in entries))
+            step = self._state_from(batch, parts, dev)
             logits = self.model.forward(step, self.storage.entries, self.max_logit_rows)
         for e in entries:
             self.manager.advance(e.request_id, len(e.tokens))
@@ -260,15 +282,21 @@ class ModelRunner:
             gs = _GraphedStep(torch.empty(max(total, 1), dtype=torch.int32, device=self.rt.device))
             self._graphs[bk] = gs
         dev = self._upload(parts, gs.meta)
+        feedback = self.token_feedback is not None
         if gs.graph is None:
             step = self._state_from(batch, parts, dev)
             with self.rt.scope(f"graph{bk}"):
+                self._feed(dev, feedback)
                 self.model.forward(step, self.storage.entries, bk)          # makes the buffers
                 torch.cuda.current_stream().synchronize()
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
+                    self._feed(dev, feedback)          # part of the graph: a no-op when no token comes from the device
                     gs.logits = self.model.forward(step, self.storage.entries, bk)
             gs.graph = graph
+            gs.feedback = feedback
+        elif gs.feedback != feedback:
+            raise StepError("the token feedback buffer must be set before the first captured step")
         gs.graph.replay()
         wanted = [i for i, e in enumerate(entries) if e.want]
         if not wanted:
@@ -283,3 +311,4 @@ class _GraphedStep:
         self.meta = meta
         self.graph = None
         self.logits = None
+        self.feedback = False

@@ -23,6 +23,7 @@ _SIGNATURES = {
     "fl_rope_kv_write": [P, I, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, P],
     "fl_attn_plain": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
     "fl_silu_mul": [P, I, P, I, I, I, P],
+    "fl_feed_tokens": [P, P, P, I, P],
     "fl_argmax": [P, P, I, I, P],
     "fl_sample": [P, P, P, P, I, I, P],
 }

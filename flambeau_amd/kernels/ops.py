@@ -140,6 +140,14 @@ def silu_mul(gu, out):
     return out
 
 
+def feed_tokens(tokens, ids, src):
+    """``tokens[i] = ids[src[i]]`` where ``src[i] >= 0``: ids drawn on the device in the step before."""
+    n = tokens.shape[0]
+    call("fl_feed_tokens", _check(tokens, "feed.tokens", torch.int32, (n,)), _check(ids, "feed.ids", torch.int32),
+         _check(src, "feed.src", torch.int32, (n,)), n, stream_handle())
+    return tokens
+
+
 def argmax(logits, out):
     R, V = logits.shape
     call("fl_argmax", _check(logits, "argmax.logits", torch.float32), _check(out, "argmax.out", torch.int32, (R,)),

@@ -117,7 +117,7 @@ def prepare_gate_up(gate: torch.Tensor, up: torch.Tensor) -> Weight:
 # longer portions go to the tiled prefill kernel.
 SHORT_PORTION = 8
 DECODE_TARGET_BLOCKS = 1024
-DECODE_MIN_KEYS_PER_SPLIT = 128
+DECODE_MIN_KEYS_PER_SPLIT = 256
 
 
 PREFILL_TILE = 64        # query tokens per block of the tiled kernel
@@ -184,7 +184,7 @@ def attn_prefill(q, out, cache, tiles, positions, table, n_heads, scale, window,
 
 def decode_supported(cache) -> bool:
     return cache.pool.dtype == torch.bfloat16 and cache.head_dim % 8 == 0 and cache.head_dim <= 256 \
-        and cache.page_size % 4 == 0
+        and cache.page_size % 8 == 0
 
 
 PREFILL_MAX_PAGES = 4096     # block-table entries per request the tiled kernel keeps in LDS

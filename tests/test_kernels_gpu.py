@@ -334,7 +334,7 @@ def test_sample_is_the_inverse_cdf_in_index_order(V):
 # ---------------------------------------------------------------- tuned attention for single rows
 @pytest.mark.parametrize("n_split", [1, 2, 5])
 @pytest.mark.parametrize("nh,nkv,hd,ps,window", [(32, 8, 128, 16, 0), (4, 2, 16, 8, 16), (6, 1, 24, 16, 0),
-                                                (5, 5, 32, 16, 24), (20, 1, 64, 4, 0), (8, 4, 256, 32, 100),
+                                                (5, 5, 32, 16, 24), (20, 1, 64, 8, 0), (8, 4, 256, 32, 100),
                                                 (3, 1, 40, 64, 0)])
 def test_attn_decode_against_plain_and_reference(nh, nkv, hd, ps, window, n_split):
     seqs = [(700, 1), (33, 1), (ps * 3, 1), (1, 1), (257, 3), (64, 2), (32, 1), (31, 1)]

@@ -208,3 +208,39 @@ def test_abort_gives_everything_back():
     while s.has_work():
         run_step(m, s)
     assert m.free_pages() == [16] and m.n_free_slots == 2
+
+
+def test_commit_in_two_halves_with_a_step_enqueued_in_between():
+    """The engine enqueues step i + 1 before it has seen the tokens of step i: ``advance`` counts a
+    token whose value is pending, ``resolve`` fills it in; a stop token found late ends the request
+    and the token of the wasted step is dropped."""
+    from flambeau_amd.engine.scheduler import PENDING
+    m, s = mk(eos_token_id=7)
+    a = s.add("a", [1, 2, 3], SamplingParams(max_tokens=4))
+    b = s.add("b", [4, 5], SamplingParams(max_tokens=10))
+
+    def enqueue():
+        sched = s.schedule()
+        for e in sched:
+            m.ensure(e.request.request_id, e.request.n_computed + len(e.tokens))
+            m.advance(e.request.request_id, len(e.tokens))
+        s.advance(sched)
+        return sched
+
+    s1 = enqueue()                                       # prompts; both draw
+    assert a.output == [PENDING] and b.output == [PENDING] and (a.pending_row, b.pending_row) == (0, 1)
+    s2 = enqueue()                                       # decode rows fed from the device
+    assert [e.tokens for e in s2] == [[PENDING], [PENDING]]
+    assert s.resolve(s1, {"a": 11, "b": 7}) == [b]       # b drew the stop token in step 1
+    assert b.output == [7] and b.finish_reason == "stop" and b not in s.running
+    assert a.output == [11, PENDING]
+    s3 = enqueue()                                       # only a is left
+    assert [e.request.request_id for e in s3] == ["a"]
+    assert s.resolve(s2, {"a": 12, "b": 99}) == []       # b's token of the wasted step is dropped
+    assert b.output == [7] and a.output == [11, 12, PENDING]
+    s4 = enqueue()                                       # a's fourth token: the length ends it at once
+    assert a.status == "finished" and a not in s.running and m.n_free_slots == 3
+    assert s.resolve(s3, {"a": 13}) == []                # not reported before its last token is known
+    assert s.resolve(s4, {"a": 14}) == [a] and a.output == [11, 12, 13, 14] and a.finish_reason == "length"
+    m.check_invariants()
+    assert m.free_pages() == [16]
