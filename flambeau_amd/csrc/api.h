@@ -42,6 +42,12 @@ int fl_sample(const float* logits, const float* inv_temp, const float* uniform, 
 int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
                    int nw_hint, int epilogue, int out_cols, hipStream_t stream);
 
+// 17 to 64 rows, K a multiple of 32; a shape with fl_gemm_mid_splits > 1 needs a float workspace
+// of splits * M * N values
+int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
+int fl_gemm_mid_splits(int M, int N, int K);
+
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_tiled_splits(int M, int N, int K);

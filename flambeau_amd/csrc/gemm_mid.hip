@@ -1,0 +1,285 @@
+// bf16 matrix product for 17 to 64 rows: out[m, n] = sum_k x[m, k] w[n, k], a decode batch of
+// that many requests.  Like the skinny kernel it is bound by the stream of w out of HBM, which a
+// wave reads tile by tile (1 KB of packed w per load instruction) straight into registers.  With
+// more than one tile of tokens the second operand becomes the problem: each 1 KB of w wants up
+// to 4 KB of x, and when every wave fetches those from the caches itself the loop waits for the
+// cache four times per iteration.  So here the eight waves of a block walk the SAME range of k,
+// each with a row group of its own, and share x through LDS:
+//
+//  * x is read in chunks of GM_CH k-steps; the waves of the block share the loads of a chunk
+//    (every lane reads the 16 bytes that the operand layout wants at its place, so that a tile
+//    is 1 KB in lane order in LDS too) and keep them in registers for one chunk's time before
+//    they write them into one of two LDS slots;
+//  * per chunk: issue the loads of x for the chunk after the next and of w for the next; read
+//    the operands of this chunk from its LDS slot, GM_CH * MT products; write the x registers of
+//    the next chunk into the other slot; one bare s_barrier.  All loads go to registers, so the
+//    compiler counts them and every wait lets the younger loads stay in flight;
+//  * K is split over blockIdx.y when the row groups alone do not fill the chip; the parts are
+//    float partial sums that a second kernel adds in a fixed order;
+//  * nothing is zero-filled: token rows beyond M are clamped to the last row (their columns are
+//    never stored), K is a multiple of 32 (other shapes stay with the skinny kernel), and k-steps
+//    beyond the matrix take a zero tile of w.
+//
+// The reference's nearest kernel is its batched float GEMV, one block per output row
+// (crates/kernels-hip/src/kernels/dense_gemv_f16_f16_batched.cu:17-63).
+#include "common.h"
+#include "api.h"
+
+
+template <typename TOut>
+__device__ __forceinline__ void gm_store4(TOut* p, f32x4 v);
+template <> __device__ __forceinline__ void gm_store4<float>(float* p, f32x4 v) { *(f32x4*)p = v; }
+template <> __device__ __forceinline__ void gm_store4<bf16_t>(bf16_t* p, f32x4 v) {
+    bf16x4 o = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+    *(bf16x4*)p = o;
+}
+
+// GM_NW waves (row groups) per block, GM_CH k-steps per chunk
+template <int MT, int GM_NW, int GM_CH, typename TOut, bool SWIGLU>
+__global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K,
+                                                              int n_steps, int chunks_per_split, int out_cols) {
+    constexpr int FR = GM_CH * MT;                    // 1 KB operand tiles of x per chunk
+    constexpr int XL = (FR + GM_NW - 1) / GM_NW;      // x loads per wave and chunk
+    __shared__ __attribute__((aligned(16))) bf16_t slots[2][FR * 512];
+
+    // wave-uniform values live in scalar registers, so that a load's address is a scalar base plus
+    // a per-lane offset that never changes: no vector arithmetic per load
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int li = lane & 15, g = lane >> 4;
+    const int n_groups = (N + 15) >> 4;
+    const int group = blockIdx.x * GM_NW + wave;
+    const int gg = min(group, n_groups - 1);          // waves beyond the matrix repeat the last group, store nothing
+    const bf16_t* wt = wp + (size_t)gg * n_steps * 512;
+    const unsigned w_lane = lane * 8;
+
+    const int n_chunks = (n_steps + GM_CH - 1) / GM_CH;
+    const int c_begin = blockIdx.y * chunks_per_split;
+    const int n_iter = max(0, min(n_chunks, c_begin + chunks_per_split) - c_begin);
+    if (n_iter == 0 && !(!SWIGLU && gridDim.y > 1)) return;       // an empty part still writes its zeros
+
+    // this wave's share of a chunk's x tiles: tile f = (k-step f / MT of the chunk, token tile f % MT)
+    unsigned x_lane[XL];
+    int xstep[XL], xdst[XL];
+#pragma unroll
+    for (int u = 0; u < XL; ++u) {
+        const int f = min(wave + GM_NW * u, FR - 1);  // a surplus load repeats the last tile
+        const int mt = f % MT;
+        xstep[u] = f / MT;
+        xdst[u] = f * 512 + lane * 8;
+        x_lane[u] = (unsigned)min(mt * 16 + li, M - 1) * (unsigned)K + 8 * g;
+    }
+    const int last = max(n_iter - 1, 0);
+    // chunks beyond the part are clamped to its last chunk and k-steps beyond the matrix to its last
+    // step: loads without branches, whose results nobody uses
+    auto load_x = [&](bf16x8 (&xr)[XL], int i) {
+        const int c = c_begin + min(i, last);
+#pragma unroll
+        for (int u = 0; u < XL; ++u) {
+            const bf16_t* base = x + (size_t)min(c * GM_CH + xstep[u], n_steps - 1) * 32;
+            xr[u] = *(const bf16x8*)(base + x_lane[u]);
+        }
+    };
+    auto store_x = [&](const bf16x8 (&xr)[XL], int slot) {
+#pragma unroll
+        for (int u = 0; u < XL; ++u) *(bf16x8*)(&slots[slot][xdst[u]]) = xr[u];
+    };
+    auto load_w = [&](bf16x8 (&a)[GM_CH], int i) {
+        const int c = c_begin + min(i, last);
+#pragma unroll
+        for (int j = 0; j < GM_CH; ++j) {
+            const bf16_t* base = wt + (size_t)min(c * GM_CH + j, n_steps - 1) * 512;
+            a[j] = __builtin_nontemporal_load((const bf16x8*)(base + w_lane));
+        }
+    };
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    bf16x8 a_even[GM_CH], a_odd[GM_CH], x_even[XL], x_odd[XL];
+    load_x(x_even, 0);
+    load_w(a_even, 0);
+    load_x(x_odd, 1);
+    store_x(x_even, 0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0): my part of the slot is written
+    asm volatile("s_barrier" ::: "memory");
+
+    // chunk i: a_cur holds its w, x_nxt the x of chunk i + 1; a_nxt and x_nn receive the loads of
+    // chunks i + 1 and i + 2 (the register sets swap roles from chunk to chunk, no copies)
+    auto chunk = [&](int i, bf16x8 (&a_cur)[GM_CH], bf16x8 (&a_nxt)[GM_CH], bf16x8 (&x_nxt)[XL], bf16x8 (&x_nn)[XL]) {
+        load_x(x_nn, i + 2);
+        load_w(a_nxt, i + 1);
+        __builtin_amdgcn_sched_barrier(0);            // ... and before the products, not after them
+        const bf16_t* slot = &slots[i & 1][lane * 8];
+        bf16x8 b[GM_CH][MT];
+#pragma unroll
+        for (int j = 0; j < GM_CH; ++j)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) b[j][mt] = *(const bf16x8*)(slot + (j * MT + mt) * 512);
+#pragma unroll
+        for (int j = 0; j < GM_CH; ++j) {
+            const bf16x8 a = ((c_begin + i) * GM_CH + j < n_steps) ? a_cur[j] : zero;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j][mt], acc[mt], 0, 0, 0);
+        }
+        store_x(x_nxt, (i + 1) & 1);
+        // a bare barrier: __syncthreads() would wait for every load in flight
+        __builtin_amdgcn_s_waitcnt(0xC07F);           // lgkmcnt(0)
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);            // the next chunk's loads are issued after the barrier, in this order
+    };
+    int i = 0;
+    for (; i + 1 < n_iter; i += 2) {                  // no branch inside: the compiler's count of the loads in flight stays exact
+        chunk(i, a_even, a_odd, x_odd, x_even);
+        chunk(i + 1, a_odd, a_even, x_even, x_odd);
+    }
+    if (i < n_iter) chunk(i, a_even, a_odd, x_odd, x_even);
+
+    if (group >= n_groups) return;
+    // lane (token li, quarter g) holds features 16 * group + 4 g .. + 3 of token mt * 16 + li
+    if (SWIGLU) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int tok = mt * 16 + li;
+            f32x4 up;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) up[r] = __shfl_down(acc[mt][r], 16, 64);      // quarter g + 1 holds the up rows
+            const int f0 = group * 8 + 2 * g;
+            if ((g & 1) == 0 && tok < M && f0 < out_cols) {
+                f32x4 act;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) act[r] = acc[mt][r] / (1.0f + expf(-acc[mt][r])) * up[r];
+                TOut* p = out + (size_t)tok * out_cols + f0;
+                if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
+                    gm_store4<TOut>(p, act);
+                } else {
+                    for (int r = 0; r < 4 && f0 + r < out_cols; ++r) p[r] = from_f32<TOut>(act[r]);
+                }
+            }
+        }
+        return;
+    }
+    TOut* obase = out + (size_t)blockIdx.y * M * N;
+    const int f0 = group * 16 + 4 * g;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int tok = mt * 16 + li;
+        if (tok < M && f0 < N) {
+            TOut* p = obase + (size_t)tok * N + f0;
+            if (N % 4 == 0 && f0 + 4 <= N) {
+                gm_store4<TOut>(p, acc[mt]);
+            } else {
+                for (int r = 0; r < 4 && f0 + r < N; ++r) p[r] = from_f32<TOut>(acc[mt][r]);
+            }
+        }
+    }
+}
+
+template <typename TOut>
+__global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __restrict__ part, TOut* __restrict__ out,
+                                                              size_t total, int splits) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float s = part[i];
+    for (int z = 1; z < splits; ++z) s += part[(size_t)z * total + i];
+    out[i] = from_f32<TOut>(s);
+}
+
+static int g_mid_splits = 0;             // 0: chosen from the sizes (a fixed number for experiments)
+static int g_mid_waves = 0;              // waves per block: 0 = chosen from the sizes, else 4 or 8
+extern "C" int fl_gemm_mid_set_splits(int s) { g_mid_splits = s; return 0; }
+extern "C" int fl_gemm_mid_set_waves(int w) { g_mid_waves = w; return 0; }
+
+#define GM_STEPS 4                       // k-steps per chunk
+
+// Waves per block: eight row groups share x where the matrix has row groups enough to fill the
+// chip with such blocks, four otherwise.
+static int mid_waves(int N) {
+    if (g_mid_waves == 4 || g_mid_waves == 8) return g_mid_waves;
+    return ceil_div(N, 16) >= 1024 ? 8 : 4;
+}
+
+// How many ways K is split.  These products are short (tens of microseconds) and run best with
+// about one block per compute unit (measured on the 7B shapes at 32 and 64 rows); a part is at
+// least 4 chunks long.
+extern "C" int fl_gemm_mid_splits(int M, int N, int K) {
+    (void)M;
+    const int blocks = ceil_div(ceil_div(N, 16), mid_waves(N));
+    const int n_chunks = ceil_div(ceil_div(K, 32), GM_STEPS);
+    if (g_mid_splits > 0) return min(g_mid_splits, n_chunks);
+    int splits = 1;
+    while (blocks * splits * 2 <= 320 && n_chunks / (splits * 2) >= 4 && splits < 32) splits *= 2;
+    return splits;
+}
+
+template <int MT, int NW, int CH, typename TOut, bool SWIGLU>
+static void launch_mid_shape(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits, int out_cols,
+                             hipStream_t stream) {
+    const int n_steps = ceil_div(K, 32);
+    const int n_chunks = ceil_div(n_steps, CH);
+    const int per = ceil_div(n_chunks, splits);
+    dim3 grid(ceil_div(ceil_div(N, 16), NW), splits);
+    gemm_mid_kernel<MT, NW, CH, TOut, SWIGLU><<<grid, NW * 64, 0, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols);
+}
+
+template <int MT, typename TOut, bool SWIGLU>
+static void launch_mid(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits, int out_cols,
+                       hipStream_t stream) {
+    if (mid_waves(N) == 8) launch_mid_shape<MT, 8, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream);
+    else launch_mid_shape<MT, 4, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream);
+}
+
+template <typename TOut, bool SWIGLU>
+static void launch_mid_mt(int mt, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits,
+                          int out_cols, hipStream_t stream) {
+    switch (mt) {
+        case 1: launch_mid<1, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
+        case 2: launch_mid<2, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
+        case 3: launch_mid<3, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
+        default: launch_mid<4, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
+    }
+}
+
+// epilogue 0: out[M, N] = x w^T; a shape that splits K (fl_gemm_mid_splits > 1) needs a float
+// workspace of splits * M * N values.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up
+// from the N interleaved gate/up rows of w; K is not split then.
+extern "C" int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                           int M, int N, int K, int epilogue, int out_cols, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_mid: bad sizes M=%d N=%d K=%d", M, N, K);
+    FL_CHECK(M <= 64, "gemm_mid: %d rows, at most 64", M);
+    FL_CHECK(K % 32 == 0, "gemm_mid: K=%d is no multiple of 32 (whole k-steps of x)", K);
+    FL_CHECK((size_t)M * K < ((size_t)1 << 31), "gemm_mid: x of %d x %d values is beyond 32-bit offsets", M, K);
+    FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_mid: unknown output dtype %d", out_dtype);
+    FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_mid: unknown epilogue %d", epilogue);
+    FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
+             "gemm_mid: %d output columns do not fit %d rows of w", out_cols, N);
+    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
+             "gemm_mid: operands must be 16-byte aligned");
+    if (M == 0) return 0;
+    const int mt = ceil_div(M, 16);
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)w_packed;
+    const int splits = epilogue ? 1 : fl_gemm_mid_splits(M, N, K);
+    FL_CHECK(splits == 1 || workspace, "gemm_mid: this shape splits K %d ways and needs a workspace", splits);
+    if (epilogue) {
+        if (out_dtype == FL_F32) launch_mid_mt<float, true>(mt, xb, wb, (float*)out, M, N, K, 1, out_cols, stream);
+        else launch_mid_mt<bf16_t, true>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, out_cols, stream);
+    } else if (splits > 1) {
+        launch_mid_mt<float, false>(mt, xb, wb, workspace, M, N, K, splits, N, stream);
+        FL_LAUNCH_CHECK();
+        const size_t total = (size_t)M * N;
+        const unsigned rb = (unsigned)((total + 255) / 256);
+        if (out_dtype == FL_F32)
+            gemm_mid_reduce_kernel<float><<<rb, 256, 0, stream>>>(workspace, (float*)out, total, splits);
+        else
+            gemm_mid_reduce_kernel<bf16_t><<<rb, 256, 0, stream>>>(workspace, (bf16_t*)out, total, splits);
+    } else if (out_dtype == FL_F32) {
+        launch_mid_mt<float, false>(mt, xb, wb, (float*)out, M, N, K, 1, N, stream);
+    } else {
+        launch_mid_mt<bf16_t, false>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, N, stream);
+    }
+    FL_LAUNCH_CHECK();
+    return 0;
+}

@@ -14,13 +14,16 @@ from .packing import Weight, interleave_gate_up, pack_weight
 
 register_signatures({
     "fl_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, P],
+    "fl_gemm_mid": [P, P, P, P, I, I, I, I, I, I, P],
+    "fl_gemm_mid_splits": [I, I, I],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
 })
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64     # rows the decode kernels take
+SKINNY_BEST_ROWS = 16    # beyond one tile of tokens the kernel that shares x through LDS is faster
 
 
 def _packed_size(n_rows: int, K: int) -> int:
@@ -38,6 +41,29 @@ def gemm_skinny(x, w_packed, out, waves_per_block: int = 0, swiglu_rows: int = 0
     call("fl_gemm_skinny", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
          _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, int(waves_per_block),
          1 if swiglu_rows else 0, out.shape[1], stream_handle())
+    return out
+
+
+def gemm_mid_splits(M: int, N: int, K: int) -> int:
+    from .library import load
+    return load().fl_gemm_mid_splits(M, N, K)
+
+
+def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0):
+    """``out = x @ w.T`` for 17 to 64 rows of x (fewer are allowed) and K a multiple of 32: the
+    waves of a block share x through LDS.  A narrow matrix splits K and needs ``workspace``
+    (float32, ``gemm_mid_splits(M, N, K) * M * N`` values).  ``swiglu_rows`` as in ``gemm_skinny``."""
+    M, K = x.shape
+    N = swiglu_rows or out.shape[1]
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    splits = 1 if swiglu_rows else gemm_mid_splits(M, N, K)
+    if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
+        raise KernelError(f"gemm_mid: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
+    call("fl_gemm_mid", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(out, "gemm.out", None, (M, None)),
+         _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
+         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], stream_handle())
     return out
 
 
@@ -68,17 +94,19 @@ def gemm(x, w: Weight, out, rt=None):
     """``out = x @ w.T`` with the best kernel that takes the shape."""
     M, K = x.shape
     if w.packed is not None and not w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
-        if M <= SKINNY_MAX_ROWS:
-            return gemm_skinny(x, w.packed, out)
         N = w.rows
-        splits = gemm_tiled_splits(M, N, K)
+        mid = SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0
+        if M <= SKINNY_MAX_ROWS and not mid:
+            return gemm_skinny(x, w.packed, out)
+        splits = gemm_mid_splits(M, N, K) if mid else gemm_tiled_splits(M, N, K)
         workspace = None
         if splits > 1:
             if rt is None:
                 workspace = torch.empty(splits * M * N, dtype=torch.float32, device=x.device)
-            else:
-                workspace = rt.buffer("gemm_splitk", 1, splits * M * N, torch.float32, max_rows=1)
-        return gemm_tiled(x, w.packed, out, workspace)
+            else:       # one buffer for all shapes, in rows of 4096 floats
+                workspace = rt.buffer("gemm_splitk", -(-splits * M * N // 4096), 4096, torch.float32,
+                                      max_rows=1 << 20).view(-1)
+        return (gemm_mid if mid else gemm_tiled)(x, w.packed, out, workspace)
     if w.rowmajor is None:
         raise KernelError(f"gemm: no kernel for {M} rows of a packed [{w.rows}, {w.cols}] matrix")
     return ops.gemm_plain(x, w.rowmajor, out)
@@ -88,6 +116,8 @@ def gemm_swiglu(x, w: Weight, out, rt):
     """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``."""
     M, K = x.shape
     if w.packed is not None and w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
+        if SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0:
+            return gemm_mid(x, w.packed, out, swiglu_rows=w.packed_rows)
         if M <= SKINNY_MAX_ROWS:
             return gemm_skinny(x, w.packed, out, swiglu_rows=w.packed_rows)
         return gemm_tiled(x, w.packed, out, swiglu_rows=w.packed_rows)

@@ -397,8 +397,54 @@ def test_gemm_tiled_splits_k_for_small_grids():
         tuned().gemm_tiled(x, pack_weight(w), torch.empty(128, 256, dtype=torch.float32, device=DEV))
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("waves", [0, 4, 8])
+@pytest.mark.parametrize("M,N,K", [(64, 6144, 4096), (33, 4096, 14336), (17, 250, 96), (48, 37, 2048), (64, 16, 32),
+                                   (20, 1000, 160), (1, 300, 64), (49, 16400, 512)])
+def test_gemm_mid_against_plain(out_dtype, waves, M, N, K):
+    """The kernel for 17 to 64 rows, with both block shapes and with K split or whole."""
+    from flambeau_amd.kernels.library import load
+    from flambeau_amd.kernels.packing import pack_weight
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=41), rnd(N, K, dtype=torch.bfloat16, seed=42, scale=0.05)
+    packed = pack_weight(w)
+    ref = x.double() @ w.double().T
+    tol = 1e-5 if out_dtype == torch.float32 else 5e-3
+    load().fl_gemm_mid_set_waves(waves)
+    try:
+        for splits in (0, 1, 3):
+            load().fl_gemm_mid_set_splits(splits)
+            n = tuned().gemm_mid_splits(M, N, K)
+            ws = torch.full((n * M * N,), float("nan"), dtype=torch.float32, device=DEV) if n > 1 else None
+            got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+            tuned().gemm_mid(x, packed, got, ws)
+            assert (got.double() - ref).abs().max() < tol * ref.abs().max(), (splits, n)
+    finally:
+        load().fl_gemm_mid_set_splits(0)
+        load().fl_gemm_mid_set_waves(0)
+
+
+def test_gemm_mid_refuses_what_it_cannot_do():
+    from flambeau_amd.kernels import KernelError
+    from flambeau_amd.kernels.packing import pack_weight
+    out = torch.empty(20, 64, dtype=torch.float32, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 32"):
+        tuned().gemm_mid(rnd(20, 40, dtype=torch.bfloat16), pack_weight(rnd(64, 40, dtype=torch.bfloat16)), out)
+    with pytest.raises(KernelError, match="at most 64"):
+        tuned().gemm_mid(rnd(65, 64, dtype=torch.bfloat16), pack_weight(rnd(64, 64, dtype=torch.bfloat16)),
+                         torch.empty(65, 64, dtype=torch.float32, device=DEV))
+    w = rnd(64, 4096, dtype=torch.bfloat16)
+    assert tuned().gemm_mid_splits(20, 64, 4096) > 1
+    with pytest.raises(KernelError, match="workspace"):
+        tuned().gemm_mid(rnd(20, 4096, dtype=torch.bfloat16), pack_weight(w), out)
+    # a K the kernel does not take goes to the skinny kernel through the dispatcher
+    w40 = rnd(64, 40, dtype=torch.bfloat16, scale=0.1)
+    x40 = rnd(20, 40, dtype=torch.bfloat16)
+    tuned().gemm(x40, tuned().prepare_weight(w40), out)
+    assert (out.double() - x40.double() @ w40.double().T).abs().max() < 1e-4
+
+
 def test_gemm_dispatch_rows_agree_across_kernels():
-    """The same row through the skinny and the tiled kernel: equal up to float rounding of sums."""
+    """The same rows through the skinny, the middle and the tiled kernel: equal up to float rounding of sums."""
     w = rnd(512, 1024, dtype=torch.bfloat16, seed=23, scale=0.05)
     x = rnd(200, 1024, dtype=torch.bfloat16, seed=24)
     W = tuned().prepare_weight(w)
@@ -407,6 +453,9 @@ def test_gemm_dispatch_rows_agree_across_kernels():
     small = torch.empty(3, 512, dtype=torch.float32, device=DEV)
     tuned().gemm(x[17:20].contiguous(), W, small)
     assert (big[17:20] - small).abs().max() < 1e-5 * big.abs().max()
+    middle = torch.empty(40, 512, dtype=torch.float32, device=DEV)       # the kernel for 17 to 64 rows
+    tuned().gemm(x[10:50].contiguous(), W, middle)
+    assert (big[10:50] - middle).abs().max() < 1e-5 * big.abs().max()
 
 
 # ---------------------------------------------------------------- tiled attention for portions
@@ -485,7 +534,7 @@ def test_attn_prefill_peaked_scores_find_single_keys():
 # ---------------------------------------------------------------- gated feed-forward in the product's epilogue
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,I,K", [(1, 14336, 4096), (8, 224, 96), (64, 136, 80), (5, 13, 40), (200, 14336, 512),
-                                   (65, 160, 64), (300, 52, 72), (16, 8, 8)])
+                                   (65, 160, 64), (300, 52, 72), (16, 8, 8), (40, 14336, 4096), (23, 100, 96)])
 def test_gemm_swiglu_epilogue(out_dtype, M, I, K):
     gate = rnd(I, K, dtype=torch.bfloat16, seed=31, scale=0.3)
     up = rnd(I, K, dtype=torch.bfloat16, seed=32, scale=0.3)
@@ -501,3 +550,7 @@ def test_gemm_swiglu_epilogue(out_dtype, M, I, K):
     ref = g / (1 + torch.exp(-g)) * u
     tol = 2e-5 if out_dtype == torch.float32 else 6e-3
     assert (got.double() - ref).abs().max() < tol * ref.abs().max()
+    if M <= 64 and K % 32 == 0:
+        mid = torch.full((M, I), float("nan"), dtype=out_dtype, device=DEV)
+        tuned().gemm_mid(x, W.packed, mid, swiglu_rows=W.packed_rows)
+        assert (mid.double() - ref).abs().max() < tol * ref.abs().max()
