@@ -42,6 +42,15 @@ int fl_sample(const float* logits, const float* inv_temp, const float* uniform, 
 int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
                    int nw_hint, int epilogue, int out_cols, hipStream_t stream);
 
+// The same product fused with the norms around it (at most 16 rows).  in_ssq (or null): [M, in_parts]
+// partial sums of squares; every row of the result is multiplied by rsqrt(sum / K + eps).
+// epilogue 2: resid[M, N] += the product, xg[M, N] = bf16(resid * g), out_ssq[M, ceil(N / 16)] = the
+// blocks' sums of resid^2; nothing is stored in out.
+int fl_gemm_skinny_fused(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
+                         int epilogue, int out_cols, const float* in_ssq, int in_parts, float eps,
+                         float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream);
+int fl_gemm_skinny_scale_parts(int N, int K, int in_parts);
+
 // 17 to 64 rows, K a multiple of 32; a shape with fl_gemm_mid_splits > 1 needs a float workspace
 // of splits * M * N values
 int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,

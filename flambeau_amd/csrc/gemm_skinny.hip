@@ -17,6 +17,16 @@
 //    consecutive features of one token, i.e. one 16-byte store.  Rows of x beyond M are not
 //    loaded.  With MT > 1 the same w registers feed MT token tiles.
 //
+// Two fusions with the norm around a product save a kernel each in a decode step:
+//  * epilogue 2 (residual): instead of storing the product the block adds it to the residual
+//    stream r (float, in place), stores bf16(r * g) for the next product (g = the weight of the
+//    norm that follows) and the sum of r^2 over its 16 features, one value per token and block;
+//  * row scale: a product whose x is such a bf16(r * g) multiplies every token's results by
+//    rsqrt(sum r^2 / K + eps), the sums of the producing blocks added in a fixed order.  The
+//    scale commutes with the product, so together the two are norm(r) W^T without a norm kernel
+//    (the reference fuses the add into its norm kernel instead,
+//    crates/kernels-hip/src/kernels/rmsnorm_f16_add_residual.cu).
+//
 // The reference's nearest kernels are its float GEMV, one block per output row
 // (crates/kernels-hip/src/kernels/dense_gemv_f16_f16.cu:27-71, ..._batched.cu:17-63).
 #include "common.h"
@@ -31,12 +41,28 @@ __device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
 // SWIGLU: the rows of w are gate and up rows interleaved in fours ([g0-3 | u0-3 | g4-7 | u4-7] per
 // group of 16, see interleave_gate_up in kernels/packing.py); the kernel then writes
 // silu(gate) * up, N / 2 values per token, instead of the N products.
-template <int MT, typename TOut, bool SWIGLU>
+struct SkinnyFusion {
+    const float* in_ssq;      // [M][in_parts] sums of squares of the rows of x before the norm's weight, or null
+    int in_parts;
+    float eps;
+    float* resid;             // epilogue 2: [M][N], read and written
+    const float* g;           // epilogue 2: [N] weight of the following norm
+    bf16_t* xg;               // epilogue 2: [M][N] bf16(resid * g)
+    float* out_ssq;           // epilogue 2: [M][blocks] sum of resid^2 over the block's features
+};
+
+#define SKINNY_SCALE_LOADS 4     // loads of partial sums per thread for the row scale
+#define EPI_PLAIN 0
+#define EPI_SWIGLU 1
+#define EPI_RESIDUAL 2
+
+template <int MT, typename TOut, int EPI>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ wp,
                                                            TOut* __restrict__ out, int M, int N, int K,
-                                                           int n_steps, int out_cols) {
-    extern __shared__ float red[];               // [NW][MT][64][4]
+                                                           int n_steps, int out_cols, SkinnyFusion fu) {
+    constexpr bool SWIGLU = EPI == EPI_SWIGLU;
+    extern __shared__ float red[];               // [NW][MT][64][4], then [NW * 4][16] for the row scale
     const int nw = blockDim.x >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int li = lane & 15, g = lane >> 4;
@@ -59,6 +85,53 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // row scale (one tile of tokens only): thread t fetches its share of the parts of token t % 16
+    // (in fours where the number of parts allows 16-byte loads); the loads are in flight during
+    // the loop and are added after it
+    constexpr int SSV = SKINNY_SCALE_LOADS;
+    f32x4 sv[SSV];
+#pragma unroll
+    for (int j = 0; j < SSV; ++j) sv[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (MT == 1 && fu.in_ssq) {
+        const int n_slices = blockDim.x >> 4;
+        const int tok = threadIdx.x & 15;
+        if (tok < M) {
+            const float* row = fu.in_ssq + (size_t)tok * fu.in_parts;
+            if ((fu.in_parts & 3) == 0) {
+#pragma unroll
+                for (int j = 0; j < SSV; ++j) {
+                    const int p = ((threadIdx.x >> 4) + j * n_slices) * 4;
+                    if (p < fu.in_parts) sv[j] = *(const f32x4*)(row + p);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < SSV; ++j) {
+                    const int p = (threadIdx.x >> 4) + j * n_slices;
+                    if (p < fu.in_parts) sv[j][0] = row[p];
+                }
+            }
+        }
+    }
+    // epilogue 2: wave 0 fetches its part of the residual stream and of g before the loop
+    f32x4 r_in[MT], g_in = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) r_in[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (EPI == EPI_RESIDUAL && MT == 1 && wave == 0) {
+        const int f0 = blockIdx.x * 16 + 4 * g;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (f0 + r < N) g_in[r] = fu.g[f0 + r];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int tok = mt * 16 + li;
+            if (tok < M) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (f0 + r < N) r_in[mt][r] = fu.resid[(size_t)tok * N + f0 + r];
+            }
+        }
+    }
 
     int s = s0;
     // iterations of U steps: every load of the iteration is issued before the first product needs
@@ -86,6 +159,13 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     // add the waves' partial sums in wave order
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *(f32x4*)(red + (((size_t)wave * MT + mt) * 64 + lane) * 4) = acc[mt];
+    float* ssred = red + (size_t)nw * MT * 256;                  // [MT][slices][16]
+    if (MT == 1 && fu.in_ssq) {
+        float t = 0.f;
+#pragma unroll
+        for (int j = 0; j < SSV; ++j) t += (sv[j][0] + sv[j][1]) + (sv[j][2] + sv[j][3]);
+        ssred[(threadIdx.x >> 4) * 16 + (threadIdx.x & 15)] = t;
+    }
     __syncthreads();
     if (wave == 0) {
 #pragma unroll
@@ -97,7 +177,45 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
             }
             // lane (token li, group g) holds rows 16*block + 4g .. 4g+3 of token mt*16 + li
             const int tok = mt * 16 + li;
-            if (SWIGLU) {
+            if (MT == 1 && fu.in_ssq) {
+                // the token's sum of squares: slices g, g + 4, ... by this lane, then the four lanes of the token
+                const int n_slices = blockDim.x >> 4;
+                float t = 0.f;
+                for (int sl = g; sl < n_slices; sl += 4) t += ssred[sl * 16 + li];
+                t += __shfl_xor(t, 16, 64);
+                t += __shfl_xor(t, 32, 64);
+                const float scale = rsqrtf(t / (float)K + fu.eps);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sum[r] *= scale;
+            }
+            if (EPI == EPI_RESIDUAL) {
+                const int f0 = blockIdx.x * 16 + 4 * g;
+                f32x4 nr;
+                float sq = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    nr[r] = r_in[mt][r] + sum[r];
+                    if (f0 + r < N) sq += nr[r] * nr[r];
+                }
+                sq += __shfl_xor(sq, 16, 64);
+                sq += __shfl_xor(sq, 32, 64);
+                if (tok < M) {
+                    if (g == 0) fu.out_ssq[(size_t)tok * gridDim.x + blockIdx.x] = sq;
+                    if (f0 < N) {
+                        float* pr = fu.resid + (size_t)tok * N + f0;
+                        bf16_t* px = fu.xg + (size_t)tok * N + f0;
+                        if (N % 4 == 0 && f0 + 4 <= N) {
+                            store4(pr, nr);
+                            store4(px, (f32x4){nr[0] * g_in[0], nr[1] * g_in[1], nr[2] * g_in[2], nr[3] * g_in[3]});
+                        } else {
+                            for (int r = 0; r < 4 && f0 + r < N; ++r) {
+                                pr[r] = nr[r];
+                                px[r] = from_f32<bf16_t>(nr[r] * g_in[r]);
+                            }
+                        }
+                    }
+                }
+            } else if (SWIGLU) {
                 f32x4 up;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) up[r] = __shfl_down(sum[r], 16, 64);      // lane g+1 holds the up rows
@@ -128,9 +246,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     }
 }
 
-template <int MT, typename TOut>
-static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
-                         int swiglu, int out_cols, hipStream_t stream) {
+static int skinny_waves(int N, int K, int nw_hint) {
     const int groups = ceil_div(N, 16);
     const int n_steps = ceil_div(K, 32);
     // enough waves in flight to cover the memory latency: about 2048 and more over the chip
@@ -138,32 +254,59 @@ static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, in
     while (nw < 16 && groups * nw < 2048) nw *= 2;
     if (nw_hint > 0) nw = nw_hint;
     while (nw > 1 && n_steps < nw * 2) nw /= 2;
-    const size_t lds = (size_t)nw * MT * 64 * 4 * sizeof(float);
-    if (swiglu)
-        gemm_skinny_kernel<MT, TOut, true><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols);
+    return nw;
+}
+
+// How many partial sums per token the row scale of a product of this shape can add.
+extern "C" int fl_gemm_skinny_scale_parts(int N, int K, int in_parts) {
+    const int slices = 4 * skinny_waves(N, K, 0);
+    return SKINNY_SCALE_LOADS * slices * ((in_parts & 3) == 0 ? 4 : 1);
+}
+
+template <int MT, typename TOut>
+static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
+                         int epilogue, int out_cols, const SkinnyFusion& fu, hipStream_t stream) {
+    const int groups = ceil_div(N, 16);
+    const int n_steps = ceil_div(K, 32);
+    const int nw = skinny_waves(N, K, nw_hint);
+    const size_t lds = (size_t)nw * MT * 64 * 4 * sizeof(float) + (size_t)nw * 4 * 16 * sizeof(float);
+    if (epilogue == EPI_SWIGLU)
+        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu);
+    else if (epilogue == EPI_RESIDUAL)
+        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu);
     else
-        gemm_skinny_kernel<MT, TOut, false><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols);
+        gemm_skinny_kernel<MT, TOut, EPI_PLAIN><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu);
     return 0;
 }
 
-// epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): w holds N interleaved gate/up rows and
-// out[M, out_cols] = silu(gate) * up with out_cols <= N / 2.
-extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N,
-                              int K, int nw_hint, int epilogue, int out_cols, hipStream_t stream) {
+static int skinny_entry(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
+                        int nw_hint, int epilogue, int out_cols, const SkinnyFusion& fu, hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
     FL_CHECK(nw_hint >= 0 && nw_hint <= 16, "gemm_skinny: %d waves per block, at most 16", nw_hint);
     FL_CHECK(K % 8 == 0, "gemm_skinny: K=%d is no multiple of 8 (16-byte loads)", K);
-    FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_skinny: unknown epilogue %d", epilogue);
-    FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
+    FL_CHECK(epilogue >= 0 && epilogue <= 2, "gemm_skinny: unknown epilogue %d", epilogue);
+    FL_CHECK(epilogue != EPI_SWIGLU ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
              "gemm_skinny: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
              "gemm_skinny: operands must be 16-byte aligned");
+    if (epilogue == EPI_RESIDUAL) {
+        FL_CHECK(fu.resid && fu.g && fu.xg && fu.out_ssq, "gemm_skinny: the residual epilogue needs resid, g, xg and out_ssq");
+        FL_CHECK(((uintptr_t)fu.resid % 16 == 0) && ((uintptr_t)fu.xg % 8 == 0), "gemm_skinny: resid and xg must be aligned to 16 and 8 bytes");
+    }
+    if (fu.in_ssq || epilogue == EPI_RESIDUAL)
+        FL_CHECK(M <= 16, "gemm_skinny: the fusions with the norm take at most 16 rows, not %d", M);
+    if (fu.in_ssq) {
+        const int cap = fl_gemm_skinny_scale_parts(N, K, fu.in_parts);
+        FL_CHECK(fu.in_parts > 0 && fu.in_parts <= cap, "gemm_skinny: a row scale over %d parts (at most %d for this shape)",
+                 fu.in_parts, cap);
+        FL_CHECK((uintptr_t)fu.in_ssq % 16 == 0, "gemm_skinny: the partial sums must be 16-byte aligned");
+    }
     if (M == 0) return 0;
     const int mt = ceil_div(M, 16);
 #define FL_SK(MT_)                                                                                         \
-    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N, K, nw_hint, epilogue, out_cols, stream); \
-    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M, N, K, nw_hint, epilogue, out_cols, stream)
+    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N, K, nw_hint, epilogue, out_cols, fu, stream); \
+    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M, N, K, nw_hint, epilogue, out_cols, fu, stream)
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
     switch (mt) {
         case 1: FL_SK(1); break;
@@ -175,3 +318,29 @@ extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, in
     FL_LAUNCH_CHECK();
     return 0;
 }
+
+// epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): w holds N interleaved gate/up rows and
+// out[M, out_cols] = silu(gate) * up with out_cols <= N / 2.
+extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N,
+                              int K, int nw_hint, int epilogue, int out_cols, hipStream_t stream) {
+    FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_skinny: unknown epilogue %d", epilogue);
+    const SkinnyFusion none = {nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr};
+    return skinny_entry(x, w_packed, out, out_dtype, M, N, K, nw_hint, epilogue, out_cols, none, stream);
+}
+
+// The same product fused with the norms around it.  in_ssq (or null): [M, in_parts] partial sums of
+// squares of the rows that x was made from; every token's results are multiplied by
+// rsqrt(sum / K + eps).  epilogue 2: nothing is stored in out (it may be null); resid[M, N] += the
+// product, xg[M, N] = bf16(resid * g), out_ssq[M, blocks] = the blocks' sums of resid^2, blocks =
+// fl_gemm_skinny_blocks(N).
+extern "C" int fl_gemm_skinny_fused(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N,
+                                    int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
+                                    float eps, float* resid, const float* g, void* xg, float* out_ssq,
+                                    hipStream_t stream) {
+    const SkinnyFusion fu = {in_ssq, in_parts, eps, resid, g, (bf16_t*)xg, out_ssq};
+    if (epilogue == EPI_RESIDUAL && !out) out = resid;
+    return skinny_entry(x, w_packed, out, epilogue == EPI_RESIDUAL ? FL_F32 : out_dtype, M, N, K, 0, epilogue,
+                        out_cols, fu, stream);
+}
+
+extern "C" int fl_gemm_skinny_blocks(int N) { return ceil_div(N, 16); }

@@ -5,6 +5,8 @@ kernel does not take a shape (a K that is no multiple of 8, a head size beyond 2
 kernel runs instead, so a size is never answered with a wrong result."""
 from __future__ import annotations
 
+from dataclasses import dataclass
+
 import torch
 
 from . import ops
@@ -14,6 +16,8 @@ from .packing import Weight, interleave_gate_up, pack_weight
 
 register_signatures({
     "fl_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, P],
+    "fl_gemm_skinny_fused": [P, P, P, I, I, I, I, I, I, P, I, F, P, P, P, P, P],
+    "fl_gemm_skinny_scale_parts": [I, I, I],
     "fl_gemm_mid": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_mid_splits": [I, I, I],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
@@ -30,18 +34,81 @@ def _packed_size(n_rows: int, K: int) -> int:
     return (-(-n_rows // 16) * 16) * (-(-K // 32) * 32)
 
 
-def gemm_skinny(x, w_packed, out, waves_per_block: int = 0, swiglu_rows: int = 0):
+FUSED_NORM_MAX_ROWS = 16     # the fusions of a product with the norms around it take one tile of tokens
+
+
+@dataclass
+class NormedRows:
+    """Rows ``norm(r)`` that exist only in factors: ``xg = bf16(r * g)`` (g = the norm's weight)
+    and ``ssq[m, p]``, the sum of ``r[m]^2`` in parts, so that ``norm(r)[m] = xg[m] * rsqrt(sum_p
+    ssq[m, p] / H + eps)``.  A product takes the factor out of its sum and applies it to its
+    results (``gemm_skinny`` with ``row_scale``).  ``resid`` and ``weight`` are kept for kernels
+    that want the rows themselves (``materialize``)."""
+    xg: torch.Tensor
+    ssq: torch.Tensor
+    eps: float
+    resid: torch.Tensor
+    weight: torch.Tensor
+
+    @property
+    def shape(self):
+        return self.xg.shape
+
+    @property
+    def dtype(self):
+        return self.xg.dtype
+
+    def materialize(self, rt):
+        out = rt.buffer("normed_rows", self.xg.shape[0], self.xg.shape[1])
+        return ops.rmsnorm(self.resid, self.weight, out, self.eps)
+
+
+def skinny_parts(n_features: int) -> int:
+    """Parts in which ``gemm_skinny_residual`` leaves the sums of squares of its N features."""
+    return -(-n_features // 16)
+
+
+def _row_scale_args(row_scale, M, K):
+    if row_scale is None:
+        return None, 0, 0.0
+    parts = row_scale.ssq.shape[1]
+    return _check(row_scale.ssq, "gemm.row_scale", torch.float32, (M, parts)), parts, float(row_scale.eps)
+
+
+def gemm_skinny(x, w_packed, out, waves_per_block: int = 0, swiglu_rows: int = 0, row_scale: NormedRows | None = None):
     """``out = x @ w.T`` for up to 64 rows of x; ``w_packed`` = ``pack_weight(w)``, N rows taken
     from ``out``.  With ``swiglu_rows`` the packed matrix holds that many interleaved gate/up
-    rows and ``out`` receives ``silu(gate) * up``."""
+    rows and ``out`` receives ``silu(gate) * up``.  With ``row_scale`` (then ``x`` is its ``xg``,
+    at most 16 rows) every row of the product is scaled by the norm's factor first."""
     M, K = x.shape
     N = swiglu_rows or out.shape[1]
     if w_packed.numel() != _packed_size(N, K):
         raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
-    call("fl_gemm_skinny", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, int(waves_per_block),
-         1 if swiglu_rows else 0, out.shape[1], stream_handle())
+    if row_scale is None:
+        call("fl_gemm_skinny", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+             _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, int(waves_per_block),
+             1 if swiglu_rows else 0, out.shape[1], stream_handle())
+        return out
+    ssq, parts, eps = _row_scale_args(row_scale, M, K)
+    call("fl_gemm_skinny_fused", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0,
+         out.shape[1], ssq, parts, eps, None, None, None, None, stream_handle())
     return out
+
+
+def gemm_skinny_residual(x, w_packed, resid, g, xg, ssq, eps: float, row_scale: NormedRows | None = None) -> NormedRows:
+    """``resid += x @ w.T`` (float32, in place) for at most 16 rows, and the factors of the norm that
+    follows: ``xg = bf16(resid * g)``, ``ssq[m, p]`` = sum of ``resid[m]^2`` over features 16 p .. 16 p + 15."""
+    M, K = x.shape
+    N = resid.shape[1]
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    in_ssq, parts, in_eps = _row_scale_args(row_scale, M, K)
+    call("fl_gemm_skinny_fused", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         None, 0, M, N, K, 2, N, in_ssq, parts, in_eps, _check(resid, "gemm.resid", torch.float32, (M, N)),
+         _check(g, "gemm.g", torch.float32, (N,)), _check(xg, "gemm.xg", torch.bfloat16, (M, N)),
+         _check(ssq, "gemm.ssq", torch.float32, (M, skinny_parts(N))), stream_handle())
+    return NormedRows(xg, ssq, float(eps), resid, g)
 
 
 def gemm_mid_splits(M: int, N: int, K: int) -> int:
@@ -90,9 +157,25 @@ def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0):
     return out
 
 
+def _rows_for(x, w: Weight, rt):
+    """``x`` and its row scale for a product with ``w``: factored rows stay factored where the
+    skinny kernel runs, else the rows are made."""
+    if not isinstance(x, NormedRows):
+        return x, None
+    if w.packed is not None and x.shape[0] <= FUSED_NORM_MAX_ROWS and x.shape[1] % 8 == 0:
+        from .library import load
+        parts = x.ssq.shape[1]
+        if parts <= load().fl_gemm_skinny_scale_parts(w.packed_rows, x.shape[1], parts):
+            return x.xg, x
+    return x.materialize(rt), None
+
+
 def gemm(x, w: Weight, out, rt=None):
-    """``out = x @ w.T`` with the best kernel that takes the shape."""
+    """``out = x @ w.T`` with the best kernel that takes the shape; ``x`` may be ``NormedRows``."""
+    x, scale = _rows_for(x, w, rt)
     M, K = x.shape
+    if scale is not None:
+        return gemm_skinny(x, w.packed, out, row_scale=scale)
     if w.packed is not None and not w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
         N = w.rows
         mid = SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0
@@ -113,8 +196,13 @@ def gemm(x, w: Weight, out, rt=None):
 
 
 def gemm_swiglu(x, w: Weight, out, rt):
-    """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``."""
+    """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``; ``x`` may be ``NormedRows``."""
+    x, scale = _rows_for(x, w, rt)
     M, K = x.shape
+    if scale is not None and w.swiglu_cols:
+        return gemm_skinny(x, w.packed, out, swiglu_rows=w.packed_rows, row_scale=scale)
+    if scale is not None:
+        x = scale.materialize(rt)
     if w.packed is not None and w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
         if SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0:
             return gemm_mid(x, w.packed, out, swiglu_rows=w.packed_rows)

@@ -44,6 +44,9 @@ class ModelSpec:
     bos_token_id: int | None = None
 
 
+SMALL_STEP = 16      # up to this many rows the output head runs on every row of a step
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, rt):
         self.spec = spec
@@ -120,5 +123,12 @@ class DecoderModel:
         if step.logit_rows.shape[0] == 0:
             stream.flush()
             return None
+        every_row = step.host.n_logit_rows == step.n_tokens          # a decode step: rows 0 .. n - 1 in order
+        if every_row or step.n_tokens <= SMALL_STEP:
+            # a few rows cost what one row costs: all of them take the path of a decode step (the
+            # same kernels whatever is wanted), and the wanted ones are picked afterwards
+            x = stream.normed(self.final_norm, name="final", lazy=True)
+            logits = self.head.forward(x, max(max_logit_rows, step.n_tokens))
+            return logits if every_row else torch.index_select(logits, 0, step.logit_rows)
         x = stream.normed(self.final_norm, rows=step.logit_rows, name="final")
         return self.head.forward(x, max_logit_rows)

@@ -17,12 +17,13 @@ import math
 import torch
 
 from ..kernels import ops
-from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, TensorSpec
+from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, Product, TensorSpec
 
 
 @MIXERS.register("paged_gqa_attention")
 class PagedGQAAttention(Mixer):
     graph_safe = True
+    lazy_input = True
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, window: int = 0, scale: float | None = None):
@@ -75,6 +76,4 @@ class PagedGQAAttention(Mixer):
             tuned.attention(rt, q, out, cache.kv, step, table, nh, self.scale, self.window)
         else:
             ops.attn_plain(q, out, cache.kv, step.positions, step.tok_seq, table, nh, self.scale, self.window)
-        delta = rt.buffer("delta", n, self.hidden_size, torch.float32)
-        rt.gemm(out, self.w_o, delta)
-        return delta
+        return Product(out, self.w_o)

@@ -117,11 +117,35 @@ class Part:
         self.rt = rt
 
 
+class Product:
+    """A part's output as a matrix product that is not yet computed: ``x @ weight.T`` (``weight``
+    from ``rt.prepare_weight``).  A mixer or feed-forward may return it instead of the delta
+    tensor; the residual stream that receives it computes it, fused with what follows where a
+    kernel for that exists."""
+
+    def __init__(self, x, weight):
+        self.x = x
+        self.weight = weight
+
+    def compute(self, rt, out=None):
+        """The product itself, float32 ``[n, weight.rows]``."""
+        if out is None:
+            out = rt.buffer("delta", self.x.shape[0], self.weight.rows, torch.float32)
+        return rt.gemm(self.x, self.weight, out)
+
+
 class Norm(Part):
     def forward(self, x, out, delta=None, store_sum=False, rows=None):
         """``out = norm(x (+ delta))``; ``x`` is the 32-bit residual stream; with
         ``store_sum`` the sum is written back to ``x``; ``rows`` selects rows."""
         raise NotImplementedError
+
+    def after_product(self, rt, resid, product: Product):
+        """Optional fusion: add ``product`` to ``resid`` and return the normed sum as an object
+        that ``rt.gemm`` and ``rt.gemm_swiglu`` take in place of a tensor, or ``None`` if this
+        norm or these sizes have no such kernel (the caller then computes the product, and
+        ``forward`` norms)."""
+        return None
 
 
 class PositionEncoding(Part):
@@ -140,6 +164,9 @@ class Mixer(Part):
     # values are written by position).  A mixer that advances a state of its own is not, and a
     # model with such a mixer never replays captured steps.
     graph_safe = False
+    # True if ``forward`` hands its input ``x`` to ``rt.gemm`` / ``rt.gemm_swiglu`` only: ``x`` may
+    # then be a normed input that exists in factors (see ``Norm.after_product``), not a tensor.
+    lazy_input = False
 
     def cache_spec(self):
         """``PagedKVSpec``, ``StateSpec`` or ``None``."""
@@ -153,12 +180,16 @@ class Mixer(Part):
 
     def forward(self, x, step: StepState, cache: LayerCache):
         """``x``: normed activations [n, hidden] in the compute dtype.  Returns the
-        32-bit delta [n, hidden] that is added to the residual stream."""
+        32-bit delta [n, hidden] that is added to the residual stream, or a ``Product`` that
+        computes it."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
+    lazy_input = False      # as for Mixer
+
     def forward(self, x, step: StepState):
+        """Returns the 32-bit delta [n, hidden], or a ``Product`` that computes it."""
         raise NotImplementedError
 
 

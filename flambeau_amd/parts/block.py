@@ -8,28 +8,41 @@ which adds it, stores the sum and norms it in one kernel
 from __future__ import annotations
 
 from ..kernels import ops
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartSpec
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartSpec, Product
 
 
 class ResidualStream:
     def __init__(self, resid, rt):
         self.resid = resid          # float32 [n, hidden]
         self.rt = rt
-        self.pending = None         # float32 [n, hidden] not yet added
+        self.pending = None         # float32 [n, hidden] not yet added, or a Product not yet computed
 
     def push(self, delta):
+        """``delta``: what a part returned, a tensor or a ``Product``."""
         self.flush()
         self.pending = delta
 
+    def _pending_tensor(self):
+        if isinstance(self.pending, Product):
+            self.pending = self.pending.compute(self.rt)
+        return self.pending
+
     def flush(self):
-        if self.pending is not None:
+        if self._pending_tensor() is not None:
             ops.add_inplace(self.resid, self.pending)
             self.pending = None
         return self.resid
 
-    def normed(self, norm, rows=None, name="normed"):
-        """The normed stream in the compute dtype, the pending delta added on the way."""
+    def normed(self, norm, rows=None, name="normed", lazy=False):
+        """The normed stream in the compute dtype, the pending delta added on the way.  With
+        ``lazy`` the caller takes what ``Norm.after_product`` returns as well as a tensor."""
         n, H = self.resid.shape
+        if lazy and rows is None and isinstance(self.pending, Product):
+            fused = norm.after_product(self.rt, self.resid, self.pending)
+            if fused is not None:
+                self.pending = None
+                return fused
+        self._pending_tensor()
         if rows is not None:
             out = self.rt.buffer(name + "_rows", rows.shape[0], H)
             norm.forward(self.resid, out, delta=self.pending, rows=rows)
@@ -65,5 +78,5 @@ class PreNormBlock(Block):
             part.bind({k[len(p) + 1:]: v for k, v in weights.items() if k.startswith(p + ".")}, rt)
 
     def forward(self, stream, step, cache):
-        stream.push(self.mixer.forward(stream.normed(self.mixer_norm), step, cache))
-        stream.push(self.ffn.forward(stream.normed(self.ffn_norm), step))
+        stream.push(self.mixer.forward(stream.normed(self.mixer_norm, lazy=self.mixer.lazy_input), step, cache))
+        stream.push(self.ffn.forward(stream.normed(self.ffn_norm, lazy=self.ffn.lazy_input), step))

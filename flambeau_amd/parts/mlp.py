@@ -5,11 +5,13 @@ from __future__ import annotations
 
 import torch
 
-from .base import FEED_FORWARDS, FeedForward, TensorSpec
+from .base import FEED_FORWARDS, FeedForward, Product, TensorSpec
 
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    lazy_input = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
@@ -28,6 +30,4 @@ class SwiGLU(FeedForward):
         rt, n, I = self.rt, x.shape[0], self.intermediate_size
         act = rt.buffer("ffn_act", n, I)
         rt.gemm_swiglu(x, self.w_gate_up, act)
-        delta = rt.buffer("delta", n, self.hidden_size, torch.float32)
-        rt.gemm(act, self.w_down, delta)
-        return delta
+        return Product(act, self.w_down)

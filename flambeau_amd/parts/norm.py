@@ -3,6 +3,8 @@
 pending delta to the residual stream follows rmsnorm_f16_add_residual.cu."""
 from __future__ import annotations
 
+import torch
+
 from ..kernels import ops
 from .base import NORMS, Norm, TensorSpec
 
@@ -22,3 +24,19 @@ class RMSNorm(Norm):
 
     def forward(self, x, out, delta=None, store_sum=False, rows=None):
         return ops.rmsnorm(x, self.weight, out, self.eps, delta=delta, store_sum=store_sum, rows=rows)
+
+    def after_product(self, rt, resid, product):
+        """For a few rows (a decode step) the product's kernel adds its result to the stream and
+        leaves the norm in factors: x * w in the compute dtype and the sums of squares in parts.
+        The product that follows multiplies by rsqrt(mean + eps) itself: no norm kernel runs."""
+        if not rt.tuned:
+            return None
+        from ..kernels import tuned
+        n, H = resid.shape
+        w, x = product.weight, product.x
+        if (n > tuned.FUSED_NORM_MAX_ROWS or w.packed is None or w.swiglu_cols or isinstance(x, tuned.NormedRows)
+                or x.dtype != torch.bfloat16 or x.shape[1] % 8 or H % 8):
+            return None
+        xg = rt.buffer("normed_xg", n, H)
+        ssq = rt.buffer("normed_ssq", n, tuned.skinny_parts(H), torch.float32)
+        return tuned.gemm_skinny_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps)

@@ -122,6 +122,47 @@ def test_gemm_skinny_against_plain(out_dtype, M, N, K):
     assert (got.double() - plain.double()).abs().max() < 2 * tol * scale
 
 
+@pytest.mark.parametrize("M,H,N2,I,eps", [(1, 4096, 6144, 512, 1e-5), (8, 4096, 32768, 14336, 1e-5), (16, 72, 40, 104, 1e-2),
+                                            (3, 136, 250, 40, 1e-6), (5, 64, 16, 8, 1e-5)])
+def test_gemm_skinny_fused_with_the_norms_around_it(M, H, N2, I, eps):
+    """resid += a W1^T in the product's epilogue, norm(resid) W2^T through the row scale of the next
+    product, against the same chain in float64; and the SwiGLU epilogue after a row scale."""
+    from flambeau_amd.kernels.packing import pack_weight
+    a = rnd(M, I, dtype=torch.bfloat16, seed=51)
+    w1 = rnd(H, I, dtype=torch.bfloat16, seed=52, scale=0.05)
+    w2 = rnd(N2, H, dtype=torch.bfloat16, seed=53, scale=0.05)
+    g = rnd(H, seed=54).abs() + 0.5
+    resid0 = rnd(M, H, seed=55)
+    resid = resid0.clone()
+    xg = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ssq = torch.full((M, tuned().skinny_parts(H)), float("nan"), dtype=torch.float32, device=DEV)
+    rows = tuned().gemm_skinny_residual(a, pack_weight(w1), resid, g, xg, ssq, eps)
+    r_ref = resid0.double() + a.double() @ w1.double().T
+    assert (resid.double() - r_ref).abs().max() < 1e-5 * r_ref.abs().max()
+    assert (ssq.double().sum(1) - (r_ref ** 2).sum(1)).abs().max() < 1e-5 * (r_ref ** 2).sum(1).max()
+    assert (xg.double() - r_ref * g.double()).abs().max() < 5e-3 * (r_ref * g.double()).abs().max()
+    normed = r_ref * torch.rsqrt((r_ref ** 2).mean(1, keepdim=True) + eps) * g.double()
+    ref = normed @ w2.double().T
+    W2 = tuned().prepare_weight(w2)
+    got = torch.full((M, N2), float("nan"), dtype=torch.float32, device=DEV)
+    tuned().gemm(rows, W2, got)
+    assert (got.double() - ref).abs().max() < 6e-3 * ref.abs().max()
+    # the rows themselves, for kernels that do not take the factors
+    class Rt:
+        def buffer(self, name, n, cols, dtype=torch.bfloat16):
+            return torch.empty(n, cols, dtype=dtype, device=DEV)
+    made = rows.materialize(Rt())
+    assert (made.double() - normed).abs().max() < 5e-3 * normed.abs().max()
+    if N2 % 32 == 0:
+        gate, up = w2[:N2 // 2].contiguous(), w2[N2 // 2:].contiguous()
+        Wgu = tuned().prepare_gate_up(gate, up)
+        act = torch.full((M, N2 // 2), float("nan"), dtype=torch.float32, device=DEV)
+        tuned().gemm_swiglu(rows, Wgu, act, Rt())
+        gr, ur = normed @ gate.double().T, normed @ up.double().T
+        ref_act = gr / (1 + torch.exp(-gr)) * ur
+        assert (act.double() - ref_act).abs().max() < 1e-2 * ref_act.abs().max()
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     from flambeau_amd.kernels import KernelError
     from flambeau_amd.kernels.packing import pack_weight
@@ -138,6 +179,10 @@ def test_gemm_skinny_refuses_what_it_cannot_do():
                             torch.empty(65, 8, dtype=torch.float32, device=DEV))
     with pytest.raises(KernelError, match="packs to"):
         tuned().gemm_skinny(rnd(2, 64, dtype=torch.bfloat16), pack_weight(rnd(8, 32, dtype=torch.bfloat16)), out)
+    with pytest.raises(KernelError, match="at most 16 rows"):       # the fusions with the norm: one tile of tokens
+        tuned().gemm_skinny_residual(rnd(17, 64, dtype=torch.bfloat16), pack_weight(rnd(32, 64, dtype=torch.bfloat16)),
+                                     rnd(17, 32), rnd(32), torch.empty(17, 32, dtype=torch.bfloat16, device=DEV),
+                                     torch.empty(17, 2, dtype=torch.float32, device=DEV), 1e-5)
 
 
 # ---------------------------------------------------------------- cache, rotation, attention

@@ -24,6 +24,12 @@ def rnd(*shape, scale=1.0, seed=0):
     return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
 
 
+def delta_of(rt, result):
+    """What a mixer or feed-forward returned, as the delta tensor."""
+    from flambeau_amd.parts import Product
+    return result.compute(rt) if isinstance(result, Product) else result
+
+
 def tol(dtype):
     return 2e-5 if dtype == torch.float32 else 2e-2
 
@@ -89,7 +95,7 @@ def test_swiglu_part(dtype, tuned, n):
     w = {k: rnd(*v.shape, scale=0.2, seed=i).to(dtype) for i, (k, v) in enumerate(ffn.tensors().items())}
     ffn.bind({k: put(rt, v) for k, v in w.items()}, rt)
     x = rnd(n, H, seed=9).to(dtype)
-    got = ffn.forward(x.to(DEV), None)
+    got = delta_of(rt, ffn.forward(x.to(DEV), None))
     assert got.dtype == torch.float32
     want = pm.swiglu_mlp(x.double().numpy(), *(w[k].double().numpy() for k in ("gate.weight", "up.weight", "down.weight")))
     assert np.abs(got.double().cpu().numpy() - want).max() < tol(dtype) * np.abs(want).max()
@@ -145,7 +151,7 @@ def test_attention_mixer_part(dtype, tuned, nh, nkv, hd, window, theta, ps):
         got, at = [], 0
         for k in cuts:
             step = step_for(rt, [(at, k)], ps, 32, shuffle_seed=1)       # same seed: the same pages every step
-            got.append(mixer.forward(x[at:at + k].to(DEV).contiguous(), step, store.entries[0]).double().cpu().numpy())
+            got.append(delta_of(rt, mixer.forward(x[at:at + k].to(DEV).contiguous(), step, store.entries[0])).double().cpu().numpy())
             at += k
         got = np.concatenate(got)
         assert np.abs(got - want).max() < tol(dtype) * np.abs(want).max(), cuts
