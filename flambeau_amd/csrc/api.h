@@ -61,8 +61,7 @@ int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspa
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_tiled_splits(int M, int N, int K);
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
-                   const int* items, int n_items, const int* positions, const int* tok_seq,
-                   const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
+                   const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
                    int n_pages, float scale, int window, int n_split, hipStream_t stream);
 int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int* tiles, int n_tiles,
                     const int* positions, const int* block_table, int max_blocks, int nh, int nkv,

@@ -1,8 +1,9 @@
 // Split-K grouped-query attention over the paged cache for single query rows (decode rows, and
 // the rows of short prompt portions): bf16 storage, float arithmetic, matrix cores.
 //
-// Work item = (query row, kv head, split).  A block of four waves handles the (up to 16) query
-// heads that share one kv head over the keys of its split, 32 keys per wave at a time:
+// Work item = (query row, kv head, split); a query row comes as (row, position, request, 0).  A
+// block of four waves handles the (up to 16) query heads that share one kv head over the keys of
+// its split, 32 keys per wave at a time:
 //
 //   S^T[key][head] = K[key][:] . Q[head][:]     v_mfma_f32_16x16x32_bf16, A = K rows read
 //                                               straight from the cache pages (head dims are
@@ -16,6 +17,8 @@
 //
 // The four waves' states are merged through LDS; with more than one split the block writes a
 // partial (max, sum, O) and a second kernel merges the splits (same rule: exp(m_c - m_max)).
+// (Merging in the block that finishes last was tried and is far slower here: it needs a
+// device-wide release fence in every block, which writes the L2 back, one block after the other.)
 // Which keys a row sees depends on its own position only: [max(0, p - window + 1), p].
 //
 // Reference: crates/kernels-hip/src/kernels/attention_decode_f16_paged.cu:49-158 (paged decode),
@@ -26,26 +29,28 @@
 #define DEC_WAVES 4
 #define DEC_CHUNK 32
 
+// items[i] = (row of q and out, position, request, 0): everything a block needs to find its keys
+// comes with one load.
 template <int HDP>
-__global__ __launch_bounds__(256) void attn_decode_kernel(
-    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, PagedCache cache, const int* __restrict__ items,
-    const int* __restrict__ positions, const int* __restrict__ tok_seq,
+__global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* part_o,
+    float* part_ml, PagedCache cache, const int4* __restrict__ items,
     const int* __restrict__ block_table, int max_blocks, int nh, float scale, int window,
-    int n_split, int q_tiles) {
+    int n_split, int q_tiles, int ps_shift) {
     constexpr int QS = HDP / 32;     // k-steps of the score product
     constexpr int DT = HDP / 16;     // 16-wide tiles of head dims in the output
+    constexpr bool PIPELINED = HDP <= 128;       // two chunks of keys and values fit the registers
     __shared__ float s_m[DEC_WAVES][16], s_l[DEC_WAVES][16];
     __shared__ f32x4 s_o[DEC_WAVES - 1][DT][64];     // wave 0 keeps its own in registers
 
     const int item = blockIdx.x;
     const int kvh = blockIdx.y / q_tiles, qt = blockIdx.y % q_tiles;
     const int split = blockIdx.z;
-    const int token = items[item];
+    const int4 it = items[item];
+    const int token = it.x, p = it.y;
     const int hd = cache.head_dim, ps = cache.page_size;
     const int G = nh / cache.n_kv_heads;
-    const int p = positions[token];
-    const int* table = block_table + (size_t)tok_seq[token] * max_blocks;
+    const int* table = block_table + (size_t)it.z * max_blocks;
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int li = lane & 15, g = lane >> 4;
@@ -72,44 +77,53 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     for (int t = 0; t < DT; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int c = c0 + wave; c < c1; c += DEC_WAVES) {
-        const int t0 = c * DEC_CHUNK;
-        // ---- scores of two 16-key tiles.  Row i of tile a is key t0 + 8 (i / 4) + i % 4, of tile b
-        // the same + 4: a lane (head, g) of the accumulators then owns the 8 consecutive keys
-        // t0 + 8 g .. + 7, one 16-byte run of a row of the transposed values
-        f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-        {
-            const int ka = t0 + 8 * (li >> 2) + (li & 3), kb = ka + 4;
-            const int pa = (ka <= p && ka >= lo) ? table[ka / ps] : -1;
-            const int pb = (kb <= p && kb >= lo) ? table[kb / ps] : -1;
-            const bool oka = pa >= 0 && pa < cache.n_pages, okb = pb >= 0 && pb < cache.n_pages;
-            const bf16_t* rowa = kv + cache_k_offset(cache, oka ? pa : 0, kvh, ka % ps, 0);
-            const bf16_t* rowb = kv + cache_k_offset(cache, okb ? pb : 0, kvh, kb % ps, 0);
-            bf16x8 xa[QS], xb[QS];
+    // Row i of score tile a is key t0 + 8 (i / 4) + i % 4, of tile b the same + 4: a lane (head, g)
+    // of the accumulators then owns the 8 consecutive keys t0 + 8 g .. + 7, one 16-byte run of a
+    // row of the transposed values.  The two keys of a lane lie in one page (pages hold multiples of 8).
+    const int k_off = 8 * (li >> 2) + (li & 3), v_off = 8 * g;
+    struct Chunk { bf16x8 xa[QS], xb[QS], wv[DT]; };
+    auto page_of = [&](int key) { return ps_shift >= 0 ? key >> ps_shift : key / ps; };
+    auto row_of = [&](int key) { return ps_shift >= 0 ? key & (ps - 1) : key % ps; };
+    // Loads carry no conditions (a branch around a load would make every wait a wait for all loads
+    // in flight): keys outside [lo, p] are clamped into it, page ids outside the pool to a page of
+    // the pool, chunks beyond the split to its last chunk; what such a load brings is masked in
+    // compute().  Pages of chunk c for this lane: of its two keys and of its eight values.
+    const int c_last = c1 - 1;
+    auto page_ids = [&](int c, int& pk, int& pv) {
+        c = min(c, c_last);
+        const int ka = min(max(c * DEC_CHUNK + k_off, lo), p), vk = min(max(c * DEC_CHUNK + v_off, lo), p);
+        pk = table[page_of(ka)];
+        pv = table[page_of(vk)];
+    };
+    auto load_chunk = [&](Chunk& f, int c, int pk, int pv) {
+        c = min(c, c_last);
+        const int ka = c * DEC_CHUNK + k_off, vk = c * DEC_CHUNK + v_off;
+        pk = (int)min((unsigned)pk, (unsigned)cache.n_pages - 1u);
+        pv = (int)min((unsigned)pv, (unsigned)cache.n_pages - 1u);
+        const bf16_t* rowa = kv + cache_k_offset(cache, pk, kvh, row_of(ka), 0);
+        const bf16_t* rowb = rowa + 4 * hd;          // key ka + 4: the same page
 #pragma unroll
-            for (int s = 0; s < QS; ++s) {
-                const int d = 32 * s + 8 * g;
-                const bool din = d + 8 <= hd;
-                xa[s] = (oka && din) ? *(const bf16x8*)(rowa + d) : zero8;
-                xb[s] = (okb && din) ? *(const bf16x8*)(rowb + d) : zero8;
-            }
-#pragma unroll
-            for (int s = 0; s < QS; ++s) {
-                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[s], qreg[s], sa, 0, 0, 0);
-                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[s], sb, 0, 0, 0);
-            }
+        for (int s = 0; s < QS; ++s) {
+            const int d = min(32 * s + 8 * g, hd - 8);       // head dims beyond hd: q is zero there
+            f.xa[s] = *(const bf16x8*)(rowa + d);
+            f.xb[s] = *(const bf16x8*)(rowb + d);
         }
-        // ---- values: lane (dim li of tile t, group g) reads the keys t0 + 8 g .. + 7 of its dim
-        const int vk = t0 + 8 * g;
-        const int pv = (vk <= p && vk + 7 >= lo) ? table[vk / ps] : -1;
-        const bool okv = pv >= 0 && pv < cache.n_pages;
-        bf16x8 wv[DT];
+        const bf16_t* vrow = kv + cache_v_offset(cache, pv, kvh, row_of(vk), 0);
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
-            const int d = 16 * t + li;
-            wv[t] = (okv && d < hd) ? *(const bf16x8*)(kv + cache_v_offset(cache, pv, kvh, vk % ps, d)) : zero8;
+            const int d = min(16 * t + li, hd - 1);          // rows beyond hd are never stored
+            f.wv[t] = *(const bf16x8*)(vrow + (size_t)d * ps);
         }
-        // ---- online softmax; this lane holds keys t0 + 8 g + r (tile a) and + 4 + r (tile b) for head li
+    };
+    auto compute = [&](const Chunk& f, int c) {
+        const int t0 = c * DEC_CHUNK;
+        f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < QS; ++s) {
+            sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.xa[s], qreg[s], sa, 0, 0, 0);
+            sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.xb[s], qreg[s], sb, 0, 0, 0);
+        }
+        // online softmax; this lane holds keys t0 + 8 g + r (tile a) and + 4 + r (tile b) for head li
         float mt = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -133,10 +147,65 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         }
         l = l * corr + ls;
         m = m_new;
+        if (t0 < lo || t0 + DEC_CHUNK - 1 > p) {
+            // a chunk at an end of the range: values of keys outside it (whatever the page holds
+            // there) are zeroed, since 0 * NaN would not be 0
+            u32x4 keep;
 #pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            o[t] *= corr;
-            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[t], pb8, o[t], 0, 0, 0);
+            for (int e = 0; e < 4; ++e) {
+                const int k0 = t0 + 8 * g + 2 * e;
+                keep[e] = ((k0 >= lo && k0 <= p) ? 0x0000FFFFu : 0u) | ((k0 + 1 >= lo && k0 + 1 <= p) ? 0xFFFF0000u : 0u);
+            }
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                o[t] *= corr;
+                const u32x4 v = __builtin_bit_cast(u32x4, f.wv[t]) & keep;
+                o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb8, o[t], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                o[t] *= corr;
+                o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.wv[t], pb8, o[t], 0, 0, 0);
+            }
+        }
+    };
+
+    // The wave's chunks are c0 + wave, + 4, ...  What bounds a short split is the chain page id ->
+    // key and value loads -> arithmetic, so the chain is pipelined: page ids two chunks ahead, keys
+    // and values one chunk ahead, in two register sets that swap roles.  The loop body has no
+    // branch, so the compiler's count of the loads in flight is exact.
+    int c = c0 + wave;
+    if (c < c1) {
+        if (PIPELINED) {
+            Chunk fa, fb;
+            int pk0, pv0, pk1, pv1;
+            page_ids(c, pk0, pv0);
+            page_ids(c + DEC_WAVES, pk1, pv1);
+            load_chunk(fa, c, pk0, pv0);
+            for (; c + 2 * DEC_WAVES < c1; c += 2 * DEC_WAVES) {
+                page_ids(c + 2 * DEC_WAVES, pk0, pv0);
+                load_chunk(fb, c + DEC_WAVES, pk1, pv1);
+                compute(fa, c);
+                page_ids(c + 3 * DEC_WAVES, pk1, pv1);
+                load_chunk(fa, c + 2 * DEC_WAVES, pk0, pv0);
+                compute(fb, c + DEC_WAVES);
+            }
+            if (c + DEC_WAVES < c1) {               // two chunks left
+                load_chunk(fb, c + DEC_WAVES, pk1, pv1);
+                compute(fa, c);
+                compute(fb, c + DEC_WAVES);
+            } else {
+                compute(fa, c);
+            }
+        } else {
+            Chunk f;
+            for (; c < c1; c += DEC_WAVES) {
+                int pk, pv;
+                page_ids(c, pk, pv);
+                load_chunk(f, c, pk, pv);
+                compute(f, c);
+            }
         }
     }
     // sum over the four key groups of a head
@@ -150,42 +219,42 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         for (int t = 0; t < DT; ++t) s_o[wave - 1][t][lane] = o[t];
     }
     __syncthreads();
-    if (wave != 0) return;
-    float mm = -INFINITY;
+    if (wave == 0) {
+        float mm = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) mm = fmaxf(mm, s_m[w][li]);
-    float f[DEC_WAVES], ll = 0.f;
+        for (int w = 0; w < DEC_WAVES; ++w) mm = fmaxf(mm, s_m[w][li]);
+        float f[DEC_WAVES], ll = 0.f;
 #pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) {
-        f[w] = s_m[w][li] == -INFINITY ? 0.f : expf(s_m[w][li] - mm);
-        ll += s_l[w][li] * f[w];
-    }
-    if (!head_ok) return;
-    // lane (head li, group g) holds dims 16 t + 4 g + r
-    if (n_split == 1) {
-        const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-        bf16_t* orow = out + ((size_t)token * nh + head) * hd;
-#pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            f32x4 acc = o[t] * f[0];
-#pragma unroll
-            for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w - 1][t][lane] * f[w];
-            const int d = 16 * t + 4 * g;
-            if (d + 4 <= hd) {
-                bf16x4 ov = {(bf16_t)(acc[0] * inv), (bf16_t)(acc[1] * inv), (bf16_t)(acc[2] * inv), (bf16_t)(acc[3] * inv)};
-                *(bf16x4*)(orow + d) = ov;
-            }
+        for (int w = 0; w < DEC_WAVES; ++w) {
+            f[w] = s_m[w][li] == -INFINITY ? 0.f : expf(s_m[w][li] - mm);
+            ll += s_l[w][li] * f[w];
         }
-    } else {
-        const size_t slot = ((size_t)item * nh + head) * n_split + split;
-        if (g == 0) { part_ml[slot * 2] = mm; part_ml[slot * 2 + 1] = ll; }
-        float* prow = part_o + slot * HDP;
+        // lane (head li, group g) holds dims 16 t + 4 g + r
+        if (head_ok && n_split == 1) {
+            const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+            bf16_t* orow = out + ((size_t)token * nh + head) * hd;
 #pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            f32x4 acc = o[t] * f[0];
+            for (int t = 0; t < DT; ++t) {
+                f32x4 acc = o[t] * f[0];
 #pragma unroll
-            for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w - 1][t][lane] * f[w];
-            *(f32x4*)(prow + 16 * t + 4 * g) = acc;
+                for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w - 1][t][lane] * f[w];
+                const int d = 16 * t + 4 * g;
+                if (d + 4 <= hd) {
+                    bf16x4 ov = {(bf16_t)(acc[0] * inv), (bf16_t)(acc[1] * inv), (bf16_t)(acc[2] * inv), (bf16_t)(acc[3] * inv)};
+                    *(bf16x4*)(orow + d) = ov;
+                }
+            }
+        } else if (head_ok) {
+            const size_t slot = ((size_t)item * nh + head) * n_split + split;
+            if (g == 0) { part_ml[slot * 2] = mm; part_ml[slot * 2 + 1] = ll; }
+            float* prow = part_o + slot * HDP;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                f32x4 acc = o[t] * f[0];
+#pragma unroll
+                for (int w = 1; w < DEC_WAVES; ++w) acc += s_o[w - 1][t][lane] * f[w];
+                *(f32x4*)(prow + 16 * t + 4 * g) = acc;
+            }
         }
     }
 }
@@ -196,12 +265,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __restrict__ part_o,
                                                                 const float* __restrict__ part_ml,
                                                                 bf16_t* __restrict__ out,
-                                                                const int* __restrict__ items, int nh,
+                                                                const int4* __restrict__ items, int nh,
                                                                 int hd, int hdp, int n_split) {
     __shared__ float s_f[256];       // exp(m_s - m_max) per split (n_split <= 256)
     __shared__ float s_inv;
     const int item = blockIdx.x, head = blockIdx.y;
-    const int token = items[item];
+    const int token = items[item].x;
     const size_t base = ((size_t)item * nh + head) * n_split;
     const int t = threadIdx.x;
     float ms = -INFINITY, ls = 0.f;
@@ -251,8 +320,7 @@ extern "C" int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split
 }
 
 extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml,
-                              const void* cache_base, const int* items, int n_items,
-                              const int* positions, const int* tok_seq, const int* block_table,
+                              const void* cache_base, const int* items, int n_items, const int* block_table,
                               int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
                               float scale, int window, int n_split, hipStream_t stream) {
     FL_CHECK(n_items >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_decode: bad head counts %d/%d", nh, nkv);
@@ -261,16 +329,20 @@ extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* pa
     FL_CHECK(n_split >= 1 && n_split <= 256, "attn_decode: %d splits", n_split);
     FL_CHECK(n_split == 1 || (part_o && part_ml), "attn_decode: splits need a workspace");
     FL_CHECK(window >= 0, "attn_decode: negative window");
+    FL_CHECK((uintptr_t)items % 16 == 0, "attn_decode: the items must be 16-byte aligned");
     if (n_items == 0) return 0;
+    int ps_shift = -1;
+    if ((page_size & (page_size - 1)) == 0)
+        for (ps_shift = 0; (1 << ps_shift) < page_size; ++ps_shift) {}
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
     const int G = nh / nkv;
     const int q_tiles = ceil_div(G, 16);
     dim3 grid(n_items, nkv * q_tiles, n_split);
     const int hdp = ceil_div(hd, 32) * 32;
 #define FL_DEC(HDP_)                                                                                  \
-    attn_decode_kernel<HDP_><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, part_ml, c, items, \
-                                                       positions, tok_seq, block_table, max_blocks, nh, scale,   \
-                                                       window, n_split, q_tiles)
+    attn_decode_kernel<HDP_><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, part_ml, c,       \
+                                                       (const int4*)items, block_table, max_blocks, nh, scale,   \
+                                                       window, n_split, q_tiles, ps_shift)
     switch (hdp) {
         case 32: FL_DEC(32); break;
         case 64: FL_DEC(64); break;
@@ -286,7 +358,7 @@ extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* pa
     if (n_split > 1) {
         dim3 mg(n_items, nh);
         attn_decode_merge_kernel<<<mg, 256, 0, stream>>>(
-            part_o, part_ml, (bf16_t*)out, items, nh, hd, hdp, n_split);
+            part_o, part_ml, (bf16_t*)out, (const int4*)items, nh, hd, hdp, n_split);
         FL_LAUNCH_CHECK();
     }
     return 0;

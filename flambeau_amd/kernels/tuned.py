@@ -23,7 +23,7 @@ register_signatures({
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
-    "fl_attn_decode": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+    "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
 })
 
 SKINNY_MAX_ROWS = 64     # rows the decode kernels take
@@ -234,26 +234,26 @@ def prepare_gate_up(gate: torch.Tensor, up: torch.Tensor) -> Weight:
 # Rows of portions up to this length are treated as single query rows by the split-K kernel;
 # longer portions go to the tiled prefill kernel.
 SHORT_PORTION = 8
-DECODE_TARGET_BLOCKS = 1024
-DECODE_MIN_KEYS_PER_SPLIT = 256
+DECODE_TARGET_BLOCKS = 512           # two blocks per compute unit (measured best at 1, 8 and 64 rows)
+DECODE_MIN_KEYS_PER_SPLIT = 128
 
 
 PREFILL_TILE = 64        # query tokens per block of the tiled kernel
 
 
 def attention_metadata(batch) -> dict:
-    """Work lists for the attention kernels of one batch: ``attn_rows`` = the rows that run as
-    single queries (decode rows and rows of short portions); ``attn_tiles`` = (request, first
-    row, rows) for every 64 rows of the longer portions."""
+    """Work lists for the attention kernels of one batch: ``attn_rows`` = (row, position, request,
+    0) of the rows that run as single queries (decode rows and rows of short portions);
+    ``attn_tiles`` = (request, first row, rows) for every 64 rows of the longer portions."""
     import numpy as np
     rows, tiles = [], []
-    for s, (q0, ql) in enumerate(zip(batch.q_starts, batch.q_lens)):
+    for s, (q0, ql, p0) in enumerate(zip(batch.q_starts, batch.q_lens, batch.start_pos)):
         if ql <= SHORT_PORTION:
-            rows += range(q0, q0 + ql)
+            rows += [(q0 + i, p0 + i, s, 0) for i in range(ql)]
         else:
             for off in range(0, ql, PREFILL_TILE):
                 tiles.append((s, q0 + off, min(PREFILL_TILE, ql - off)))
-    return {"attn_rows": np.asarray(rows, dtype=np.int32),
+    return {"attn_rows": np.asarray(rows, dtype=np.int32).reshape(-1, 4),
             "attn_tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 3)}
 
 
@@ -266,8 +266,9 @@ def decode_splits(n_items: int, n_kv_heads: int, group: int, max_ctx: int) -> in
     return int(min(by_blocks, by_keys, 64))
 
 
-def attn_decode(q, out, cache, rows, positions, tok_seq, table, n_heads, scale, window, n_split, part_o=None,
-                part_ml=None):
+def attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, part_o=None, part_ml=None):
+    """Attention of single query rows; ``rows[i] = (row of q and out, position, index of the request's
+    row in ``table``, 0)``."""
     n = q.shape[0]
     hd = cache.head_dim
     n_items = rows.shape[0]
@@ -280,8 +281,7 @@ def attn_decode(q, out, cache, rows, positions, tok_seq, table, n_heads, scale, 
          _check(out, "attn.out", torch.bfloat16, (n, n_heads * hd)),
          _check(part_o, "attn.part_o", torch.float32) if part_o is not None else None,
          _check(part_ml, "attn.part_ml", torch.float32) if part_ml is not None else None,
-         _check(cache.pool, "attn.cache", torch.bfloat16), _check(rows, "attn.rows", torch.int32, (n_items,)), n_items,
-         _check(positions, "attn.positions", torch.int32, (n,)), _check(tok_seq, "attn.tok_seq", torch.int32, (n,)),
+         _check(cache.pool, "attn.cache", torch.bfloat16), _check(rows, "attn.rows", torch.int32, (n_items, 4)), n_items,
          _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads,
          hd, cache.page_size, cache.n_pages, float(scale), int(window), int(n_split), stream_handle())
     return out
@@ -336,6 +336,5 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
             cap = slots if batch.ctx_bound else max(slots, 4096 * n_heads)     # a fixed-shape step never grows
             part_o = rt.buffer("attn_part_o", slots, hdp, torch.float32, max_rows=cap)
             part_ml = rt.buffer("attn_part_ml", slots, 2, torch.float32, max_rows=cap)
-        attn_decode(q, out, cache, rows, step.positions, step.tok_seq, table, n_heads, scale, window,
-                    n_split, part_o, part_ml)
+        attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, part_o, part_ml)
     return out

@@ -377,6 +377,12 @@ def test_sample_is_the_inverse_cdf_in_index_order(V):
 
 
 # ---------------------------------------------------------------- tuned attention for single rows
+def decode_rows(case, picked):
+    """(row, position, request, 0) of the picked rows, as the decode kernel wants them."""
+    pos, seq = case["pos_d"].cpu().tolist(), case["seq_d"].cpu().tolist()
+    return torch.tensor([[r, pos[r], seq[r], 0] for r in picked], dtype=torch.int32, device=DEV).reshape(-1, 4)
+
+
 @pytest.mark.parametrize("n_split", [1, 2, 5])
 @pytest.mark.parametrize("nh,nkv,hd,ps,window", [(32, 8, 128, 16, 0), (4, 2, 16, 8, 16), (6, 1, 24, 16, 0),
                                                 (5, 5, 32, 16, 24), (20, 1, 64, 8, 0), (8, 4, 256, 32, 100),
@@ -387,13 +393,12 @@ def test_attn_decode_against_plain_and_reference(nh, nkv, hd, ps, window, n_spli
     n = case["n"]
     scale = 1 / math.sqrt(hd)
     q2 = case["q"].reshape(n, nh * hd)
-    rows = torch.arange(n, dtype=torch.int32, device=DEV).flip(0).contiguous()      # any order of rows
+    rows = decode_rows(case, reversed(range(n)))      # any order of rows
     out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     hdp = -(-hd // 32) * 32
     part_o = torch.empty(n * nh * n_split * hdp, dtype=torch.float32, device=DEV)
     part_ml = torch.empty(n * nh * n_split * 2, dtype=torch.float32, device=DEV)
-    tuned().attn_decode(q2, out, case["cache"], rows, case["pos_d"], case["seq_d"], case["table"], nh, scale,
-                        window, n_split, part_o, part_ml)
+    tuned().attn_decode(q2, out, case["cache"], rows, case["table"], nh, scale, window, n_split, part_o, part_ml)
     plain = torch.empty_like(out)
     ops().attn_plain(q2, plain, case["cache"], case["pos_d"], case["seq_d"], case["table"], nh, scale, window)
     ref = attention_case_ref(case, scale, window)
@@ -408,8 +413,7 @@ def test_attn_decode_subset_of_rows_leaves_the_others_alone():
     n = case["n"]
     q2 = case["q"].reshape(n, nh * hd)
     out = torch.full((n, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
-    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
-    tuned().attn_decode(q2, out, case["cache"], rows, case["pos_d"], case["seq_d"], case["table"], nh, 0.125, 0, 1)
+    tuned().attn_decode(q2, out, case["cache"], decode_rows(case, [4, 1]), case["table"], nh, 0.125, 0, 1)
     ref = attention_case_ref(case, 0.125, 0)
     assert (out[[0, 2, 3]] == 7.0).all()
     assert (out[[1, 4]].double().reshape(2, nh, hd) - ref[[1, 4]]).abs().max() < 1e-2 * ref.abs().max()
