@@ -4,9 +4,9 @@
 //  * w arrives packed (kernels/packing.py): a tile of 16 features x 32 k is 1 KB in lane order.
 //    Operand tiles of both matrices go from memory straight into LDS with
 //    global_load_lds_dwordx4 (no staging registers, no ds_write): for w a wave copies the tile as
-//    it lies; for the row-major x every lane reads the 16 bytes that the tile layout wants at its
-//    place.  A wave then reads an operand from LDS with one ds_read_b128 per lane at consecutive
-//    addresses (no bank conflicts, no transposition);
+//    it lies; of the row-major x a wave copies 16 rows of 64 bytes, four lanes per row.  A wave
+//    then reads an operand from LDS with one ds_read_b128 per lane (w at consecutive addresses, x
+//    through an exchange of pieces that keeps the banks apart);
 //  * LDS is a ring of NS stages of one k-step (32 values of k); one bare s_barrier per stage;
 //  * the w tile is the A operand and the x tile the B operand: C[feature][token] leaves each
 //    lane with four consecutive features of one token, one 16-byte store;
@@ -46,21 +46,32 @@ template <> __device__ __forceinline__ void tg_store4<bf16_t>(bf16_t* p, f32x4 v
 //     stage i - 1 just left; read the operands of stage i from LDS; FT * TT products.
 // Nothing is zero-filled: rows beyond M and feature groups beyond N are clamped to valid ones (their
 // results are never stored), and k beyond K meets the zero padding of the packed w.
-template <int FT, int TT, int NS, int OCC, typename TOut, bool SWIGLU>
-__global__ __launch_bounds__(256, OCC) void gemm_async_kernel(const bf16_t* __restrict__ x,
+template <int FT, int TT, int WT, int NS, int OCC, typename TOut, bool SWIGLU, bool KWHOLE>
+__global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t* __restrict__ x,
                                                             const bf16_t* __restrict__ wp,
                                                             TOut* __restrict__ out, int M, int N, int K,
                                                             int n_steps, int steps_per_split, int out_cols) {
-    constexpr int NTF = 2 * FT, NTT = 2 * TT;         // operand tiles of the block: features, tokens
+    constexpr int NW = 2 * WT;                        // waves: 2 along the features, WT along the tokens
+    constexpr int NTF = 2 * FT, NTT = WT * TT;        // operand tiles of the block: features, tokens
     constexpr int TILES = NTF + NTT;                  // 1 KB tiles per stage
-    constexpr int LPS = TILES / 4;                    // load instructions per wave and stage
-    static_assert(TILES % 4 == 0, "tiles must divide among four waves");
+    constexpr int LPS = TILES / NW;                   // load instructions per wave and stage
+    static_assert(TILES % NW == 0, "tiles must divide among the waves");
     extern __shared__ __attribute__((aligned(16))) bf16_t ring[];      // [NS][TILES][512]
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wf = wave & 1, wt = wave >> 1;
-    const int m0 = blockIdx.y * (NTT * 16), n0 = blockIdx.x * (NTF * 16);
+    // Which tile: blocks go to the eight dies of the chip in turn (block b to die b % 8), each die
+    // with an L2 of its own.  A die gets one contiguous eighth of the tiles, ordered in groups of 8
+    // feature tiles by all token tiles, so that the blocks it runs at one time share rows of w and x.
+    const int n_ft = (N + NTF * 16 - 1) / (NTF * 16), n_tt = (M + NTT * 16 - 1) / (NTT * 16);
+    const int total = n_ft * n_tt, per_die = (total + 7) >> 3;
+    const int lin = (blockIdx.x & 7) * per_die + (blockIdx.x >> 3);
+    if (lin >= total) return;
+    const int grp = lin / (8 * n_tt), within = lin - grp * (8 * n_tt);
+    const int gf = min(8, n_ft - grp * 8);
+    const int tile_f = grp * 8 + within % gf, tile_t = within / gf;
+    const int m0 = tile_t * (NTT * 16), n0 = tile_f * (NTF * 16);
     const int n_groups = (N + 15) >> 4;
     const int s_begin = blockIdx.z * steps_per_split;
     const int s_end = min(n_steps, s_begin + steps_per_split);
@@ -72,36 +83,49 @@ __global__ __launch_bounds__(256, OCC) void gemm_async_kernel(const bf16_t* __re
 #pragma unroll
         for (int b = 0; b < TT; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // per-lane source addresses of this wave's tiles at k-step 0 (tile t = wave + 4 u)
-    const bf16_t* src[LPS];
-    int kstride[LPS];                                 // values to advance per k-step
+    // per-lane source addresses of this wave's tiles at the next stage to load; a wave copies LW
+    // tiles of w and LX tiles of x per stage
+    constexpr int LW = NTF / NW, LX = NTT / NW;
+    static_assert(NTF % NW == 0 && NTT % NW == 0, "tiles must divide among the waves");
+    const bf16_t* wsrc[LW];
+    const bf16_t* xsrc[LX];
 #pragma unroll
-    for (int u = 0; u < LPS; ++u) {
-        const int t = wave + 4 * u;
-        if (t < NTF) {
-            const int gg = min((n0 >> 4) + t, n_groups - 1);
-            src[u] = wp + (((size_t)gg * n_steps) * 64 + lane) * 8;
-            kstride[u] = 512;
-        } else {
-            const int row = min(m0 + (t - NTF) * 16 + (lane & 15), M - 1);
-            src[u] = x + (size_t)row * K + 8 * (lane >> 4);
-            kstride[u] = 32;
-        }
+    for (int u = 0; u < LW; ++u) {
+        const int gg = min((n0 >> 4) + wave * LW + u, n_groups - 1);
+        wsrc[u] = wp + (((size_t)gg * n_steps + s_begin) * 64 + lane) * 8;
+    }
+    // x: the four lanes of a quad read 64 consecutive bytes of one row (a quad that spreads over four
+    // rows costs four cache lookups instead of one: measured 15 against 37 bytes per clock and CU).
+    // The tile then lies row by row in LDS; the 16-byte pieces of a row are exchanged by
+    // (row / 2) % 4, with which the operand reads below meet no bank twice (measured: 4.3 clocks per
+    // read instruction against 8.2 without or with other exchanges).
+    const int x_piece = 8 * ((lane & 3) ^ ((lane >> 3) & 3));
+#pragma unroll
+    for (int u = 0; u < LX; ++u) {
+        const int row = min(m0 + (wave * LX + u) * 16 + (lane >> 2), M - 1);
+        xsrc[u] = x + (size_t)row * K + (size_t)s_begin * 32 + x_piece;
     }
     const int x_kmax = K - 8;                         // last whole 16-byte chunk of a row of x
+    // operand lane (token i = lane % 16, k-piece g = lane / 16) finds its 16 bytes of an x tile here
+    const int x_read = 32 * (lane & 15) + 8 * ((lane >> 4) ^ (((lane & 15) >> 1) & 3));
     auto issue = [&](int i) {                         // loads of stage i (k-step s_begin + i) into slot i % NS
-        const int s = s_begin + i;
         bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
 #pragma unroll
-        for (int u = 0; u < LPS; ++u) {
-            const int t = wave + 4 * u;
-            const bf16_t* g = src[u] + (size_t)s * kstride[u];
-            if (t >= NTF) {                           // x: keep the chunk inside the row
-                const int k = s * 32 + 8 * (lane >> 4);
+        for (int u = 0; u < LW; ++u) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)wsrc[u],
+                                             (__attribute__((address_space(3))) void*)(slot + (wave * LW + u) * 512), 16, 0, 0);
+            wsrc[u] += 512;
+        }
+#pragma unroll
+        for (int u = 0; u < LX; ++u) {
+            const bf16_t* g = xsrc[u];
+            if (!KWHOLE) {                            // K is no multiple of 32: keep the last pieces inside the row
+                const int k = (s_begin + i) * 32 + x_piece;
                 if (k > x_kmax) g -= (k - x_kmax);
             }
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                             (__attribute__((address_space(3))) void*)(slot + t * 512), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(slot + (NTF + wave * LX + u) * 512), 16, 0, 0);
+            xsrc[u] += 32;
         }
     };
 
@@ -118,22 +142,22 @@ __global__ __launch_bounds__(256, OCC) void gemm_async_kernel(const bf16_t* __re
         // a bare barrier: __syncthreads() would add a fence that waits for ALL loads in flight,
         // also those of the later stages, and the ring would be one stage deep
         asm volatile("s_barrier" ::: "memory");
-        if (i + NS - 1 < n_iter) issue(i + NS - 1);
+        // the operand reads of this stage go first (x, then w in the order the products want them);
+        // the loads of a later stage are issued while they are on their way
         const bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
         bf16x8 a[FT], b[TT];
 #pragma unroll
-        for (int t = 0; t < FT; ++t) a[t] = *(const bf16x8*)(slot + (wf * FT + t) * 512 + lane * 8);
+        for (int t = 0; t < TT; ++t) b[t] = *(const bf16x8*)(slot + (NTF + wt * TT + t) * 512 + x_read);
 #pragma unroll
-        for (int t = 0; t < TT; ++t) b[t] = *(const bf16x8*)(slot + (NTF + wt * TT + t) * 512 + lane * 8);
+        for (int t = 0; t < FT; ++t) a[t] = *(const bf16x8*)(slot + (wf * FT + t) * 512 + lane * 8);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i + NS - 1 < n_iter) issue(i + NS - 1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ta = 0; ta < FT; ++ta)
 #pragma unroll
             for (int tb = 0; tb < TT; ++tb)
                 acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ta], b[tb], acc[ta][tb], 0, 0, 0);
-        // all operand reads first, then the products (the scheduler would otherwise wait for LDS
-        // once per pair of feature tiles)
-        __builtin_amdgcn_sched_group_barrier(0x100, FT + TT, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, FT * TT, 0);
     }
     // the loads are done (the last stage waited for vmcnt(0)); LDS is not touched again
 
@@ -186,18 +210,22 @@ __global__ __launch_bounds__(256, OCC) void gemm_async_kernel(const bf16_t* __re
     }
 }
 
-template <int FT, int TT, int NS, int OCC, typename TOut, bool SWIGLU>
+template <int FT, int TT, int WT, int NS, int OCC, typename TOut, bool SWIGLU>
 static void launch_async(int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N,
                          int K, int n_steps, int per, int out_cols) {
-    constexpr int LDS = NS * (2 * FT + 2 * TT) * 1024;
+    constexpr int LDS = NS * (2 * FT + WT * TT) * 1024;
     static bool configured = false;
-    auto kern = gemm_async_kernel<FT, TT, NS, OCC, TOut, SWIGLU>;
+    auto whole = gemm_async_kernel<FT, TT, WT, NS, OCC, TOut, SWIGLU, true>;
+    auto ragged = gemm_async_kernel<FT, TT, WT, NS, OCC, TOut, SWIGLU, false>;
     if (!configured) {
-        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        (void)hipFuncSetAttribute((const void*)whole, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        (void)hipFuncSetAttribute((const void*)ragged, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         configured = true;
     }
-    dim3 grid(ceil_div(N, 2 * FT * 16), ceil_div(M, 2 * TT * 16), splits);
-    kern<<<grid, 256, LDS, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols);
+    auto kern = (K % 32 == 0) ? whole : ragged;
+    const int tiles = ceil_div(N, 2 * FT * 16) * ceil_div(M, WT * TT * 16);
+    dim3 grid(ceil_div(tiles, 8) * 8, 1, splits);
+    kern<<<grid, 128 * WT, LDS, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols);
 }
 
 template <typename TOut>
@@ -211,18 +239,24 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     out[i] = from_f32<TOut>(s);
 }
 
-// Shape of the block tile: 0 = chosen from the sizes, 1 = 128 x 128, 2 = 256 x 128 (for experiments).
+// Shape of the block: 0 = chosen from the sizes; for experiments 1 = 128 x 128 (4 waves, ring of 4), 2 and 3 =
+// 256 x 128 (4 waves, ring of 2 and 3), 4 = 256 x 256 (8 waves, ring of 4), 6 = 128 x 256 (8 waves, ring of 4).
 static int g_tiled_variant = 0;
 extern "C" int fl_gemm_tiled_set_variant(int v) { g_tiled_variant = v; return 0; }
 
 template <typename TOut, bool SWIGLU>
 static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out,
                          int M, int N, int K, int n_steps, int per, int out_cols) {
-    if (variant == 0) variant = (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320) ? 2 : 1;
-    if (variant == 2)
-        launch_async<8, 4, 2, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols);
-    else
-        launch_async<4, 4, 4, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols);
+    // 256 features x 128 tokens with four waves, two blocks per compute unit, where that fills the
+    // chip; else 128 x 256 with eight waves, one block per compute unit
+    if (variant == 0) variant = (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320 || M < 192) ? 3 : 6;
+    switch (variant) {
+        case 1: launch_async<4, 4, 2, 4, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 2: launch_async<8, 4, 2, 2, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 4: launch_async<8, 4, 4, 4, 1, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 6: launch_async<4, 4, 4, 4, 1, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        default: launch_async<8, 4, 2, 3, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+    }
 }
 
 // How many ways K is split for a product of this shape: 1 if the grid fills the chip.
