@@ -11,8 +11,9 @@
 //
 // Everything is computed transposed, so that a query is a lane column:
 //   S^T[key][query] = K . Q^T        A = K tile (LDS, stored as matrix-core tiles), B = Q (registers)
-//   softmax per column: running max m and sum l live in the lanes that own the column; rescaling
-//       the output needs no broadcast and is skipped when no maximum moved
+//   softmax per column: the base m of the exponents and the sum l live in the lanes that own the
+//       column; rescaling the output needs no broadcast and happens only when a base moves, which
+//       it does lazily (when the maximum has run ahead of it by more than a factor of 256)
 //   O^T[d][query] += V^T . P^T       A = V^T tile (the cache stores values transposed inside a
 //       page, so its rows are runs of keys), B = P straight from the S^T accumulator
 // Scores are scaled by scale * log2(e) and exponentiated with exp2.  Query at position p sees keys
@@ -198,11 +199,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 }
                 mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m[t], mx);            // m holds raw (unscaled) maxima; scale > 0
+                // m holds the raw (unscaled) score that the exponents are taken against.  It follows
+                // the running maximum lazily: only when a chunk's maximum exceeds it by more than 8 in
+                // the exponent (a factor of 256, harmless in float) does the column move its base and
+                // rescale what it has summed.  With 64 columns per wave some running maximum moves
+                // in nearly every chunk, a base almost never after the first ones.  (-inf - -inf is
+                // NaN and compares false: a column without keys stays at -inf.)
+                const bool rebase = (mx - m[t]) * scale_log2e > 8.0f;
+                const float m_new = rebase ? mx : m[t];
                 // a column that has seen no key yet keeps m = -inf: use 0 as the base then
                 const float base = m_new == -INFINITY ? 0.f : m_new * scale_log2e;
-                corr[t] = __builtin_amdgcn_exp2f(fmaf(m[t], scale_log2e, -base));      // exp2(-inf) = 0
-                if (m_new != m[t]) moved = true;
+                corr[t] = rebase ? __builtin_amdgcn_exp2f(fmaf(m[t], scale_log2e, -base)) : 1.0f;      // exp2(-inf) = 0
+                if (rebase) moved = true;
                 float ls = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -215,7 +223,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 l[t] = l[t] * corr[t] + ls;
                 m[t] = m_new;
             }
-            // ---- rescale the output only if some maximum in the wave moved
+            // ---- rescale the output only if some base in the wave moved
             if (__any(moved)) {
 #pragma unroll
                 for (int t = 0; t < QT; ++t)

@@ -23,6 +23,7 @@
 //
 // The reference's nearest kernel multiplies a 64 x 8 tile per 64-thread block without matrix
 // cores (crates/kernels-hip/src/kernels/mmq_f16_tile.cu:33-107).
+#include <type_traits>
 #include "common.h"
 #include "api.h"
 
@@ -46,7 +47,7 @@ template <> __device__ __forceinline__ void tg_store4<bf16_t>(bf16_t* p, f32x4 v
 //     stage i - 1 just left; read the operands of stage i from LDS; FT * TT products.
 // Nothing is zero-filled: rows beyond M and feature groups beyond N are clamped to valid ones (their
 // results are never stored), and k beyond K meets the zero padding of the packed w.
-template <int FT, int TT, int WT, int NS, int OCC, typename TOut, bool SWIGLU, bool KWHOLE>
+template <int FT, int TT, int WT, int NS, int OCC, bool PIPE, typename TOut, bool SWIGLU, bool KWHOLE>
 __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t* __restrict__ x,
                                                             const bf16_t* __restrict__ wp,
                                                             TOut* __restrict__ out, int M, int N, int K,
@@ -132,32 +133,71 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
 #pragma unroll
     for (int i = 0; i < NS - 1; ++i)
         if (i < n_iter) issue(i);
-    for (int i = 0; i < n_iter; ++i) {
-        // my loads of stage i have landed when at most the later stages' are still in flight
-        if (i + NS - 2 < n_iter) {
-            __builtin_amdgcn_s_waitcnt(0xF70 | ((LPS * (NS - 2)) & 0xF) | ((((LPS * (NS - 2)) >> 4) & 3) << 14));
+    auto read_operands = [&](bf16x8 (&a)[FT], bf16x8 (&b)[TT], int i) {
+        const bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
+#pragma unroll
+        for (int t = 0; t < TT; ++t) b[t] = *(const bf16x8*)(slot + (NTF + wt * TT + t) * 512 + x_read);
+#pragma unroll
+        for (int t = 0; t < FT; ++t) a[t] = *(const bf16x8*)(slot + (wf * FT + t) * 512 + lane * 8);
+    };
+    auto products = [&](const bf16x8 (&a)[FT], const bf16x8 (&b)[TT]) {
+#pragma unroll
+        for (int ta = 0; ta < FT; ++ta)
+#pragma unroll
+            for (int tb = 0; tb < TT; ++tb)
+                acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ta], b[tb], acc[ta][tb], 0, 0, 0);
+    };
+    // my loads of stage j have landed when at most BEHIND later stages' are still in flight
+    auto wait_stage = [&](int j, auto behind) {
+        constexpr int N_LATER = LPS * decltype(behind)::value;
+        if (j + decltype(behind)::value < n_iter) {
+            __builtin_amdgcn_s_waitcnt(0xF70 | (N_LATER & 0xF) | (((N_LATER >> 4) & 3) << 14));
         } else {
             __builtin_amdgcn_s_waitcnt(0xF70);        // vmcnt(0)
         }
         // a bare barrier: __syncthreads() would add a fence that waits for ALL loads in flight,
         // also those of the later stages, and the ring would be one stage deep
         asm volatile("s_barrier" ::: "memory");
-        // the operand reads of this stage go first (x, then w in the order the products want them);
-        // the loads of a later stage are issued while they are on their way
-        const bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
-        bf16x8 a[FT], b[TT];
-#pragma unroll
-        for (int t = 0; t < TT; ++t) b[t] = *(const bf16x8*)(slot + (NTF + wt * TT + t) * 512 + x_read);
-#pragma unroll
-        for (int t = 0; t < FT; ++t) a[t] = *(const bf16x8*)(slot + (wf * FT + t) * 512 + lane * 8);
-        __builtin_amdgcn_sched_barrier(0);
-        if (i + NS - 1 < n_iter) issue(i + NS - 1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ta = 0; ta < FT; ++ta)
-#pragma unroll
-            for (int tb = 0; tb < TT; ++tb)
-                acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ta], b[tb], acc[ta][tb], 0, 0, 0);
+    };
+    using Behind1 = std::integral_constant<int, NS - 2>;       // reads follow the loads NS - 1 stages behind
+    using Behind2 = std::integral_constant<int, (NS >= 3 ? NS - 3 : 0)>;
+    if (PIPE) {
+        // The operands of stage i + 1 are read into a second set of registers while the products
+        // of stage i run: the matrix cores do not wait for LDS.  Loads run NS - 2 stages ahead of
+        // the reads.
+        bf16x8 a0[FT], b0[TT], a1[FT], b1[TT];
+        auto stage = [&](int i, bf16x8 (&ac)[FT], bf16x8 (&bc)[TT], bf16x8 (&an)[FT], bf16x8 (&bn)[TT]) {
+            if (i + 1 < n_iter) {
+                wait_stage(i + 1, Behind2{});
+                read_operands(an, bn, i + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + NS - 1 < n_iter) issue(i + NS - 1);
+            __builtin_amdgcn_sched_barrier(0);
+            products(ac, bc);
+        };
+        if (n_iter > 0) {
+            wait_stage(0, Behind1{});
+            read_operands(a0, b0, 0);
+        }
+        int i = 0;
+        for (; i + 1 < n_iter; i += 2) {
+            stage(i, a0, b0, a1, b1);
+            stage(i + 1, a1, b1, a0, b0);
+        }
+        if (i < n_iter) stage(i, a0, b0, a1, b1);
+    } else {
+        for (int i = 0; i < n_iter; ++i) {
+            wait_stage(i, Behind1{});
+            // the operand reads of this stage go first (x, then w in the order the products want
+            // them); the loads of a later stage are issued while they are on their way
+            bf16x8 a[FT], b[TT];
+            read_operands(a, b, i);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + NS - 1 < n_iter) issue(i + NS - 1);
+            __builtin_amdgcn_sched_barrier(0);
+            products(a, b);
+        }
     }
     // the loads are done (the last stage waited for vmcnt(0)); LDS is not touched again
 
@@ -210,13 +250,13 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
     }
 }
 
-template <int FT, int TT, int WT, int NS, int OCC, typename TOut, bool SWIGLU>
+template <int FT, int TT, int WT, int NS, int OCC, bool PIPE, typename TOut, bool SWIGLU>
 static void launch_async(int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N,
                          int K, int n_steps, int per, int out_cols) {
     constexpr int LDS = NS * (2 * FT + WT * TT) * 1024;
     static bool configured = false;
-    auto whole = gemm_async_kernel<FT, TT, WT, NS, OCC, TOut, SWIGLU, true>;
-    auto ragged = gemm_async_kernel<FT, TT, WT, NS, OCC, TOut, SWIGLU, false>;
+    auto whole = gemm_async_kernel<FT, TT, WT, NS, OCC, PIPE, TOut, SWIGLU, true>;
+    auto ragged = gemm_async_kernel<FT, TT, WT, NS, OCC, PIPE, TOut, SWIGLU, false>;
     if (!configured) {
         (void)hipFuncSetAttribute((const void*)whole, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         (void)hipFuncSetAttribute((const void*)ragged, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
@@ -251,11 +291,13 @@ static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16
     // chip; else 128 x 256 with eight waves, one block per compute unit
     if (variant == 0) variant = (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320 || M < 192) ? 3 : 6;
     switch (variant) {
-        case 1: launch_async<4, 4, 2, 4, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 2: launch_async<8, 4, 2, 2, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 4: launch_async<8, 4, 4, 4, 1, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 6: launch_async<4, 4, 4, 4, 1, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        default: launch_async<8, 4, 2, 3, 2, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 1: launch_async<4, 4, 2, 4, 2, false, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 2: launch_async<8, 4, 2, 4, 1, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 4: launch_async<8, 4, 4, 4, 1, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 5: launch_async<8, 4, 2, 3, 2, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 7: launch_async<4, 4, 4, 4, 1, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        case 6: launch_async<4, 4, 4, 4, 1, false, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
+        default: launch_async<8, 4, 2, 3, 2, false, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
     }
 }
 
