@@ -13,7 +13,8 @@
 //   S^T[key][query] = K . Q^T        A = K tile (LDS, stored as matrix-core tiles), B = Q (registers)
 //   softmax per column: the base m of the exponents and the sum l live in the lanes that own the
 //       column; rescaling the output needs no broadcast and happens only when a base moves, which
-//       it does lazily (when the maximum has run ahead of it by more than a factor of 256)
+//       it does lazily (when a score exceeds it by more than a factor of 256): the usual chunk
+//       costs no exchange between lanes
 //   O^T[d][query] += V^T . P^T       A = V^T tile (the cache stores values transposed inside a
 //       page, so its rows are runs of keys), B = P straight from the S^T accumulator
 // Scores are scaled by scale * log2(e) and exponentiated with exp2.  Query at position p sees keys
@@ -45,8 +46,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     constexpr int KT = 4 * QS;                // 1 KB tiles of a K stage: [chunk (2)][a/b (2)][k-step]
     constexpr int VT = 2 * DT;                // of a V stage: [chunk (2)][dim tile]
     constexpr int LPW = (KT + VT) / 4;        // tile loads per wave and stage
-    extern __shared__ __attribute__((aligned(16))) bf16_t ring[];       // [NS][KT + VT][512]
-    __shared__ int s_pages[PF_MAX_PAGES];
+    extern __shared__ __attribute__((aligned(16))) bf16_t ring[];       // [NS][KT + VT][512], then the pages
+    int* s_pages = (int*)(ring + (size_t)NS * (KT + VT) * 512);         // [max_blocks]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int j = lane & 15, g = lane >> 4;
@@ -93,10 +94,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         }
     }
     f32x4 o[QT][DT];
-    float m[QT], l[QT];
+    float m[QT], l[QT], thr[QT];              // base of the exponents, sum, and the score that moves the base
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
         m[t] = -INFINITY;
+        thr[t] = -INFINITY;
         l[t] = 0.f;
 #pragma unroll
         for (int d = 0; d < DT; ++d) o[t][d] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -111,9 +113,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int u = 0; u < LPW; ++u) {
         const int tl = wave + 4 * u;
         if (tl < KT) {                                         // K tile: chunk, a/b, k-step
+            // the four lanes of a quad copy 64 consecutive bytes of one key row (a quad spread over
+            // four rows costs four cache lookups); the pieces of a row are exchanged by (row / 2) % 4
+            // so that the operand reads meet no bank twice (see gemm_tiled.hip)
             const int c2 = tl / (2 * QS), ab = (tl / QS) & 1, s = tl % QS;
-            key_off[u] = 32 * c2 + pf_key_of_row(j, ab);
-            int d = 32 * s + 8 * g;
+            key_off[u] = 32 * c2 + pf_key_of_row(lane >> 2, ab);
+            int d = 32 * s + 8 * ((lane & 3) ^ ((lane >> 3) & 3));
             if (d + 8 > hd) d = 0;                             // padding dims: any finite data (Q is zero there)
             blk_off[u] = d;                                    // + row * hd, row known per stage
         } else {                                               // V tile: chunk, dim tile
@@ -125,6 +130,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             blk_off[u] = d * ps;                               // + row
         }
     }
+    // operand lane (key row j, k-piece g) finds its 16 bytes of a K tile here
+    const int k_read = 32 * j + 8 * (g ^ ((j >> 1) & 3));
     const int n_stage = (p_last / PF_STAGE) - (lo / PF_STAGE) + 1;
     const int t_base = (lo / PF_STAGE) * PF_STAGE;
     auto issue = [&](int i) {
@@ -172,45 +179,63 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             for (int t = 0; t < QT; ++t) { sa[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; sb[t] = sa[t]; }
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
-                const bf16x8 ka = *(const bf16x8*)(slot + ((2 * half) * QS + s) * 512 + lane * 8);
-                const bf16x8 kb = *(const bf16x8*)(slot + ((2 * half + 1) * QS + s) * 512 + lane * 8);
+                const bf16x8 ka = *(const bf16x8*)(slot + ((2 * half) * QS + s) * 512 + k_read);
+                const bf16x8 kb = *(const bf16x8*)(slot + ((2 * half + 1) * QS + s) * 512 + k_read);
 #pragma unroll
                 for (int t = 0; t < QT; ++t) {
                     sa[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[t][s], sa[t], 0, 0, 0);
                     sb[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[t][s], sb[t], 0, 0, 0);
                 }
             }
-            // ---- softmax per query column; this lane holds keys t0 + 8 g + r (a) and + 4 + r (b)
-            bf16x8 pmat[QT];
-            bool moved = false;
-            float corr[QT];
+            // ---- softmax per query column; this lane holds keys t0 + 8 g + r (a) and + 4 + r (b).
+            // m holds the raw (unscaled) score that the exponents are taken against.  It follows the
+            // running maximum lazily: only when a score exceeds it by more than 8 in the exponent (a
+            // factor of 256, harmless in float) does the column move its base and rescale what it
+            // has summed.  With 64 columns per wave some running maximum moves in nearly every
+            // chunk, a base almost never after the first ones; and whether any base has to move
+            // is a vote of the lanes over their own scores, so the usual chunk needs no exchange
+            // between lanes at all.
+            if (need_mask) {
+#pragma unroll
+                for (int t = 0; t < QT; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int ka = t0 + 8 * g + r, kb = ka + 4;
+                        sa[t][r] = (ka > p || ka < my_lo) ? -INFINITY : sa[t][r];
+                        sb[t][r] = (kb > p || kb < my_lo) ? -INFINITY : sb[t][r];
+                    }
+            }
+            float mx[QT];
+            bool above = false;
 #pragma unroll
             for (int t = 0; t < QT; ++t) {
-                // raw scores; the scale (with log2 e folded in) enters inside the exponent: one fma per value
-                float mx = -INFINITY;
+                mx[t] = fmaxf(fmaxf(fmaxf(sa[t][0], sa[t][1]), fmaxf(sa[t][2], sa[t][3])),
+                              fmaxf(fmaxf(sb[t][0], sb[t][1]), fmaxf(sb[t][2], sb[t][3])));
+                above = above || mx[t] > thr[t];
+            }
+            if (__any(above)) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if (need_mask) {
-                        const int ka = t0 + 8 * g + r, kb = ka + 4;
-                        if (ka > p || ka < my_lo) sa[t][r] = -INFINITY;
-                        if (kb > p || kb < my_lo) sb[t][r] = -INFINITY;
+                for (int t = 0; t < QT; ++t) {
+                    float cm = fmaxf(mx[t], __shfl_xor(mx[t], 16, 64));
+                    cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+                    if (cm > thr[t]) {                          // the same for the four lanes of a column
+                        // exp2(-inf) = 0: a column that had no key yet forgets its (empty) sums
+                        const float corr = __builtin_amdgcn_exp2f((m[t] - cm) * scale_log2e);
+                        l[t] *= corr;
+#pragma unroll
+                        for (int d = 0; d < DT; ++d) o[t][d] *= corr;
+                        m[t] = cm;
+                        thr[t] = cm + 8.0f / scale_log2e;
                     }
-                    mx = fmaxf(mx, fmaxf(sa[t][r], sb[t][r]));
                 }
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                // m holds the raw (unscaled) score that the exponents are taken against.  It follows
-                // the running maximum lazily: only when a chunk's maximum exceeds it by more than 8 in
-                // the exponent (a factor of 256, harmless in float) does the column move its base and
-                // rescale what it has summed.  With 64 columns per wave some running maximum moves
-                // in nearly every chunk, a base almost never after the first ones.  (-inf - -inf is
-                // NaN and compares false: a column without keys stays at -inf.)
-                const bool rebase = (mx - m[t]) * scale_log2e > 8.0f;
-                const float m_new = rebase ? mx : m[t];
-                // a column that has seen no key yet keeps m = -inf: use 0 as the base then
-                const float base = m_new == -INFINITY ? 0.f : m_new * scale_log2e;
-                corr[t] = rebase ? __builtin_amdgcn_exp2f(fmaf(m[t], scale_log2e, -base)) : 1.0f;      // exp2(-inf) = 0
-                if (rebase) moved = true;
+            }
+            bf16x8 pmat[QT];
+#pragma unroll
+            for (int t = 0; t < QT; ++t) {
+                // the scale (with log2 e folded in) enters inside the exponent: one fma per value.  A
+                // column that has seen no key yet keeps m = -inf: its base is 0 then (its scores
+                // are all -inf, their exponentials 0)
+                const float base = m[t] == -INFINITY ? 0.f : m[t] * scale_log2e;
                 float ls = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -220,15 +245,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                     pmat[t][r] = (bf16_t)ea;
                     pmat[t][4 + r] = (bf16_t)eb;
                 }
-                l[t] = l[t] * corr[t] + ls;
-                m[t] = m_new;
-            }
-            // ---- rescale the output only if some base in the wave moved
-            if (__any(moved)) {
-#pragma unroll
-                for (int t = 0; t < QT; ++t)
-#pragma unroll
-                    for (int d = 0; d < DT; ++d) o[t][d] *= corr[t];
+                l[t] += ls;
             }
             // ---- O^T += V^T P^T
 #pragma unroll
@@ -267,15 +284,19 @@ template <int HDP, int QT, int NS>
 static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                                const int* tiles, const int* positions, const int* block_table, int max_blocks,
                                int nh, float scale_log2e, int window, int log2_ps) {
-    constexpr int LDS = NS * (4 * (HDP / 32) + 2 * (HDP / 16)) * 1024;
+    constexpr int RING = NS * (4 * (HDP / 32) + 2 * (HDP / 16)) * 1024;
     static bool configured = false;
     auto kern = attn_prefill_kernel<HDP, QT, NS>;
     if (!configured) {
-        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  RING + PF_MAX_PAGES * (int)sizeof(int));
         configured = true;
     }
-    kern<<<grid, 256, LDS, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
+    kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
 }
+
+static int g_pf_stages = 0;              // ring stages: 0 = two (two blocks fit a compute unit), 3 for experiments
+extern "C" int fl_attn_prefill_set_stages(int n) { g_pf_stages = n; return 0; }
 
 template <int HDP, int NS>
 static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
@@ -315,8 +336,12 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     dim3 grid(n_tiles, nkv * (G / qt));
     const float sl = scale * 1.4426950408889634f;
 #define FL_PF(HDP_, NS_)                                                                                       \
-    launch_prefill<HDP_, NS_>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                              max_blocks, nh, sl, window, log2_ps)
+    if (NS_ == 3 && g_pf_stages == 3)                                                                          \
+        launch_prefill<HDP_, NS_>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
+                                  max_blocks, nh, sl, window, log2_ps);                                        \
+    else                                                                                                       \
+        launch_prefill<HDP_, 2>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
+                                max_blocks, nh, sl, window, log2_ps)
     switch (hdp) {
         case 32: FL_PF(32, 3); break;
         case 64: FL_PF(64, 3); break;
