@@ -24,7 +24,10 @@ int fl_gemm_plain(const void* x, const void* w, void* out, int in_dtype, int out
 int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int* positions,
                      const int* tok_seq, const int* block_table, int max_blocks, void* q_out,
                      void* cache_base, int dtype, int n, int nh, int nkv, int hd, int page_size,
-                     int n_pages, int rot, float theta, int write_cache, hipStream_t stream);
+                     int n_pages, int rot, float theta, int write_cache, const float* cs, int paired,
+                     hipStream_t stream);
+// cs[n][rot / 2][2]: cosine and sine of every (token, rotation pair) of a step
+int fl_rope_table(const int* positions, int n, int rot, float theta, float* cs, hipStream_t stream);
 int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
                   const int* positions, const int* tok_seq, const int* block_table,
                   int max_blocks, int n, int nh, int nkv, int hd, int page_size, int n_pages,

@@ -241,15 +241,42 @@ extern "C" int fl_gemm_plain(const void* x, const void* w, void* out, int in_dty
 }
 
 // ------------------------------------------------------------------ rotation + cache write
+// cos and sin of every (token, pair) of a step: cs[token][i] = (cos, sin)(position * theta^(-2 i / rot)).
+// Made once per step, read by every layer's rotation.
+__global__ __launch_bounds__(64) void rope_table_kernel(const int* __restrict__ positions, int rot, float theta,
+                                                        float2* __restrict__ cs) {
+    const int token = blockIdx.x, half = rot >> 1;
+    const float pos = (float)positions[token];
+    for (int i = threadIdx.x; i < half; i += 64) {
+        const float exponent = 2.0f * (float)i / (float)rot;
+        const float inv_freq = 1.0f / powf(theta, exponent);
+        const float angle = pos * inv_freq;
+        cs[(size_t)token * half + i] = make_float2(cosf(angle), sinf(angle));
+    }
+}
+
+extern "C" int fl_rope_table(const int* positions, int n, int rot, float theta, float* cs, hipStream_t stream) {
+    FL_CHECK(n >= 0 && rot > 0 && rot % 2 == 0, "rope_table: %d rotated dims", rot);
+    FL_CHECK((uintptr_t)cs % 8 == 0, "rope_table: the table must be 8-byte aligned");
+    if (n == 0) return 0;
+    rope_table_kernel<<<n, 64, 0, stream>>>(positions, rot, theta, (float2*)cs);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+
 // One block per (token, head) over the fused projection row [q heads | k heads | v heads].
 // Q heads: rotated, written to q_out.  K heads: rotated, written to the cache at the token's
 // position.  V heads: written to the cache as they are.  rot = rotated dims (pairs (i, i+rot/2));
-// rot = 0 means no rotation at all (another position encoding has run, or none).
+// rot = 0 means no rotation at all (another position encoding has run, or none).  cs: the step's
+// table of cosines and sines, or null (then they are computed here).  paired: the rotated dims of
+// a q or k head arrive in the order of fl_rotary_paired_rows (8 dims, their 8 partners, the next
+// 8 dims, ...), as the projection's fused kernels want them.
 template <typename TIn, typename T>
 __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const TIn* __restrict__ qkv, int ld, const int* __restrict__ positions,
     const int* __restrict__ tok_seq, const int* __restrict__ block_table, int max_blocks,
-    T* __restrict__ q_out, PagedCache cache, int nh, int hd, int rot, float theta, int write_cache) {
+    T* __restrict__ q_out, PagedCache cache, int nh, int hd, int rot, float theta, int write_cache,
+    const float2* __restrict__ cs, int paired) {
     const int token = blockIdx.x;
     const int head = blockIdx.y;
     const int nkv = cache.n_kv_heads;
@@ -279,11 +306,18 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const int half = rot >> 1;
     if (rotate && rot > 0) {
         for (int i = threadIdx.x; i < half; i += 64) {
-            const float exponent = 2.0f * (float)i / (float)rot;
-            const float inv_freq = 1.0f / powf(theta, exponent);
-            const float angle = (float)pos * inv_freq;
-            const float c = cosf(angle), s = sinf(angle);
-            const float x0 = to_f32(src[i]), x1 = to_f32(src[i + half]);
+            float c, s;
+            if (cs) {
+                const float2 v = cs[(size_t)token * half + i];
+                c = v.x; s = v.y;
+            } else {
+                const float exponent = 2.0f * (float)i / (float)rot;
+                const float inv_freq = 1.0f / powf(theta, exponent);
+                const float angle = (float)pos * inv_freq;
+                c = cosf(angle); s = sinf(angle);
+            }
+            const int at = paired ? 16 * (i >> 3) + (i & 7) : i;
+            const float x0 = to_f32(src[at]), x1 = to_f32(src[paired ? at + 8 : i + half]);
             dst[i] = from_f32<T>(x0 * c - x1 * s);
             dst[i + half] = from_f32<T>(x0 * s + x1 * c);
         }
@@ -297,17 +331,18 @@ extern "C" int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int
                                 const int* tok_seq, const int* block_table, int max_blocks,
                                 void* q_out, void* cache_base, int dtype, int n, int nh, int nkv,
                                 int hd, int page_size, int n_pages, int rot, float theta,
-                                int write_cache, hipStream_t stream) {
+                                int write_cache, const float* cs, int paired, hipStream_t stream) {
     FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && hd > 0 && page_size > 0, "rope_kv_write: bad sizes");
     FL_CHECK(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotated dims %d of head %d", rot, hd);
     FL_CHECK(ld >= (nh + 2 * nkv) * hd, "rope_kv_write: row stride %d too small", ld);
+    FL_CHECK(!paired || (rot % 16 == 0 && hd % 16 == 0), "rope_kv_write: the paired order needs rotated dims and head size in steps of 16 (%d of %d)", rot, hd);
     if (n == 0) return 0;
     PagedCache c{cache_base, nkv, page_size, hd, n_pages};
     dim3 grid(n, nh + 2 * nkv);
 #define FL_ROPE(TIN, TT)                                                                       \
     rope_kv_write_kernel<TIN, TT><<<grid, 64, 0, stream>>>((const TIN*)qkv, ld, positions, tok_seq, \
                                                            block_table, max_blocks, (TT*)q_out, c, \
-                                                           nh, hd, rot, theta, write_cache)
+                                                           nh, hd, rot, theta, write_cache, (const float2*)cs, paired)
     if (in_dtype == FL_F32 && dtype == FL_F32) FL_ROPE(float, float);
     else if (in_dtype == FL_F32 && dtype == FL_BF16) FL_ROPE(float, bf16_t);
     else if (in_dtype == FL_BF16 && dtype == FL_BF16) FL_ROPE(bf16_t, bf16_t);

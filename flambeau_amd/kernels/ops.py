@@ -101,8 +101,19 @@ def gemm_plain(x, w, out):
     return out
 
 
+def rope_table(positions, rotated_dims, theta, out):
+    """``out[n, rotated_dims / 2, 2]`` = (cos, sin)(position * theta^(-2 i / rotated_dims)), float32."""
+    n = positions.shape[0]
+    call("fl_rope_table", _check(positions, "rope.positions", torch.int32, (n,)), n, int(rotated_dims), float(theta),
+         _check(out, "rope.table", torch.float32, (n, rotated_dims // 2, 2)), stream_handle())
+    return out
+
+
 def rope_kv_write(qkv, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads,
-                  rotated_dims, theta, write_cache=True):
+                  rotated_dims, theta, write_cache=True, table=None, paired=False):
+    """Rotate q and k, store q and the cache rows.  ``table``: the step's ``rope_table`` (else the
+    angles are computed here); ``paired``: the projection's rows come in the order of
+    ``rotary_paired_rows``."""
     n, ld = qkv.shape
     nkv, hd = cache.n_kv_heads, cache.head_dim
     if ld != (n_heads + 2 * nkv) * hd:
@@ -114,7 +125,8 @@ def rope_kv_write(qkv, positions, tok_seq, block_table, q_out, cache: PagedLayer
          _check(q_out, "rope.q_out", cache.pool.dtype, (n, n_heads * hd)),
          _check(cache.pool, "rope.cache"), dtype_code(cache.pool.dtype), n, n_heads, nkv, hd,
          cache.page_size, cache.n_pages, int(rotated_dims), float(theta), int(bool(write_cache)),
-         stream_handle())
+         _check(table, "rope.table", torch.float32, (n, rotated_dims // 2, 2)) if table is not None and rotated_dims else None,
+         int(bool(paired)), stream_handle())
     return q_out
 
 

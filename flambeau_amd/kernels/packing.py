@@ -63,3 +63,24 @@ class Weight:
     @property
     def dtype(self):
         return (self.packed if self.packed is not None else self.rowmajor).dtype
+
+
+def rotary_paired_rows(n_heads: int, n_kv_heads: int, head_dim: int, rotated_dims: int):
+    """Order of the rows of a joined q/k/v projection in which a split-half rotation can be applied
+    by the product's own kernel: within every q and k head the rotated dims come as 8 dims, their 8
+    partners (dim + rotated_dims / 2), the next 8 dims, ...; a group of 16 output features then
+    holds whole pairs, four lanes apart in the accumulators.  Dims beyond the rotated ones and the
+    v heads keep their places.  ``perm[new row] = old row``; ``None`` if the sizes are not in
+    steps of 16."""
+    if rotated_dims <= 0 or rotated_dims % 16 or head_dim % 16:
+        return None
+    half = rotated_dims // 2
+    head = []
+    for b in range(half // 8):
+        head += list(range(8 * b, 8 * b + 8)) + list(range(half + 8 * b, half + 8 * b + 8))
+    head += list(range(rotated_dims, head_dim))
+    perm = []
+    for h in range(n_heads + n_kv_heads):
+        perm += [h * head_dim + d for d in head]
+    perm += list(range((n_heads + n_kv_heads) * head_dim, (n_heads + 2 * n_kv_heads) * head_dim))
+    return torch.tensor(perm, dtype=torch.long)

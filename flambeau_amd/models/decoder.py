@@ -115,6 +115,7 @@ class DecoderModel:
         """Logits ``[R, vocab]`` (float32) at ``step.logit_rows``; ``caches[i]`` belongs to
         run-order entry ``i``."""
         rt = self.rt
+        step.scratch.clear()
         resid = rt.buffer("residual", step.n_tokens, self.spec.hidden_size, torch.float32)
         self.embedding.forward(step.tokens, resid)
         stream = ResidualStream(resid, rt)

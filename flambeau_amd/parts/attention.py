@@ -64,12 +64,15 @@ class PagedGQAAttention(Mixer):
         qkv = rt.buffer("attn_qkv", n, (nh + 2 * nkv) * hd, torch.float32)
         rt.gemm(x, self.w_qkv, qkv)
         rotary = self.position.rotary_parameters()
+        angles = None
         if rotary is None:
             self.position.apply(qkv, step.positions, nh, nkv, hd)
             rotary = (0, 1.0)
+        elif rotary[0]:
+            angles = self.position.rotary_table(rt, step)
         q = rt.buffer("attn_q", n, nh * hd)
         ops.rope_kv_write(qkv, step.positions, step.tok_seq, table, q, cache.kv, nh, rotary[0], rotary[1],
-                          write_cache=cache.writes)
+                          write_cache=cache.writes, table=angles)
         out = rt.buffer("attn_out", n, nh * hd)
         if rt.tuned:
             from ..kernels import tuned

@@ -80,6 +80,7 @@ class StepState:
     logit_rows: torch.Tensor       # int32 [R] rows whose logits are wanted
     host: "HostBatch"              # the same numbers on the host, for choosing kernels
     extra: dict = field(default_factory=dict)   # metadata parts asked for (step_metadata)
+    scratch: dict = field(default_factory=dict)  # what parts compute once per forward pass and share between layers; emptied when a pass begins
 
 
 @dataclass
@@ -152,6 +153,12 @@ class PositionEncoding(Part):
     def rotary_parameters(self):
         """``(rotated_dims, theta)`` if this encoding is the split-half rotation the fused
         rotate-and-store kernel implements, else ``None`` (then ``apply`` is called)."""
+        return None
+
+    def rotary_table(self, rt, step):
+        """Optional: cosines and sines ``[n, rotated_dims / 2, 2]`` (float32) of the step's
+        positions for the rotation of ``rotary_parameters``, or ``None`` (the kernels then compute
+        the angles themselves)."""
         return None
 
     def apply(self, q, k, positions, n_heads, n_kv_heads, head_dim):

@@ -7,6 +7,9 @@ itself runs inside the mixer's rotate-and-store kernel; this part only carries i
 constants."""
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
 from .base import POSITION_ENCODINGS, PositionEncoding
 
 
@@ -21,6 +24,19 @@ class RotaryNeoX(PositionEncoding):
 
     def rotary_parameters(self):
         return self.rotated_dims, self.theta
+
+    def rotary_table(self, rt, step):
+        """The angles depend on the positions only: their cosines and sines are made once per
+        forward pass and shared by all layers with the same constants."""
+        key = ("rope_neox", self.rotated_dims, self.theta)
+        table = step.scratch.get(key)
+        if table is None:
+            half = self.rotated_dims // 2
+            table = rt.buffer(f"rope_table_{self.rotated_dims}_{self.theta}", step.n_tokens, 2 * half, torch.float32)
+            table = table.view(step.n_tokens, half, 2)
+            ops.rope_table(step.positions, self.rotated_dims, self.theta, table)
+            step.scratch[key] = table
+        return table
 
 
 @POSITION_ENCODINGS.register("none")

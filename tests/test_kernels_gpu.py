@@ -255,6 +255,25 @@ def test_rope_kv_write(dtype, nh, nkv, hd, ps, rot, theta):
     for p in range(n_pages):
         if p not in touched:
             assert not cache.pool[p].any()
+    # the same with the angles from the step's table, and with the projection's rows in paired order
+    from flambeau_amd.kernels.packing import rotary_paired_rows
+    variants = []
+    if rot:
+        angles = torch.full((n, rot // 2, 2), float("nan"), dtype=torch.float32, device=DEV)
+        ops().rope_table(pos_d, rot, theta, angles)
+        variants.append(dict(table=angles))
+        order = rotary_paired_rows(nh, nkv, hd, rot)
+        assert (order is None) == bool(rot % 16 or hd % 16)
+        if order is not None:
+            assert sorted(order.tolist()) == list(range((nh + 2 * nkv) * hd))
+            variants.append(dict(table=angles, paired=True, order=order))
+    for v in variants:
+        cache2 = make_cache(n_pages, nkv, ps, hd, dtype)
+        q2 = torch.empty_like(q_out)
+        order = v.pop("order", None)
+        src = qkv if order is None else qkv[:, order.to(DEV)].contiguous()
+        ops().rope_kv_write(src, pos_d, seq_d, table.to(DEV), q2, cache2, nh, rot, theta, **v)
+        assert torch.equal(q2, q_out) and torch.equal(cache2.pool, cache.pool)
 
 
 def attention_ref(q, keys, vals, pos, scale, window):
