@@ -63,6 +63,17 @@ int fl_gemm_mid_splits(int M, int N, int K);
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_tiled_splits(int M, int N, int K);
+// The joined q/k/v projection (rows of w in paired order) with rotation and the stores of q and the
+// cache rows in the product's kernel: at most 16 rows, and many rows (shapes whose K is not split).
+int fl_gemm_skinny_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
+                        int in_parts, float eps, const int* positions, const int* tok_seq,
+                        const int* block_table, int max_blocks, const float* cs, void* q_out,
+                        void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages, int rot,
+                        int write_cache, hipStream_t stream);
+int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const int* positions,
+                       const int* tok_seq, const int* block_table, int max_blocks, const float* cs,
+                       void* q_out, void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages,
+                       int rot, int write_cache, hipStream_t stream);
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                    const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
                    int n_pages, float scale, int window, int n_split, hipStream_t stream);

@@ -31,6 +31,7 @@
 // (crates/kernels-hip/src/kernels/dense_gemv_f16_f16.cu:27-71, ..._batched.cu:17-63).
 #include "common.h"
 #include "api.h"
+#include "rope_store.h"
 
 __device__ __forceinline__ void store4(float* p, f32x4 v) { *(f32x4*)p = v; }
 __device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
@@ -55,12 +56,13 @@ struct SkinnyFusion {
 #define EPI_PLAIN 0
 #define EPI_SWIGLU 1
 #define EPI_RESIDUAL 2
+#define EPI_ROPE 3               // rotate q and k, store q and the cache rows (rope_store.h)
 
 template <int MT, typename TOut, int EPI>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ wp,
                                                            TOut* __restrict__ out, int M, int N, int K,
-                                                           int n_steps, int out_cols, SkinnyFusion fu) {
+                                                           int n_steps, int out_cols, SkinnyFusion fu, RopeStore rs) {
     constexpr bool SWIGLU = EPI == EPI_SWIGLU;
     extern __shared__ float red[];               // [NW][MT][64][4], then [NW * 4][16] for the row scale
     const int nw = blockDim.x >> 6;
@@ -133,6 +135,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
         }
     }
 
+    // epilogue 3: where this token's key and value go (two dependent loads, early)
+    TokenPlace place = {-1, 0};
+    if (EPI == EPI_ROPE && MT == 1 && wave == 0 && li < M) place = rope_token_place(rs, li);
+
     int s = s0;
     // iterations of U steps: every load of the iteration is issued before the first product needs
     // its data.  x beyond K does not exist (w is zero there): such chunks count as zero.
@@ -188,7 +194,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 #pragma unroll
                 for (int r = 0; r < 4; ++r) sum[r] *= scale;
             }
-            if (EPI == EPI_RESIDUAL) {
+            if (EPI == EPI_ROPE) {
+                const int f0 = blockIdx.x * 16 + 4 * g;
+                rope_store4(rs, tok, place, f0, g, sum, MT == 1 && tok < M && f0 < N);
+            } else if (EPI == EPI_RESIDUAL) {
                 const int f0 = blockIdx.x * 16 + 4 * g;
                 f32x4 nr;
                 float sq = 0.f;
@@ -265,27 +274,30 @@ extern "C" int fl_gemm_skinny_scale_parts(int N, int K, int in_parts) {
 
 template <int MT, typename TOut>
 static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
-                         int epilogue, int out_cols, const SkinnyFusion& fu, hipStream_t stream) {
+                         int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs, hipStream_t stream) {
     const int groups = ceil_div(N, 16);
     const int n_steps = ceil_div(K, 32);
     const int nw = skinny_waves(N, K, nw_hint);
     const size_t lds = (size_t)nw * MT * 64 * 4 * sizeof(float) + (size_t)nw * 4 * 16 * sizeof(float);
     if (epilogue == EPI_SWIGLU)
-        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu);
+        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else if (epilogue == EPI_RESIDUAL)
-        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu);
+        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+    else if (epilogue == EPI_ROPE)
+        gemm_skinny_kernel<MT, TOut, EPI_ROPE><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else
-        gemm_skinny_kernel<MT, TOut, EPI_PLAIN><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu);
+        gemm_skinny_kernel<MT, TOut, EPI_PLAIN><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     return 0;
 }
 
 static int skinny_entry(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
-                        int nw_hint, int epilogue, int out_cols, const SkinnyFusion& fu, hipStream_t stream) {
+                        int nw_hint, int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs,
+                        hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
     FL_CHECK(nw_hint >= 0 && nw_hint <= 16, "gemm_skinny: %d waves per block, at most 16", nw_hint);
     FL_CHECK(K % 8 == 0, "gemm_skinny: K=%d is no multiple of 8 (16-byte loads)", K);
-    FL_CHECK(epilogue >= 0 && epilogue <= 2, "gemm_skinny: unknown epilogue %d", epilogue);
+    FL_CHECK(epilogue >= 0 && epilogue <= 3, "gemm_skinny: unknown epilogue %d", epilogue);
     FL_CHECK(epilogue != EPI_SWIGLU ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
              "gemm_skinny: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
@@ -294,7 +306,15 @@ static int skinny_entry(const void* x, const void* w_packed, void* out, int out_
         FL_CHECK(fu.resid && fu.g && fu.xg && fu.out_ssq, "gemm_skinny: the residual epilogue needs resid, g, xg and out_ssq");
         FL_CHECK(((uintptr_t)fu.resid % 16 == 0) && ((uintptr_t)fu.xg % 8 == 0), "gemm_skinny: resid and xg must be aligned to 16 and 8 bytes");
     }
-    if (fu.in_ssq || epilogue == EPI_RESIDUAL)
+    if (epilogue == EPI_ROPE) {
+        const int hd = rs.cache.head_dim;
+        FL_CHECK(rs.positions && rs.tok_seq && rs.block_table && rs.cs && rs.q_out && rs.cache.base,
+                 "gemm_skinny: the rotate-and-store epilogue needs positions, requests, block table, angles, q and the cache");
+        FL_CHECK(hd % 16 == 0 && rs.rot % 16 == 0 && rs.rot <= hd && N == (rs.nh + 2 * rs.cache.n_kv_heads) * hd,
+                 "gemm_skinny: rotate-and-store over %d features with heads of %d (%d rotated), %d + 2 x %d heads", N, hd,
+                 rs.rot, rs.nh, rs.cache.n_kv_heads);
+    }
+    if (fu.in_ssq || epilogue == EPI_RESIDUAL || epilogue == EPI_ROPE)
         FL_CHECK(M <= 16, "gemm_skinny: the fusions with the norm take at most 16 rows, not %d", M);
     if (fu.in_ssq) {
         const int cap = fl_gemm_skinny_scale_parts(N, K, fu.in_parts);
@@ -305,8 +325,8 @@ static int skinny_entry(const void* x, const void* w_packed, void* out, int out_
     if (M == 0) return 0;
     const int mt = ceil_div(M, 16);
 #define FL_SK(MT_)                                                                                         \
-    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N, K, nw_hint, epilogue, out_cols, fu, stream); \
-    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M, N, K, nw_hint, epilogue, out_cols, fu, stream)
+    if (out_dtype == FL_F32) launch_skinny<MT_, float>((const bf16_t*)x, (const bf16_t*)w_packed, (float*)out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream); \
+    else launch_skinny<MT_, bf16_t>((const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream)
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
     switch (mt) {
         case 1: FL_SK(1); break;
@@ -325,7 +345,7 @@ extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, in
                               int K, int nw_hint, int epilogue, int out_cols, hipStream_t stream) {
     FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_skinny: unknown epilogue %d", epilogue);
     const SkinnyFusion none = {nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr};
-    return skinny_entry(x, w_packed, out, out_dtype, M, N, K, nw_hint, epilogue, out_cols, none, stream);
+    return skinny_entry(x, w_packed, out, out_dtype, M, N, K, nw_hint, epilogue, out_cols, none, RopeStore{}, stream);
 }
 
 // The same product fused with the norms around it.  in_ssq (or null): [M, in_parts] partial sums of
@@ -337,10 +357,25 @@ extern "C" int fl_gemm_skinny_fused(const void* x, const void* w_packed, void* o
                                     int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
                                     float eps, float* resid, const float* g, void* xg, float* out_ssq,
                                     hipStream_t stream) {
+    FL_CHECK(epilogue != EPI_ROPE, "gemm_skinny_fused: the rotate-and-store epilogue has its own entry point");
     const SkinnyFusion fu = {in_ssq, in_parts, eps, resid, g, (bf16_t*)xg, out_ssq};
     if (epilogue == EPI_RESIDUAL && !out) out = resid;
     return skinny_entry(x, w_packed, out, epilogue == EPI_RESIDUAL ? FL_F32 : out_dtype, M, N, K, 0, epilogue,
-                        out_cols, fu, stream);
+                        out_cols, fu, RopeStore{}, stream);
+}
+
+// The joined q/k/v projection of at most 16 rows with its rows in paired order: q is rotated and
+// written to q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens'
+// positions; cs[M, rot / 2, 2] are the step's cosines and sines.  in_ssq as in fl_gemm_skinny_fused.
+extern "C" int fl_gemm_skinny_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
+                                   int in_parts, float eps, const int* positions, const int* tok_seq,
+                                   const int* block_table, int max_blocks, const float* cs, void* q_out,
+                                   void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages, int rot,
+                                   int write_cache, hipStream_t stream) {
+    const SkinnyFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
+    const RopeStore rs = {positions, tok_seq, block_table, max_blocks, (const float2*)cs, (bf16_t*)q_out,
+                          PagedCache{cache_base, nkv, page_size, hd, n_pages}, nh, rot, write_cache};
+    return skinny_entry(x, w_packed, q_out, FL_BF16, M, N, K, 0, EPI_ROPE, N, fu, rs, stream);
 }
 
 extern "C" int fl_gemm_skinny_blocks(int N) { return ceil_div(N, 16); }

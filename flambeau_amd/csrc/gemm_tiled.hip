@@ -26,9 +26,13 @@
 #include <type_traits>
 #include "common.h"
 #include "api.h"
+#include "rope_store.h"
 
 #define TG_BM 128                        // block tile the split-K rule counts with
 #define TG_BN 128
+#define TG_PLAIN 0                       // epilogues
+#define TG_SWIGLU 1
+#define TG_ROPE 2
 
 
 template <typename TOut>
@@ -47,11 +51,12 @@ template <> __device__ __forceinline__ void tg_store4<bf16_t>(bf16_t* p, f32x4 v
 //     stage i - 1 just left; read the operands of stage i from LDS; FT * TT products.
 // Nothing is zero-filled: rows beyond M and feature groups beyond N are clamped to valid ones (their
 // results are never stored), and k beyond K meets the zero padding of the packed w.
-template <int FT, int TT, int WT, int NS, int OCC, bool PIPE, typename TOut, bool SWIGLU, bool KWHOLE>
+template <int FT, int TT, int WT, int NS, int OCC, typename TOut, int EPI, bool KWHOLE>
 __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t* __restrict__ x,
                                                             const bf16_t* __restrict__ wp,
                                                             TOut* __restrict__ out, int M, int N, int K,
-                                                            int n_steps, int steps_per_split, int out_cols) {
+                                                            int n_steps, int steps_per_split, int out_cols,
+                                                            RopeStore rs) {
     constexpr int NW = 2 * WT;                        // waves: 2 along the features, WT along the tokens
     constexpr int NTF = 2 * FT, NTT = WT * TT;        // operand tiles of the block: features, tokens
     constexpr int TILES = NTF + NTT;                  // 1 KB tiles per stage
@@ -160,33 +165,7 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
         asm volatile("s_barrier" ::: "memory");
     };
     using Behind1 = std::integral_constant<int, NS - 2>;       // reads follow the loads NS - 1 stages behind
-    using Behind2 = std::integral_constant<int, (NS >= 3 ? NS - 3 : 0)>;
-    if (PIPE) {
-        // The operands of stage i + 1 are read into a second set of registers while the products
-        // of stage i run: the matrix cores do not wait for LDS.  Loads run NS - 2 stages ahead of
-        // the reads.
-        bf16x8 a0[FT], b0[TT], a1[FT], b1[TT];
-        auto stage = [&](int i, bf16x8 (&ac)[FT], bf16x8 (&bc)[TT], bf16x8 (&an)[FT], bf16x8 (&bn)[TT]) {
-            if (i + 1 < n_iter) {
-                wait_stage(i + 1, Behind2{});
-                read_operands(an, bn, i + 1);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (i + NS - 1 < n_iter) issue(i + NS - 1);
-            __builtin_amdgcn_sched_barrier(0);
-            products(ac, bc);
-        };
-        if (n_iter > 0) {
-            wait_stage(0, Behind1{});
-            read_operands(a0, b0, 0);
-        }
-        int i = 0;
-        for (; i + 1 < n_iter; i += 2) {
-            stage(i, a0, b0, a1, b1);
-            stage(i + 1, a1, b1, a0, b0);
-        }
-        if (i < n_iter) stage(i, a0, b0, a1, b1);
-    } else {
+    {
         for (int i = 0; i < n_iter; ++i) {
             wait_stage(i, Behind1{});
             // the operand reads of this stage go first (x, then w in the order the products want
@@ -202,7 +181,22 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
     // the loads are done (the last stage waited for vmcnt(0)); LDS is not touched again
 
     const int j = lane & 15, g = lane >> 4;
-    if (SWIGLU) {
+    if (EPI == TG_ROPE) {
+        // the joined q/k/v projection: rotate, store q and the cache rows (rope_store.h)
+#pragma unroll
+        for (int tb = 0; tb < TT; ++tb) {
+            const int tok = m0 + (wt * TT + tb) * 16 + j;
+            TokenPlace place = {-1, 0};
+            if (tok < M) place = rope_token_place(rs, tok);
+#pragma unroll
+            for (int ta = 0; ta < FT; ++ta) {
+                const int f0 = n0 + (wf * FT + ta) * 16 + 4 * g;
+                rope_store4(rs, tok, place, f0, g, acc[ta][tb], tok < M && f0 < N);
+            }
+        }
+        return;
+    }
+    if (EPI == TG_SWIGLU) {
 #pragma unroll
         for (int tb = 0; tb < TT; ++tb) {
             const int tok = m0 + (wt * TT + tb) * 16 + j;
@@ -250,13 +244,13 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
     }
 }
 
-template <int FT, int TT, int WT, int NS, int OCC, bool PIPE, typename TOut, bool SWIGLU>
+template <int FT, int TT, int WT, int NS, int OCC, typename TOut, int EPI>
 static void launch_async(int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N,
-                         int K, int n_steps, int per, int out_cols) {
+                         int K, int n_steps, int per, int out_cols, const RopeStore& rs) {
     constexpr int LDS = NS * (2 * FT + WT * TT) * 1024;
     static bool configured = false;
-    auto whole = gemm_async_kernel<FT, TT, WT, NS, OCC, PIPE, TOut, SWIGLU, true>;
-    auto ragged = gemm_async_kernel<FT, TT, WT, NS, OCC, PIPE, TOut, SWIGLU, false>;
+    auto whole = gemm_async_kernel<FT, TT, WT, NS, OCC, TOut, EPI, true>;
+    auto ragged = gemm_async_kernel<FT, TT, WT, NS, OCC, TOut, EPI, false>;
     if (!configured) {
         (void)hipFuncSetAttribute((const void*)whole, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         (void)hipFuncSetAttribute((const void*)ragged, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
@@ -265,7 +259,7 @@ static void launch_async(int splits, hipStream_t stream, const bf16_t* x, const 
     auto kern = (K % 32 == 0) ? whole : ragged;
     const int tiles = ceil_div(N, 2 * FT * 16) * ceil_div(M, WT * TT * 16);
     dim3 grid(ceil_div(tiles, 8) * 8, 1, splits);
-    kern<<<grid, 128 * WT, LDS, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols);
+    kern<<<grid, 128 * WT, LDS, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols, rs);
 }
 
 template <typename TOut>
@@ -279,26 +273,20 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     out[i] = from_f32<TOut>(s);
 }
 
-// Shape of the block: 0 = chosen from the sizes; for experiments 1 = 128 x 128 (4 waves, ring of 4), 2 and 3 =
-// 256 x 128 (4 waves, ring of 2 and 3), 4 = 256 x 256 (8 waves, ring of 4), 6 = 128 x 256 (8 waves, ring of 4).
+// Shape of the block: 0 = chosen from the sizes, 3 = 256 features x 128 tokens (4 waves, ring of 3, two blocks
+// per compute unit), 6 = 128 x 256 (8 waves, ring of 4, one block per compute unit); set for tests and experiments.
 static int g_tiled_variant = 0;
 extern "C" int fl_gemm_tiled_set_variant(int v) { g_tiled_variant = v; return 0; }
 
-template <typename TOut, bool SWIGLU>
+template <typename TOut, int EPI>
 static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out,
-                         int M, int N, int K, int n_steps, int per, int out_cols) {
-    // 256 features x 128 tokens with four waves, two blocks per compute unit, where that fills the
-    // chip; else 128 x 256 with eight waves, one block per compute unit
+                         int M, int N, int K, int n_steps, int per, int out_cols, const RopeStore& rs) {
+    // 256 x 128 where that fills the chip (and for few rows), else 128 x 256
     if (variant == 0) variant = (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320 || M < 192) ? 3 : 6;
-    switch (variant) {
-        case 1: launch_async<4, 4, 2, 4, 2, false, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 2: launch_async<8, 4, 2, 4, 1, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 4: launch_async<8, 4, 4, 4, 1, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 5: launch_async<8, 4, 2, 3, 2, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 7: launch_async<4, 4, 4, 4, 1, true, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        case 6: launch_async<4, 4, 4, 4, 1, false, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-        default: launch_async<8, 4, 2, 3, 2, false, TOut, SWIGLU>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols); break;
-    }
+    if (variant == 6)
+        launch_async<4, 4, 4, 4, 1, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs);
+    else
+        launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs);
 }
 
 // How many ways K is split for a product of this shape: 1 if the grid fills the chip.
@@ -331,13 +319,14 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
     const int v = g_tiled_variant;
+    const RopeStore none{};
     if (epilogue) {
         if (out_dtype == FL_F32)
-            launch_tiled<float, true>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, out_cols);
+            launch_tiled<float, TG_SWIGLU>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, out_cols, none);
         else
-            launch_tiled<bf16_t, true>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, out_cols);
+            launch_tiled<bf16_t, TG_SWIGLU>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, out_cols, none);
     } else if (splits > 1) {
-        launch_tiled<float, false>(v, splits, stream, xb, wb, workspace, M, N, K, n_steps, per, N);
+        launch_tiled<float, TG_PLAIN>(v, splits, stream, xb, wb, workspace, M, N, K, n_steps, per, N, none);
         FL_LAUNCH_CHECK();
         const size_t total = (size_t)M * N;
         const unsigned rb = (unsigned)((total + 255) / 256);
@@ -346,10 +335,36 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
         else
             gemm_splitk_reduce_kernel<bf16_t><<<rb, 256, 0, stream>>>(workspace, (bf16_t*)out, total, splits);
     } else if (out_dtype == FL_F32) {
-        launch_tiled<float, false>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, N);
+        launch_tiled<float, TG_PLAIN>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, N, none);
     } else {
-        launch_tiled<bf16_t, false>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, N);
+        launch_tiled<bf16_t, TG_PLAIN>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, N, none);
     }
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+
+// The joined q/k/v projection of many rows with its rows in paired order: q is rotated and written to
+// q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens' positions; cs[M,
+// rot / 2, 2] are the step's cosines and sines.  Only for shapes whose K is not split
+// (fl_gemm_tiled_splits == 1).
+extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const int* positions,
+                                  const int* tok_seq, const int* block_table, int max_blocks, const float* cs,
+                                  void* q_out, void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages,
+                                  int rot, int write_cache, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_rope: bad sizes M=%d N=%d K=%d", M, N, K);
+    FL_CHECK(K % 8 == 0, "gemm_tiled_rope: K=%d is no multiple of 8 (16-byte loads)", K);
+    FL_CHECK(positions && tok_seq && block_table && cs && q_out && cache_base,
+             "gemm_tiled_rope: needs positions, requests, block table, angles, q and the cache");
+    FL_CHECK(hd % 16 == 0 && rot % 16 == 0 && rot <= hd && N == (nh + 2 * nkv) * hd,
+             "gemm_tiled_rope: %d features with heads of %d (%d rotated), %d + 2 x %d heads", N, hd, rot, nh, nkv);
+    FL_CHECK(fl_gemm_tiled_splits(M, N, K) == 1, "gemm_tiled_rope: this shape splits K");
+    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0), "gemm_tiled_rope: operands must be 16-byte aligned");
+    if (M == 0) return 0;
+    const RopeStore rs = {positions, tok_seq, block_table, max_blocks, (const float2*)cs, (bf16_t*)q_out,
+                          PagedCache{cache_base, nkv, page_size, hd, n_pages}, nh, rot, write_cache};
+    const int n_steps = ceil_div(K, 32);
+    launch_tiled<bf16_t, TG_ROPE>(g_tiled_variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)q_out,
+                                  M, N, K, n_steps, n_steps, N, rs);
     FL_LAUNCH_CHECK();
     return 0;
 }

@@ -97,6 +97,15 @@ class Runtime:
             return tuned.gemm(x, w, out, rt=self)
         return ops.gemm_plain(x, w.rowmajor, out)
 
+    def gemm_rope_store(self, x, w, store) -> bool:
+        """The joined q/k/v projection fused with rotation and the stores of q and the cache rows
+        (``store``: ``kernels.tuned.RopeStore``; the rows of ``w`` in paired order).  ``False`` if no
+        kernel takes the shape: the caller then runs product and rotation apart."""
+        if not self.tuned:
+            return False
+        from ..kernels import tuned
+        return tuned.gemm_rope_store(x, w, store, rt=self)
+
     def gemm_swiglu(self, x, w, out):
         """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``.  The tuned
         kernels apply the gate before they store; the plain path is a product and a gate kernel."""

@@ -18,6 +18,8 @@ register_signatures({
     "fl_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, P],
     "fl_gemm_skinny_fused": [P, P, P, I, I, I, I, I, I, P, I, F, P, P, P, P, P],
     "fl_gemm_skinny_scale_parts": [I, I, I],
+    "fl_gemm_skinny_rope": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
+    "fl_gemm_tiled_rope": [P, P, I, I, I, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
     "fl_gemm_mid": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_mid_splits": [I, I, I],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
@@ -109,6 +111,77 @@ def gemm_skinny_residual(x, w_packed, resid, g, xg, ssq, eps: float, row_scale: 
          _check(g, "gemm.g", torch.float32, (N,)), _check(xg, "gemm.xg", torch.bfloat16, (M, N)),
          _check(ssq, "gemm.ssq", torch.float32, (M, skinny_parts(N))), stream_handle())
     return NormedRows(xg, ssq, float(eps), resid, g)
+
+
+@dataclass
+class RopeStore:
+    """What the rotate-and-store epilogue of the joined q/k/v projection needs: where the tokens
+    are (``positions``, ``tok_seq``, ``block_table``), the step's cosines and sines ``angles[n,
+    rot / 2, 2]``, the buffer for the rotated q, and the layer's cache."""
+    positions: torch.Tensor
+    tok_seq: torch.Tensor
+    block_table: torch.Tensor
+    angles: torch.Tensor
+    q_out: torch.Tensor
+    cache: "ops.PagedLayerCache"
+    n_heads: int
+    rotated_dims: int
+    write_cache: bool = True
+
+
+def _rope_args(rs: RopeStore, M: int, N: int):
+    c = rs.cache
+    hd, nkv = c.head_dim, c.n_kv_heads
+    if N != (rs.n_heads + 2 * nkv) * hd:
+        raise KernelError(f"rope store: {N} features, expected {(rs.n_heads + 2 * nkv) * hd}")
+    return (_check(rs.positions, "rope.positions", torch.int32, (M,)), _check(rs.tok_seq, "rope.tok_seq", torch.int32, (M,)),
+            _check(rs.block_table, "rope.block_table", torch.int32, (None, None)), rs.block_table.shape[1],
+            _check(rs.angles, "rope.angles", torch.float32, (M, rs.rotated_dims // 2, 2)),
+            _check(rs.q_out, "rope.q_out", torch.bfloat16, (M, rs.n_heads * hd)),
+            _check(c.pool, "rope.cache", torch.bfloat16), rs.n_heads, nkv, hd, c.page_size, c.n_pages,
+            int(rs.rotated_dims), int(bool(rs.write_cache)))
+
+
+def gemm_skinny_rope(x, w_packed, n_features: int, store: RopeStore, row_scale: NormedRows | None = None):
+    """The joined q/k/v projection of at most 16 rows (rows of ``w`` in the order of
+    ``rotary_paired_rows``): q is rotated into ``store.q_out``, k rotated and v as it is into the
+    cache; nothing else is stored."""
+    M, K = x.shape
+    if w_packed.numel() != _packed_size(n_features, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{n_features}, {K}] matrix packs to {_packed_size(n_features, K)}")
+    ssq, parts, eps = _row_scale_args(row_scale, M, K)
+    call("fl_gemm_skinny_rope", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         M, n_features, K, ssq, parts, eps, *_rope_args(store, M, n_features), stream_handle())
+    return store.q_out
+
+
+def gemm_rope_store(x, w: Weight, store: RopeStore, rt=None) -> bool:
+    """The joined q/k/v projection with rotation and stores in the product's kernel, where a kernel
+    for the shape exists; ``False`` if not (the caller then computes the product and calls the
+    rotation kernel).  ``x`` may be ``NormedRows``."""
+    if w.packed is None or store.rotated_dims % 16 or store.cache.head_dim % 16 or store.cache.pool.dtype != torch.bfloat16:
+        return False
+    M, K = x.shape
+    if M <= FUSED_NORM_MAX_ROWS:
+        x, scale = _rows_for(x, w, rt)
+        gemm_skinny_rope(x, w.packed, w.rows, store, row_scale=scale)
+        return True
+    if M > SKINNY_MAX_ROWS and K % 8 == 0 and gemm_tiled_splits(M, w.rows, K) == 1:
+        if isinstance(x, NormedRows):
+            x = x.materialize(rt)
+        gemm_tiled_rope(x, w.packed, w.rows, store)
+        return True
+    return False
+
+
+def gemm_tiled_rope(x, w_packed, n_features: int, store: RopeStore):
+    """``gemm_skinny_rope`` for many rows (shapes whose K is not split)."""
+    M, K = x.shape
+    if w_packed.numel() != _packed_size(n_features, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{n_features}, {K}] matrix packs to {_packed_size(n_features, K)}")
+    call("fl_gemm_tiled_rope", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         M, n_features, K, *_rope_args(store, M, n_features), stream_handle())
+    return store.q_out
 
 
 def gemm_mid_splits(M: int, N: int, K: int) -> int:

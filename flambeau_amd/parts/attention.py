@@ -52,8 +52,19 @@ class PagedGQAAttention(Mixer):
 
     def bind(self, weights, rt):
         self.rt = rt
-        self.w_qkv = rt.prepare_weight(
-            torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0).contiguous())
+        w_qkv = torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0)
+        # With the tuned kernels the rows of a rotated projection are put in an order in which the
+        # product's own kernel can rotate (8 dims, their 8 partners, ...); the rotation kernel reads
+        # that order too.
+        rotary = self.position.rotary_parameters()
+        order = None
+        if rt.tuned and rotary is not None and rotary[0]:
+            from ..kernels.packing import rotary_paired_rows
+            order = rotary_paired_rows(self.n_heads, self.n_kv_heads, self.head_dim, rotary[0])
+        self.paired = order is not None
+        if self.paired:
+            w_qkv = w_qkv[order.to(w_qkv.device)]
+        self.w_qkv = rt.prepare_weight(w_qkv.contiguous())
         self.w_o = rt.prepare_weight(weights["o.weight"])
         self.position.bind({}, rt)
 
@@ -61,18 +72,22 @@ class PagedGQAAttention(Mixer):
         rt, n = self.rt, x.shape[0]
         nh, nkv, hd = self.n_heads, self.n_kv_heads, self.head_dim
         table = step.block_tables[cache.group]
-        qkv = rt.buffer("attn_qkv", n, (nh + 2 * nkv) * hd, torch.float32)
-        rt.gemm(x, self.w_qkv, qkv)
         rotary = self.position.rotary_parameters()
-        angles = None
-        if rotary is None:
-            self.position.apply(qkv, step.positions, nh, nkv, hd)
-            rotary = (0, 1.0)
-        elif rotary[0]:
-            angles = self.position.rotary_table(rt, step)
+        angles = self.position.rotary_table(rt, step) if rotary is not None and rotary[0] else None
         q = rt.buffer("attn_q", n, nh * hd)
-        ops.rope_kv_write(qkv, step.positions, step.tok_seq, table, q, cache.kv, nh, rotary[0], rotary[1],
-                          write_cache=cache.writes, table=angles)
+        fused = False
+        if self.paired and angles is not None:
+            from ..kernels.tuned import RopeStore
+            fused = rt.gemm_rope_store(x, self.w_qkv, RopeStore(step.positions, step.tok_seq, table, angles, q, cache.kv,
+                                                                nh, rotary[0], cache.writes))
+        if not fused:
+            qkv = rt.buffer("attn_qkv", n, (nh + 2 * nkv) * hd, torch.float32)
+            rt.gemm(x, self.w_qkv, qkv)
+            if rotary is None:
+                self.position.apply(qkv, step.positions, nh, nkv, hd)
+                rotary = (0, 1.0)
+            ops.rope_kv_write(qkv, step.positions, step.tok_seq, table, q, cache.kv, nh, rotary[0], rotary[1],
+                              write_cache=cache.writes, table=angles, paired=self.paired)
         out = rt.buffer("attn_out", n, nh * hd)
         if rt.tuned:
             from ..kernels import tuned

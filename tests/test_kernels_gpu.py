@@ -511,6 +511,67 @@ def test_gemm_mid_refuses_what_it_cannot_do():
     assert (out.double() - x40.double() @ w40.double().T).abs().max() < 1e-4
 
 
+@pytest.mark.parametrize("M,nh,nkv,hd,rot,ps,H", [(1, 32, 8, 128, 128, 16, 4096), (8, 4, 2, 16, 16, 8, 64), (16, 5, 5, 32, 16, 16, 80),
+                                                  (300, 6, 2, 64, 64, 16, 96), (2048, 32, 8, 128, 128, 16, 512),
+                                                  (130, 3, 1, 48, 32, 32, 72), (70, 8, 8, 16, 16, 8, 40)])
+def test_gemm_with_rotation_and_stores_in_its_kernel(M, nh, nkv, hd, rot, ps, H):
+    """The joined q/k/v projection with rows in paired order, rotated and stored by the product's own
+    kernel (few rows: skinny; many rows: tiled), against product + rotation kernel apart and float64."""
+    from flambeau_amd.kernels.packing import rotary_paired_rows
+    theta = 1e4
+    N = (nh + 2 * nkv) * hd
+    w = rnd(N, H, dtype=torch.bfloat16, seed=61, scale=0.1)
+    x = rnd(M, H, dtype=torch.bfloat16, seed=62)
+    order = rotary_paired_rows(nh, nkv, hd, rot).to(DEV)
+    W = tuned().prepare_weight(w[order].contiguous())
+    # requests of 1 to 40 tokens somewhere in their contexts, pages in a shuffled order
+    torch.manual_seed(5)
+    pos, seq, starts = [], [], []
+    while len(pos) < M:
+        k = min(int(torch.randint(1, 41, (1,))), M - len(pos))
+        st = int(torch.randint(0, 200, (1,)))
+        pos += range(st, st + k); seq += [len(starts)] * k; starts.append(st + k)
+    width = max(-(-e // ps) for e in starts) + 1
+    n_pages = sum(-(-e // ps) for e in starts) + 2
+    perm = torch.randperm(n_pages).int()
+    table = torch.full((len(starts), width), -1, dtype=torch.int32)
+    used = 0
+    for r, e in enumerate(starts):
+        nb = -(-e // ps)
+        table[r, :nb] = perm[used:used + nb]; used += nb
+    pos_d = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    seq_d = torch.tensor(seq, dtype=torch.int32, device=DEV)
+    table = table.to(DEV)
+    angles = torch.empty(M, rot // 2, 2, dtype=torch.float32, device=DEV)
+    ops().rope_table(pos_d, rot, theta, angles)
+    # apart
+    cache_a = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
+    qkv = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    tuned().gemm(x, W, qkv)
+    q_a = torch.empty(M, nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops().rope_kv_write(qkv, pos_d, seq_d, table, q_a, cache_a, nh, rot, theta, table=angles, paired=True)
+    # in the product's kernel
+    cache_b = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
+    q_b = torch.full((M, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    store = tuned().RopeStore(pos_d, seq_d, table, angles, q_b, cache_b, nh, rot, True)
+    if 16 < M <= 64 or (M > 64 and tuned().gemm_tiled_splits(M, N, H) > 1):
+        assert not tuned().gemm_rope_store(x, W, store)
+        return
+    assert tuned().gemm_rope_store(x, W, store)
+    top = q_a.float().abs().max()
+    assert (q_a.float() - q_b.float()).abs().max() <= 2e-2 * top
+    assert (cache_a.pool.float() - cache_b.pool.float()).abs().max() <= 2e-2 * cache_a.pool.float().abs().max()
+    assert ((cache_a.pool != 0) == (cache_b.pool != 0)).all()          # the same places were written
+    # float64 reference of q
+    ref = (x.double() @ w.double().T)[:, :nh * hd].reshape(M, nh, hd)
+    ref = rope_ref(ref, pos_d, theta, rot)
+    assert (q_b.double().reshape(M, nh, hd) - ref).abs().max() < 1.5e-2 * ref.abs().max()
+    # a layer that reads another layer's cache writes none
+    cache_c = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
+    store_c = tuned().RopeStore(pos_d, seq_d, table, angles, torch.empty_like(q_b), cache_c, nh, rot, False)
+    assert tuned().gemm_rope_store(x, W, store_c) and not cache_c.pool.any() and torch.equal(store_c.q_out, q_b)
+
+
 def test_gemm_dispatch_rows_agree_across_kernels():
     """The same rows through the skinny, the middle and the tiled kernel: equal up to float rounding of sums."""
     w = rnd(512, 1024, dtype=torch.bfloat16, seed=23, scale=0.05)
