@@ -23,7 +23,16 @@ __global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table,
     if (tok < 0 || tok >= V) tok = 0;  // the host rejects such ids before the launch
     const T* src = table + (size_t)tok * H;
     float* dst = out + (size_t)r * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(src[i]);
+    if (H % 4 == 0 && ((uintptr_t)table % 16 == 0) && ((uintptr_t)out % 16 == 0)) {       // four values per load
+        for (int i = 4 * threadIdx.x; i < H; i += 4 * blockDim.x) {
+            f32x4 v;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = to_f32(src[i + u]);
+            *(f32x4*)(dst + i) = v;
+        }
+    } else {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(src[i]);
+    }
 }
 
 extern "C" int fl_embed(const void* table, int dtype, const int* tokens, float* out, int n, int H,
@@ -487,32 +496,47 @@ extern "C" int fl_silu_mul(const void* gu, int in_dtype, void* out, int out_dtyp
 }
 
 // ------------------------------------------------------------------ sampling
-// argmax per row; the first maximum wins (crates/runtime/src/sampling.rs:486-496).
-__global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
-    __shared__ float sv[256];
-    __shared__ int si[256];
+// The better of two (value, index) candidates: the larger value, the smaller index among equals.
+__device__ __forceinline__ void take_better(float& v, int& i, float ov, int oi) {
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+
+// Best candidate of a block of NW waves, in every thread.
+template <int NW>
+__device__ __forceinline__ void block_argmax(float& v, int& i, float* sv, int* si) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) take_better(v, i, __shfl_xor(v, off, 64), __shfl_xor(i, off, 64));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { sv[wave] = v; si[wave] = i; }
+    __syncthreads();
+    v = sv[0]; i = si[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) take_better(v, i, sv[w], si[w]);
+    __syncthreads();
+}
+
+// argmax per row; the first maximum wins (crates/runtime/src/sampling.rs:486-496).  One block of
+// 1024 threads per row; a thread fetches eight values 1024 apart before it compares them, so a
+// row of 32k values costs one round trip to memory, not a hundred.
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
     const float* row = logits + (size_t)blockIdx.x * V;
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += 256) {
-        const float v = row[i];
-        if (v > best) { best = v; bi = i; }
-    }
-    sv[threadIdx.x] = best;
-    si[threadIdx.x] = bi;
-    __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) {
-            const float ov = sv[threadIdx.x + s];
-            const int oi = si[threadIdx.x + s];
-            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
-                sv[threadIdx.x] = ov;
-                si[threadIdx.x] = oi;
-            }
+    for (int base = 0; base < V; base += 8 * 1024) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + u * 1024 + threadIdx.x;
+            v[u] = i < V ? row[i] : -INFINITY;
         }
-        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (v[u] > best) { best = v[u]; bi = base + u * 1024 + threadIdx.x; }      // rising index: the first maximum stays
     }
-    if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0x7fffffff ? 0 : si[0];
+    block_argmax<16>(best, bi, sv, si);
+    if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
 }
 
 // Temperature draw per row: p_i = exp((l_i - max) * inv_t); the token is the first index at
@@ -525,41 +549,47 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
                                                      int* __restrict__ out, int V) {
     __shared__ float red[4];
     __shared__ float chunk_sum[256];
-    __shared__ float sv[256];
-    __shared__ int si[256];
+    __shared__ float sv[4];
+    __shared__ int si[4];
     const int r = blockIdx.x;
     const float* row = logits + (size_t)r * V;
     const float it = inv_temp[r];
-    const int C = (V + 255) / 256;
-    const int lo = threadIdx.x * C, hi = min(V, lo + C);
+    // the maximum (and its first index) with coalesced loads, eight in flight per thread
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = lo; i < hi; ++i) {
-        const float v = row[i];
-        if (v > best) { best = v; bi = i; }
-    }
-    sv[threadIdx.x] = best;
-    si[threadIdx.x] = bi;
-    __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) {
-            const float ov = sv[threadIdx.x + s];
-            const int oi = si[threadIdx.x + s];
-            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
-                sv[threadIdx.x] = ov;
-                si[threadIdx.x] = oi;
-            }
+    for (int base = 0; base < V; base += 8 * 256) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + u * 256 + threadIdx.x;
+            v[u] = i < V ? row[i] : -INFINITY;
         }
-        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (v[u] > best) { best = v[u]; bi = base + u * 256 + threadIdx.x; }
     }
-    const float mx = sv[0];
-    const int amax = si[0] == 0x7fffffff ? 0 : si[0];
+    block_argmax<4>(best, bi, sv, si);
+    const float mx = best;
+    const int amax = bi == 0x7fffffff ? 0 : bi;
+    // for the walk in index order thread t owns the contiguous chunk [t C, (t + 1) C)
+    const int C = (V + 255) / 256;
+    const int lo = threadIdx.x * C, hi = min(V, lo + C);
     if (!(it > 0.f)) {
         if (threadIdx.x == 0) out[r] = amax;
         return;
     }
     float part = 0.f;
-    for (int i = lo; i < hi; ++i) part += expf((row[i] - mx) * it);
+    {
+        int i = lo;
+        for (; i + 8 <= hi; i += 8) {                  // eight loads in flight; the sum keeps index order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = row[i + u];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) part += expf((v[u] - mx) * it);
+        }
+        for (; i < hi; ++i) part += expf((row[i] - mx) * it);
+    }
     chunk_sum[threadIdx.x] = part;
     const float total = block_sum<4>(part, red);
     if (threadIdx.x == 0) {
@@ -603,7 +633,7 @@ extern "C" int fl_feed_tokens(int* tokens, const int* ids, const int* src, int n
 extern "C" int fl_argmax(const float* logits, int* out, int rows, int V, hipStream_t stream) {
     FL_CHECK(rows >= 0 && V > 0, "argmax: bad sizes");
     if (rows == 0) return 0;
-    argmax_kernel<<<rows, 256, 0, stream>>>(logits, out, V);
+    argmax_kernel<<<rows, 1024, 0, stream>>>(logits, out, V);
     FL_LAUNCH_CHECK();
     return 0;
 }
