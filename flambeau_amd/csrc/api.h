@@ -59,6 +59,15 @@ int fl_gemm_skinny_scale_parts(int N, int K, int in_parts);
 int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                 int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_mid_splits(int M, int N, int K);
+// The same fused with the norms around it, as fl_gemm_skinny_fused: a row scale from partial sums of
+// squares, and the product added to the residual stream with the next norm left in factors
+// (out_ssq[M, fl_gemm_mid_parts(N)]; the workspace holds splits * M * N floats, also for one split).
+int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                       int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
+                       float eps, hipStream_t stream);
+int fl_gemm_mid_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                         float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream);
+int fl_gemm_mid_parts(int N);
 
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);

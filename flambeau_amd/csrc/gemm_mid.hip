@@ -20,6 +20,11 @@
 //    never stored), K is a multiple of 32 (other shapes stay with the skinny kernel), and k-steps
 //    beyond the matrix take a zero tile of w.
 //
+// Like the skinny kernel it fuses with the norms around it: a product whose x is bf16(r * g) (g =
+// the norm's weight) multiplies every token's results by rsqrt(sum r^2 / K + eps) (the sums come
+// in parts), and the kernel that adds the K-splits can add them to the residual stream instead and
+// leave bf16(r * g) and the sums of r^2 for the next product: no norm kernel runs between them.
+//
 // The reference's nearest kernel is its batched float GEMV, one block per output row
 // (crates/kernels-hip/src/kernels/dense_gemv_f16_f16_batched.cu:17-63).
 #include "common.h"
@@ -34,10 +39,13 @@ template <> __device__ __forceinline__ void gm_store4<bf16_t>(bf16_t* p, f32x4 v
     *(bf16x4*)p = o;
 }
 
+#define GM_SCALE_PARTS 4          // parts of a token's sum of squares the row scale can add
+
 // GM_NW waves (row groups) per block, GM_CH k-steps per chunk
 template <int MT, int GM_NW, int GM_CH, typename TOut, bool SWIGLU>
 __global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K,
-                                                              int n_steps, int chunks_per_split, int out_cols) {
+                                                              int n_steps, int chunks_per_split, int out_cols,
+                                                              const float* in_ssq, int in_parts, float eps) {
     constexpr int FR = GM_CH * MT;                    // 1 KB operand tiles of x per chunk
     constexpr int XL = (FR + GM_NW - 1) / GM_NW;      // x loads per wave and chunk
     __shared__ __attribute__((aligned(16))) bf16_t slots[2][FR * 512];
@@ -101,6 +109,23 @@ __global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, c
     load_x(x_even, 0);
     load_w(a_even, 0);
     load_x(x_odd, 1);
+    // row scale: x was bf16(r * g); every token's sums are multiplied by rsqrt(mean r^2 + eps) at the
+    // end (a partial sum of a K-split scales the same way).  The parts of the sums of squares are
+    // fetched here, behind the first loads of the operands, and not touched before the loop is over.
+    float ssq_part[MT][GM_SCALE_PARTS];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int p = 0; p < GM_SCALE_PARTS; ++p) ssq_part[mt][p] = 0.f;
+    if (in_ssq) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int tok = min(mt * 16 + li, M - 1);
+#pragma unroll
+            for (int p = 0; p < GM_SCALE_PARTS; ++p)
+                if (p < in_parts) ssq_part[mt][p] = in_ssq[(size_t)tok * in_parts + p];
+        }
+    }
     store_x(x_even, 0);
     __builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0): my part of the slot is written
     asm volatile("s_barrier" ::: "memory");
@@ -138,6 +163,17 @@ __global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, c
     if (i < n_iter) chunk(i, a_even, a_odd, x_odd, x_even);
 
     if (group >= n_groups) return;
+    if (in_ssq) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            float t = ssq_part[mt][0];
+#pragma unroll
+            for (int p = 1; p < GM_SCALE_PARTS; ++p) t += ssq_part[mt][p];
+            const float scale = rsqrtf(t / (float)K + eps);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[mt][r] *= scale;
+        }
+    }
     // lane (token li, quarter g) holds features 16 * group + 4 g .. + 3 of token mt * 16 + li
     if (SWIGLU) {
 #pragma unroll
@@ -187,6 +223,46 @@ __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __res
     out[i] = from_f32<TOut>(s);
 }
 
+// The K-splits added to the residual stream: resid[m, c] += sum_s part[s][m][c] (rising s); xg[m, c] =
+// bf16(resid * g[c]); out_ssq[m, b] = sum of resid^2 over the 4096 columns of block b.  One block
+// per (4096 columns, row).
+#define GM_RED_COLS 4096
+__global__ __launch_bounds__(1024) void gemm_mid_reduce_residual_kernel(const float* __restrict__ part,
+                                                                       float* __restrict__ resid,
+                                                                       const float* __restrict__ g,
+                                                                       bf16_t* __restrict__ xg,
+                                                                       float* __restrict__ out_ssq, int M, int N,
+                                                                       int splits) {
+    __shared__ float red[16];
+    const int row = blockIdx.y, c0 = blockIdx.x * GM_RED_COLS + 4 * threadIdx.x;
+    const size_t total = (size_t)M * N;
+    float sq = 0.f;
+    if (c0 < N) {
+        const size_t at = (size_t)row * N + c0;
+        if (N % 4 == 0) {
+            f32x4 s = *(const f32x4*)(part + at);
+            for (int z = 1; z < splits; ++z) s += *(const f32x4*)(part + (size_t)z * total + at);
+            const f32x4 r = *(const f32x4*)(resid + at) + s;
+            const f32x4 gv = *(const f32x4*)(g + c0);
+            *(f32x4*)(resid + at) = r;
+            const bf16x4 o = {(bf16_t)(r[0] * gv[0]), (bf16_t)(r[1] * gv[1]), (bf16_t)(r[2] * gv[2]), (bf16_t)(r[3] * gv[3])};
+            *(bf16x4*)(xg + at) = o;
+            sq = (r[0] * r[0] + r[1] * r[1]) + (r[2] * r[2] + r[3] * r[3]);
+        } else {
+            for (int u = 0; u < 4 && c0 + u < N; ++u) {
+                float s = part[at + u];
+                for (int z = 1; z < splits; ++z) s += part[(size_t)z * total + at + u];
+                const float r = resid[at + u] + s;
+                resid[at + u] = r;
+                xg[at + u] = from_f32<bf16_t>(r * g[c0 + u]);
+                sq += r * r;
+            }
+        }
+    }
+    sq = block_sum<16>(sq, red);
+    if (threadIdx.x == 0) out_ssq[(size_t)row * gridDim.x + blockIdx.x] = sq;
+}
+
 static int g_mid_splits = 0;             // 0: chosen from the sizes (a fixed number for experiments)
 static int g_mid_waves = 0;              // waves per block: 0 = chosen from the sizes, else 4 or 8
 extern "C" int fl_gemm_mid_set_splits(int s) { g_mid_splits = s; return 0; }
@@ -214,60 +290,78 @@ extern "C" int fl_gemm_mid_splits(int M, int N, int K) {
     return splits;
 }
 
+struct MidScale {              // the row scale of a product whose x is a norm in factors (or none)
+    const float* in_ssq;
+    int in_parts;
+    float eps;
+};
+
 template <int MT, int NW, int CH, typename TOut, bool SWIGLU>
 static void launch_mid_shape(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits, int out_cols,
-                             hipStream_t stream) {
+                             const MidScale& sc, hipStream_t stream) {
     const int n_steps = ceil_div(K, 32);
     const int n_chunks = ceil_div(n_steps, CH);
     const int per = ceil_div(n_chunks, splits);
     dim3 grid(ceil_div(ceil_div(N, 16), NW), splits);
-    gemm_mid_kernel<MT, NW, CH, TOut, SWIGLU><<<grid, NW * 64, 0, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols);
+    gemm_mid_kernel<MT, NW, CH, TOut, SWIGLU><<<grid, NW * 64, 0, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols,
+                                                                            sc.in_ssq, sc.in_parts, sc.eps);
 }
 
 template <int MT, typename TOut, bool SWIGLU>
 static void launch_mid(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits, int out_cols,
-                       hipStream_t stream) {
-    if (mid_waves(N) == 8) launch_mid_shape<MT, 8, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream);
-    else launch_mid_shape<MT, 4, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream);
+                       const MidScale& sc, hipStream_t stream) {
+    if (mid_waves(N) == 8) launch_mid_shape<MT, 8, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream);
+    else launch_mid_shape<MT, 4, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream);
 }
 
 template <typename TOut, bool SWIGLU>
 static void launch_mid_mt(int mt, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits,
-                          int out_cols, hipStream_t stream) {
+                          int out_cols, const MidScale& sc, hipStream_t stream) {
     switch (mt) {
-        case 1: launch_mid<1, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
-        case 2: launch_mid<2, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
-        case 3: launch_mid<3, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
-        default: launch_mid<4, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, stream); break;
+        case 1: launch_mid<1, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
+        case 2: launch_mid<2, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
+        case 3: launch_mid<3, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
+        default: launch_mid<4, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
     }
 }
 
-// epilogue 0: out[M, N] = x w^T; a shape that splits K (fl_gemm_mid_splits > 1) needs a float
-// workspace of splits * M * N values.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up
-// from the N interleaved gate/up rows of w; K is not split then.
-extern "C" int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
-                           int M, int N, int K, int epilogue, int out_cols, hipStream_t stream) {
+static int mid_checks(const void* x, const void* w_packed, int M, int N, int K) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_mid: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_mid: %d rows, at most 64", M);
     FL_CHECK(K % 32 == 0, "gemm_mid: K=%d is no multiple of 32 (whole k-steps of x)", K);
     FL_CHECK((size_t)M * K < ((size_t)1 << 31), "gemm_mid: x of %d x %d values is beyond 32-bit offsets", M, K);
+    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0), "gemm_mid: operands must be 16-byte aligned");
+    return 0;
+}
+
+// epilogue 0: out[M, N] = x w^T; a shape that splits K (fl_gemm_mid_splits > 1) needs a float
+// workspace of splits * M * N values.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up
+// from the N interleaved gate/up rows of w; K is not split then.  in_ssq (or null): [M, in_parts]
+// partial sums of squares of the rows that x was made from; every token's results are multiplied
+// by rsqrt(sum / K + eps).
+extern "C" int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                                  int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
+                                  float eps, hipStream_t stream) {
+    if (mid_checks(x, w_packed, M, N, K)) return -1;
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_mid: unknown output dtype %d", out_dtype);
     FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_mid: unknown epilogue %d", epilogue);
     FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
              "gemm_mid: %d output columns do not fit %d rows of w", out_cols, N);
-    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
-             "gemm_mid: operands must be 16-byte aligned");
+    FL_CHECK((uintptr_t)out % 16 == 0, "gemm_mid: operands must be 16-byte aligned");
+    FL_CHECK(!in_ssq || (in_parts > 0 && in_parts <= GM_SCALE_PARTS), "gemm_mid: a row scale over %d parts (at most %d)",
+             in_parts, GM_SCALE_PARTS);
     if (M == 0) return 0;
     const int mt = ceil_div(M, 16);
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
+    const MidScale sc = {in_ssq, in_parts, eps};
     const int splits = epilogue ? 1 : fl_gemm_mid_splits(M, N, K);
     FL_CHECK(splits == 1 || workspace, "gemm_mid: this shape splits K %d ways and needs a workspace", splits);
     if (epilogue) {
-        if (out_dtype == FL_F32) launch_mid_mt<float, true>(mt, xb, wb, (float*)out, M, N, K, 1, out_cols, stream);
-        else launch_mid_mt<bf16_t, true>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, out_cols, stream);
+        if (out_dtype == FL_F32) launch_mid_mt<float, true>(mt, xb, wb, (float*)out, M, N, K, 1, out_cols, sc, stream);
+        else launch_mid_mt<bf16_t, true>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, out_cols, sc, stream);
     } else if (splits > 1) {
-        launch_mid_mt<float, false>(mt, xb, wb, workspace, M, N, K, splits, N, stream);
+        launch_mid_mt<float, false>(mt, xb, wb, workspace, M, N, K, splits, N, sc, stream);
         FL_LAUNCH_CHECK();
         const size_t total = (size_t)M * N;
         const unsigned rb = (unsigned)((total + 255) / 256);
@@ -276,10 +370,38 @@ extern "C" int fl_gemm_mid(const void* x, const void* w_packed, void* out, float
         else
             gemm_mid_reduce_kernel<bf16_t><<<rb, 256, 0, stream>>>(workspace, (bf16_t*)out, total, splits);
     } else if (out_dtype == FL_F32) {
-        launch_mid_mt<float, false>(mt, xb, wb, (float*)out, M, N, K, 1, N, stream);
+        launch_mid_mt<float, false>(mt, xb, wb, (float*)out, M, N, K, 1, N, sc, stream);
     } else {
-        launch_mid_mt<bf16_t, false>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, N, stream);
+        launch_mid_mt<bf16_t, false>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, N, sc, stream);
     }
     FL_LAUNCH_CHECK();
     return 0;
 }
+
+extern "C" int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                           int M, int N, int K, int epilogue, int out_cols, hipStream_t stream) {
+    return fl_gemm_mid_scaled(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, stream);
+}
+
+// resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_mid_parts(N)] =
+// sums of resid^2 over 4096 columns each: the factors of the norm that follows.  The workspace holds
+// fl_gemm_mid_splits(M, N, K) * M * N floats (also when K is not split).
+extern "C" int fl_gemm_mid_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                                    float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream) {
+    if (mid_checks(x, w_packed, M, N, K)) return -1;
+    FL_CHECK(workspace && resid && g && xg && out_ssq, "gemm_mid_residual: needs workspace, resid, g, xg and out_ssq");
+    FL_CHECK(((uintptr_t)workspace % 16 == 0) && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)g % 16 == 0) &&
+             ((uintptr_t)xg % 8 == 0), "gemm_mid_residual: workspace, resid and g must be 16-byte aligned, xg 8-byte");
+    if (M == 0) return 0;
+    const int splits = fl_gemm_mid_splits(M, N, K);
+    const MidScale none = {nullptr, 0, 0.f};
+    launch_mid_mt<float, false>(ceil_div(M, 16), (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K, splits, N,
+                                none, stream);
+    FL_LAUNCH_CHECK();
+    dim3 grid(ceil_div(N, GM_RED_COLS), M);
+    gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(workspace, resid, g, (bf16_t*)xg, out_ssq, M, N, splits);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int fl_gemm_mid_parts(int N) { return ceil_div(N, GM_RED_COLS); }

@@ -22,6 +22,9 @@ register_signatures({
     "fl_gemm_tiled_rope": [P, P, I, I, I, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
     "fl_gemm_mid": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_mid_splits": [I, I, I],
+    "fl_gemm_mid_scaled": [P, P, P, P, I, I, I, I, I, I, P, I, F, P],
+    "fl_gemm_mid_residual": [P, P, P, I, I, I, P, P, P, P, P],
+    "fl_gemm_mid_parts": [I],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
@@ -36,7 +39,9 @@ def _packed_size(n_rows: int, K: int) -> int:
     return (-(-n_rows // 16) * 16) * (-(-K // 32) * 32)
 
 
-FUSED_NORM_MAX_ROWS = 16     # the fusions of a product with the norms around it take one tile of tokens
+FUSED_NORM_MAX_ROWS = 16     # the skinny kernel's fusions with the norms around it take one tile of tokens
+MID_PART_COLS = 4096         # columns per partial sum of squares that gemm_mid_residual leaves
+MID_SCALE_PARTS = 4          # parts the row scale of gemm_mid can add
 
 
 @dataclass
@@ -189,10 +194,11 @@ def gemm_mid_splits(M: int, N: int, K: int) -> int:
     return load().fl_gemm_mid_splits(M, N, K)
 
 
-def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0):
+def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None):
     """``out = x @ w.T`` for 17 to 64 rows of x (fewer are allowed) and K a multiple of 32: the
     waves of a block share x through LDS.  A narrow matrix splits K and needs ``workspace``
-    (float32, ``gemm_mid_splits(M, N, K) * M * N`` values).  ``swiglu_rows`` as in ``gemm_skinny``."""
+    (float32, ``gemm_mid_splits(M, N, K) * M * N`` values).  ``swiglu_rows`` and ``row_scale`` as in
+    ``gemm_skinny``."""
     M, K = x.shape
     N = swiglu_rows or out.shape[1]
     if w_packed.numel() != _packed_size(N, K):
@@ -200,11 +206,34 @@ def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0):
     splits = 1 if swiglu_rows else gemm_mid_splits(M, N, K)
     if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
         raise KernelError(f"gemm_mid: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
-    call("fl_gemm_mid", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+    ssq, parts, eps = _row_scale_args(row_scale, M, K)
+    call("fl_gemm_mid_scaled", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
          _check(out, "gemm.out", None, (M, None)),
          _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], stream_handle())
+         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps, stream_handle())
     return out
+
+
+def mid_parts(n_features: int) -> int:
+    """Parts in which ``gemm_mid_residual`` leaves the sums of squares of its N features."""
+    return -(-n_features // MID_PART_COLS)
+
+
+def gemm_mid_residual(x, w_packed, resid, g, xg, ssq, eps: float, workspace) -> NormedRows:
+    """``gemm_skinny_residual`` for 17 to 64 rows: the kernel that adds the K-splits adds them to
+    ``resid`` and leaves ``xg`` and ``ssq[m, p]`` (sums over 4096 features each).  ``workspace``:
+    float32, ``gemm_mid_splits(M, N, K) * M * N`` values."""
+    M, K = x.shape
+    N = resid.shape[1]
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    if workspace is None or workspace.numel() < gemm_mid_splits(M, N, K) * M * N:
+        raise KernelError(f"gemm_mid_residual: needs a workspace of {gemm_mid_splits(M, N, K) * M * N} floats")
+    call("fl_gemm_mid_residual", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(workspace, "gemm.workspace", torch.float32), M, N, K, _check(resid, "gemm.resid", torch.float32, (M, N)),
+         _check(g, "gemm.g", torch.float32, (N,)), _check(xg, "gemm.xg", torch.bfloat16, (M, N)),
+         _check(ssq, "gemm.ssq", torch.float32, (M, mid_parts(N))), stream_handle())
+    return NormedRows(xg, ssq, float(eps), resid, g)
 
 
 def gemm_tiled_splits(M: int, N: int, K: int) -> int:
@@ -235,19 +264,31 @@ def _rows_for(x, w: Weight, rt):
     skinny kernel runs, else the rows are made."""
     if not isinstance(x, NormedRows):
         return x, None
-    if w.packed is not None and x.shape[0] <= FUSED_NORM_MAX_ROWS and x.shape[1] % 8 == 0:
+    M, K = x.shape
+    if w.packed is not None and M <= FUSED_NORM_MAX_ROWS and K % 8 == 0:
         from .library import load
         parts = x.ssq.shape[1]
-        if parts <= load().fl_gemm_skinny_scale_parts(w.packed_rows, x.shape[1], parts):
+        if parts <= load().fl_gemm_skinny_scale_parts(w.packed_rows, K, parts):
             return x.xg, x
+    if w.packed is not None and FUSED_NORM_MAX_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0 \
+            and x.ssq.shape[1] <= MID_SCALE_PARTS:
+        return x.xg, x
     return x.materialize(rt), None
+
+
+def _split_workspace(rt, n_floats: int, device):
+    """Room for the partial sums of a product that splits K: one buffer for all shapes, in rows of
+    4096 floats."""
+    if rt is None:
+        return torch.empty(n_floats, dtype=torch.float32, device=device)
+    return rt.buffer("gemm_splitk", -(-n_floats // 4096), 4096, torch.float32, max_rows=1 << 20).view(-1)
 
 
 def gemm(x, w: Weight, out, rt=None):
     """``out = x @ w.T`` with the best kernel that takes the shape; ``x`` may be ``NormedRows``."""
     x, scale = _rows_for(x, w, rt)
     M, K = x.shape
-    if scale is not None:
+    if scale is not None and M <= FUSED_NORM_MAX_ROWS:
         return gemm_skinny(x, w.packed, out, row_scale=scale)
     if w.packed is not None and not w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
         N = w.rows
@@ -255,14 +296,10 @@ def gemm(x, w: Weight, out, rt=None):
         if M <= SKINNY_MAX_ROWS and not mid:
             return gemm_skinny(x, w.packed, out)
         splits = gemm_mid_splits(M, N, K) if mid else gemm_tiled_splits(M, N, K)
-        workspace = None
-        if splits > 1:
-            if rt is None:
-                workspace = torch.empty(splits * M * N, dtype=torch.float32, device=x.device)
-            else:       # one buffer for all shapes, in rows of 4096 floats
-                workspace = rt.buffer("gemm_splitk", -(-splits * M * N // 4096), 4096, torch.float32,
-                                      max_rows=1 << 20).view(-1)
-        return (gemm_mid if mid else gemm_tiled)(x, w.packed, out, workspace)
+        workspace = _split_workspace(rt, splits * M * N, x.device) if splits > 1 else None
+        if mid:
+            return gemm_mid(x, w.packed, out, workspace, row_scale=scale)
+        return gemm_tiled(x, w.packed, out, workspace)
     if w.rowmajor is None:
         raise KernelError(f"gemm: no kernel for {M} rows of a packed [{w.rows}, {w.cols}] matrix")
     return ops.gemm_plain(x, w.rowmajor, out)
@@ -273,7 +310,8 @@ def gemm_swiglu(x, w: Weight, out, rt):
     x, scale = _rows_for(x, w, rt)
     M, K = x.shape
     if scale is not None and w.swiglu_cols:
-        return gemm_skinny(x, w.packed, out, swiglu_rows=w.packed_rows, row_scale=scale)
+        kernel = gemm_skinny if M <= FUSED_NORM_MAX_ROWS else gemm_mid
+        return kernel(x, w.packed, out, swiglu_rows=w.packed_rows, row_scale=scale)
     if scale is not None:
         x = scale.materialize(rt)
     if w.packed is not None and w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:

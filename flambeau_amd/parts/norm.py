@@ -26,7 +26,7 @@ class RMSNorm(Norm):
         return ops.rmsnorm(x, self.weight, out, self.eps, delta=delta, store_sum=store_sum, rows=rows)
 
     def after_product(self, rt, resid, product):
-        """For a few rows (a decode step) the product's kernel adds its result to the stream and
+        """For up to 64 rows (a decode step) the product's kernel adds its result to the stream and
         leaves the norm in factors: x * w in the compute dtype and the sums of squares in parts.
         The product that follows multiplies by rsqrt(mean + eps) itself: no norm kernel runs."""
         if not rt.tuned:
@@ -34,9 +34,17 @@ class RMSNorm(Norm):
         from ..kernels import tuned
         n, H = resid.shape
         w, x = product.weight, product.x
-        if (n > tuned.FUSED_NORM_MAX_ROWS or w.packed is None or w.swiglu_cols or isinstance(x, tuned.NormedRows)
-                or x.dtype != torch.bfloat16 or x.shape[1] % 8 or H % 8):
+        if (w.packed is None or w.swiglu_cols or isinstance(x, tuned.NormedRows) or x.dtype != torch.bfloat16
+                or x.shape[1] % 8 or H % 8):
             return None
+        K = x.shape[1]
         xg = rt.buffer("normed_xg", n, H)
-        ssq = rt.buffer("normed_ssq", n, tuned.skinny_parts(H), torch.float32)
-        return tuned.gemm_skinny_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps)
+        if n <= tuned.FUSED_NORM_MAX_ROWS:
+            ssq = rt.buffer("normed_ssq", n, tuned.skinny_parts(H), torch.float32)
+            return tuned.gemm_skinny_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps)
+        if n <= tuned.SKINNY_MAX_ROWS and K % 32 == 0 and H % 32 == 0:
+            # 17 to 64 rows: the kernel that adds the K-splits of the product does it
+            ssq = rt.buffer("normed_ssq_mid", n, tuned.mid_parts(H), torch.float32)
+            workspace = tuned._split_workspace(rt, tuned.gemm_mid_splits(n, H, K) * n * H, x.device)
+            return tuned.gemm_mid_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps, workspace)
+        return None

@@ -123,10 +123,12 @@ def test_gemm_skinny_against_plain(out_dtype, M, N, K):
 
 
 @pytest.mark.parametrize("M,H,N2,I,eps", [(1, 4096, 6144, 512, 1e-5), (8, 4096, 32768, 14336, 1e-5), (16, 72, 40, 104, 1e-2),
-                                            (3, 136, 250, 40, 1e-6), (5, 64, 16, 8, 1e-5)])
-def test_gemm_skinny_fused_with_the_norms_around_it(M, H, N2, I, eps):
+                                            (3, 136, 250, 40, 1e-6), (5, 64, 16, 8, 1e-5),
+                                            (64, 4096, 6144, 14336, 1e-5), (17, 96, 40, 64, 1e-3), (40, 2080, 300, 160, 1e-5)])
+def test_gemm_fused_with_the_norms_around_it(M, H, N2, I, eps):
     """resid += a W1^T in the product's epilogue, norm(resid) W2^T through the row scale of the next
-    product, against the same chain in float64; and the SwiGLU epilogue after a row scale."""
+    product, against the same chain in float64; and the SwiGLU epilogue after a row scale.  Up to 16
+    rows in the skinny kernel, 17 to 64 in the kernel that shares x through LDS."""
     from flambeau_amd.kernels.packing import pack_weight
     a = rnd(M, I, dtype=torch.bfloat16, seed=51)
     w1 = rnd(H, I, dtype=torch.bfloat16, seed=52, scale=0.05)
@@ -135,22 +137,27 @@ def test_gemm_skinny_fused_with_the_norms_around_it(M, H, N2, I, eps):
     resid0 = rnd(M, H, seed=55)
     resid = resid0.clone()
     xg = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ssq = torch.full((M, tuned().skinny_parts(H)), float("nan"), dtype=torch.float32, device=DEV)
-    rows = tuned().gemm_skinny_residual(a, pack_weight(w1), resid, g, xg, ssq, eps)
+    if M <= 16:
+        ssq = torch.full((M, tuned().skinny_parts(H)), float("nan"), dtype=torch.float32, device=DEV)
+        rows = tuned().gemm_skinny_residual(a, pack_weight(w1), resid, g, xg, ssq, eps)
+    else:
+        ssq = torch.full((M, tuned().mid_parts(H)), float("nan"), dtype=torch.float32, device=DEV)
+        ws = torch.full((tuned().gemm_mid_splits(M, H, I) * M * H,), float("nan"), dtype=torch.float32, device=DEV)
+        rows = tuned().gemm_mid_residual(a, pack_weight(w1), resid, g, xg, ssq, eps, ws)
     r_ref = resid0.double() + a.double() @ w1.double().T
     assert (resid.double() - r_ref).abs().max() < 1e-5 * r_ref.abs().max()
     assert (ssq.double().sum(1) - (r_ref ** 2).sum(1)).abs().max() < 1e-5 * (r_ref ** 2).sum(1).max()
     assert (xg.double() - r_ref * g.double()).abs().max() < 5e-3 * (r_ref * g.double()).abs().max()
     normed = r_ref * torch.rsqrt((r_ref ** 2).mean(1, keepdim=True) + eps) * g.double()
     ref = normed @ w2.double().T
+    class Rt:
+        def buffer(self, name, n, cols, dtype=torch.bfloat16, max_rows=None):
+            return torch.empty(n, cols, dtype=dtype, device=DEV)
     W2 = tuned().prepare_weight(w2)
     got = torch.full((M, N2), float("nan"), dtype=torch.float32, device=DEV)
-    tuned().gemm(rows, W2, got)
+    tuned().gemm(rows, W2, got, Rt())
     assert (got.double() - ref).abs().max() < 6e-3 * ref.abs().max()
     # the rows themselves, for kernels that do not take the factors
-    class Rt:
-        def buffer(self, name, n, cols, dtype=torch.bfloat16):
-            return torch.empty(n, cols, dtype=dtype, device=DEV)
     made = rows.materialize(Rt())
     assert (made.double() - normed).abs().max() < 5e-3 * normed.abs().max()
     if N2 % 32 == 0:
