@@ -1,6 +1,8 @@
 // Shared device helpers for the gfx950 kernels: storage types, conversions,
 // wave64 reductions, the paged-cache address rule and host-side error reporting.
 #pragma once
+#include <utility>
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -10,6 +12,17 @@
 // dtype codes of the C interface
 #define FL_F32 0
 #define FL_BF16 1
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index
+// is a constant in every turn.
+template <int N, typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl<N>(f, std::make_integer_sequence<int, N>{});
+}
 
 typedef __bf16 bf16_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4;

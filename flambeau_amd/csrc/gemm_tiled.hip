@@ -33,6 +33,21 @@
 #define TG_PLAIN 0                       // epilogues
 #define TG_SWIGLU 1
 #define TG_ROPE 2
+#define TG_RESIDUAL 3
+
+// Fusion with the norms around a product (as in gemm_skinny.hip).  in_ssq: x is bf16(r * g) and every
+// token's results are multiplied by rsqrt(sum_p in_ssq[m][p] / K + eps).  TG_RESIDUAL: nothing is
+// stored in out; resid[M, N] += the product, xg = bf16(resid * g), out_ssq[m][tile of features] =
+// the block's sum of resid^2.
+struct TiledFusion {
+    const float* in_ssq;
+    int in_parts;
+    float eps;
+    float* resid;
+    const float* g;
+    bf16_t* xg;
+    float* out_ssq;
+};
 
 
 template <typename TOut>
@@ -56,13 +71,14 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
                                                             const bf16_t* __restrict__ wp,
                                                             TOut* __restrict__ out, int M, int N, int K,
                                                             int n_steps, int steps_per_split, int out_cols,
-                                                            RopeStore rs) {
+                                                            RopeStore rs, TiledFusion fu) {
     constexpr int NW = 2 * WT;                        // waves: 2 along the features, WT along the tokens
     constexpr int NTF = 2 * FT, NTT = WT * TT;        // operand tiles of the block: features, tokens
     constexpr int TILES = NTF + NTT;                  // 1 KB tiles per stage
     constexpr int LPS = TILES / NW;                   // load instructions per wave and stage
     static_assert(TILES % NW == 0, "tiles must divide among the waves");
     extern __shared__ __attribute__((aligned(16))) bf16_t ring[];      // [NS][TILES][512]
+    __shared__ float s_scale[NTT * 16];                               // row scale of the block's tokens
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -114,16 +130,17 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
     const int x_kmax = K - 8;                         // last whole 16-byte chunk of a row of x
     // operand lane (token i = lane % 16, k-piece g = lane / 16) finds its 16 bytes of an x tile here
     const int x_read = 32 * (lane & 15) + 8 * ((lane >> 4) ^ (((lane & 15) >> 1) & 3));
-    auto issue = [&](int i) {                         // loads of stage i (k-step s_begin + i) into slot i % NS
+    // load c of this wave's LPS loads of stage i (k-step s_begin + i) into slot i % NS: its LW tiles of
+    // w first, then its LX tiles of x
+    auto issue_one = [&](int i, auto c_) {
+        constexpr int c = decltype(c_)::value;
         bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
-#pragma unroll
-        for (int u = 0; u < LW; ++u) {
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)wsrc[u],
-                                             (__attribute__((address_space(3))) void*)(slot + (wave * LW + u) * 512), 16, 0, 0);
-            wsrc[u] += 512;
-        }
-#pragma unroll
-        for (int u = 0; u < LX; ++u) {
+        if constexpr (c < LW) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)wsrc[c],
+                                             (__attribute__((address_space(3))) void*)(slot + (wave * LW + c) * 512), 16, 0, 0);
+            wsrc[c] += 512;
+        } else {
+            constexpr int u = c - LW;
             const bf16_t* g = xsrc[u];
             if (!KWHOLE) {                            // K is no multiple of 32: keep the last pieces inside the row
                 const int k = (s_begin + i) * 32 + x_piece;
@@ -134,10 +151,50 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
             xsrc[u] += 32;
         }
     };
+    auto issue = [&](int i) {                         // all loads of stage i
+        static_for<LPS>([&](auto c) { issue_one(i, c); });
+    };
+
+    // One block per CU has nothing that runs beside its epilogue, so the residual epilogue's reads
+    // are issued here, ahead of all other loads, and wait in registers (there is room: half the
+    // registers of the CU belong to each wave).
+    constexpr bool PREFETCH = EPI == TG_RESIDUAL && OCC == 1;
+    const int j = lane & 15, g = lane >> 4;
+    f32x4 pre[PREFETCH ? FT : 1][PREFETCH ? TT : 1];
+    if (PREFETCH) {
+#pragma unroll
+        for (int tb = 0; tb < TT; ++tb)
+#pragma unroll
+            for (int ta = 0; ta < FT; ++ta) {
+                const int tok = min(m0 + (wt * TT + tb) * 16 + j, M - 1);
+                const int f0 = min(n0 + (wf * FT + ta) * 16 + 4 * g, N - 4);
+                pre[PREFETCH ? ta : 0][PREFETCH ? tb : 0] = *(const f32x4*)(fu.resid + (size_t)tok * N + f0);
+            }
+    }
 
 #pragma unroll
     for (int i = 0; i < NS - 1; ++i)
         if (i < n_iter) issue(i);
+    if (fu.in_ssq) {
+        // Every token's factor rsqrt(mean r^2 + eps) while the first stages are on their way: eight
+        // lanes add a token's parts (lane l parts l, l + 8, ...), then each other's sums.
+        const int lp = tid & 7;
+#pragma unroll
+        for (int t = tid >> 3; t < NTT * 16; t += NW * 8) {
+            const float* parts = fu.in_ssq + (size_t)min(m0 + t, M - 1) * fu.in_parts;
+            const int last = fu.in_parts - 1;
+            float sum = 0.f;
+            for (int p = lp; p <= last; p += 32) {
+                const float v0 = parts[p], v1 = parts[min(p + 8, last)], v2 = parts[min(p + 16, last)],
+                            v3 = parts[min(p + 24, last)];
+                sum += (v0 + (p + 8 <= last ? v1 : 0.f)) + ((p + 16 <= last ? v2 : 0.f) + (p + 24 <= last ? v3 : 0.f));
+            }
+            sum += __shfl_xor(sum, 1, 64);
+            sum += __shfl_xor(sum, 2, 64);
+            sum += __shfl_xor(sum, 4, 64);
+            if (lp == 0) s_scale[t] = rsqrtf(sum / (float)K + fu.eps);
+        }
+    }
     auto read_operands = [&](bf16x8 (&a)[FT], bf16x8 (&b)[TT], int i) {
         const bf16_t* slot = ring + (size_t)(i % NS) * TILES * 512;
 #pragma unroll
@@ -169,7 +226,8 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
         for (int i = 0; i < n_iter; ++i) {
             wait_stage(i, Behind1{});
             // the operand reads of this stage go first (x, then w in the order the products want
-            // them); the loads of a later stage are issued while they are on their way
+            // them); the loads of a later stage are issued while they are on their way (spreading
+            // them among the products instead gained nothing)
             bf16x8 a[FT], b[TT];
             read_operands(a, b, i);
             __builtin_amdgcn_sched_barrier(0);
@@ -180,18 +238,78 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
     }
     // the loads are done (the last stage waited for vmcnt(0)); LDS is not touched again
 
-    const int j = lane & 15, g = lane >> 4;
-    if (EPI == TG_ROPE) {
-        // the joined q/k/v projection: rotate, store q and the cache rows (rope_store.h)
+    if (fu.in_ssq) {
+        __syncthreads();                                              // s_scale is written
+#pragma unroll
+        for (int tb = 0; tb < TT; ++tb) {
+            const float scale = s_scale[(wt * TT + tb) * 16 + j];
+#pragma unroll
+            for (int ta = 0; ta < FT; ++ta)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[ta][tb][r] *= scale;
+        }
+    }
+    if (EPI == TG_RESIDUAL) {
+        // resid += product; xg = bf16(resid * g); the block's sum of resid^2 per token: this wave's
+        // features, then the four lanes of a token, then the two waves that share the tokens
+        float* s_part = (float*)ring;                                 // [2][NTT * 16]
+        f32x4 gain[FT];                                               // the norm's weights of this lane's features
+#pragma unroll
+        for (int ta = 0; ta < FT; ++ta) gain[ta] = *(const f32x4*)(fu.g + min(n0 + (wf * FT + ta) * 16 + 4 * g, N - 4));
+        __syncthreads();                                              // the ring is no longer read
 #pragma unroll
         for (int tb = 0; tb < TT; ++tb) {
             const int tok = m0 + (wt * TT + tb) * 16 + j;
-            TokenPlace place = {-1, 0};
-            if (tok < M) place = rope_token_place(rs, tok);
+            float sq = 0.f;
+            f32x4 old[FT];                                            // the token's residual values, read together
+#pragma unroll
+            for (int ta = 0; ta < FT; ++ta) {
+                const int f0 = min(n0 + (wf * FT + ta) * 16 + 4 * g, N - 4);
+                old[ta] = PREFETCH ? pre[PREFETCH ? ta : 0][PREFETCH ? tb : 0]
+                                   : *(const f32x4*)(fu.resid + (size_t)min(tok, M - 1) * N + f0);
+            }
 #pragma unroll
             for (int ta = 0; ta < FT; ++ta) {
                 const int f0 = n0 + (wf * FT + ta) * 16 + 4 * g;
-                rope_store4(rs, tok, place, f0, g, acc[ta][tb], tok < M && f0 < N);
+                if (tok < M && f0 < N) {
+                    const f32x4 nr = old[ta] + acc[ta][tb];
+                    const f32x4 gv = gain[ta];
+                    *(f32x4*)(fu.resid + (size_t)tok * N + f0) = nr;
+                    const bf16x4 o = {(bf16_t)(nr[0] * gv[0]), (bf16_t)(nr[1] * gv[1]), (bf16_t)(nr[2] * gv[2]), (bf16_t)(nr[3] * gv[3])};
+                    *(bf16x4*)(fu.xg + (size_t)tok * N + f0) = o;
+                    sq += (nr[0] * nr[0] + nr[1] * nr[1]) + (nr[2] * nr[2] + nr[3] * nr[3]);
+                }
+            }
+            sq += __shfl_xor(sq, 16, 64);
+            sq += __shfl_xor(sq, 32, 64);
+            if (g == 0) s_part[wf * (NTT * 16) + (wt * TT + tb) * 16 + j] = sq;
+        }
+        __syncthreads();
+        for (int t = tid; t < NTT * 16; t += NW * 64)
+            if (m0 + t < M) fu.out_ssq[(size_t)(m0 + t) * n_ft + tile_f] = s_part[t] + s_part[NTT * 16 + t];
+        return;
+    }
+    if (EPI == TG_ROPE) {
+        // the joined q/k/v projection: rotate, store q and the cache rows (rope_store.h).  What the
+        // epilogue looks up (places, angles) is loaded in batches, each with one wait.
+        int toks[TT];
+        TokenPlace places[TT];
+#pragma unroll
+        for (int tb = 0; tb < TT; ++tb) toks[tb] = m0 + (wt * TT + tb) * 16 + j;
+        rope_token_places<TT>(rs, toks, M, places);
+#pragma unroll
+        for (int tb = 0; tb < TT; ++tb) {
+            const int tok = toks[tb];
+            RopeAngles an[FT];
+            if (rs.rot) {                                             // (no table without rotated dims)
+#pragma unroll
+                for (int ta = 0; ta < FT; ++ta)
+                    an[ta] = rope_angles(rs, min(tok, M - 1), n0 + (wf * FT + ta) * 16 + 4 * g, g);
+            }
+#pragma unroll
+            for (int ta = 0; ta < FT; ++ta) {
+                const int f0 = n0 + (wf * FT + ta) * 16 + 4 * g;
+                rope_store4<true>(rs, tok, places[tb], f0, g, acc[ta][tb], tok < M && f0 < N, an[ta]);
             }
         }
         return;
@@ -246,7 +364,7 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
 
 template <int FT, int TT, int WT, int NS, int OCC, typename TOut, int EPI>
 static void launch_async(int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N,
-                         int K, int n_steps, int per, int out_cols, const RopeStore& rs) {
+                         int K, int n_steps, int per, int out_cols, const RopeStore& rs, const TiledFusion& fu) {
     constexpr int LDS = NS * (2 * FT + WT * TT) * 1024;
     static bool configured = false;
     auto whole = gemm_async_kernel<FT, TT, WT, NS, OCC, TOut, EPI, true>;
@@ -259,7 +377,7 @@ static void launch_async(int splits, hipStream_t stream, const bf16_t* x, const 
     auto kern = (K % 32 == 0) ? whole : ragged;
     const int tiles = ceil_div(N, 2 * FT * 16) * ceil_div(M, WT * TT * 16);
     dim3 grid(ceil_div(tiles, 8) * 8, 1, splits);
-    kern<<<grid, 128 * WT, LDS, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols, rs);
+    kern<<<grid, 128 * WT, LDS, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu);
 }
 
 template <typename TOut>
@@ -278,15 +396,25 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 static int g_tiled_variant = 0;
 extern "C" int fl_gemm_tiled_set_variant(int v) { g_tiled_variant = v; return 0; }
 
+static int tiled_variant(int variant, int splits, int M, int N) {
+    // 256 x 128 where that fills the chip (and for few rows), else 128 x 256
+    if (variant == 3 || variant == 6) return variant;
+    return (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320 || M < 192) ? 3 : 6;
+}
+
+// Parts in which the residual epilogue leaves a token's sum of squares: one per tile of features.
+extern "C" int fl_gemm_tiled_parts(int M, int N) {
+    return ceil_div(N, tiled_variant(g_tiled_variant, 1, M, N) == 6 ? 128 : 256);
+}
+
 template <typename TOut, int EPI>
 static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out,
-                         int M, int N, int K, int n_steps, int per, int out_cols, const RopeStore& rs) {
-    // 256 x 128 where that fills the chip (and for few rows), else 128 x 256
-    if (variant == 0) variant = (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320 || M < 192) ? 3 : 6;
-    if (variant == 6)
-        launch_async<4, 4, 4, 4, 1, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs);
+                         int M, int N, int K, int n_steps, int per, int out_cols, const RopeStore& rs,
+                         const TiledFusion& fu = TiledFusion{}) {
+    if (tiled_variant(variant, splits, M, N) == 6)
+        launch_async<4, 4, 4, 4, 1, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu);
     else
-        launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs);
+        launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu);
 }
 
 // How many ways K is split for a product of this shape: 1 if the grid fills the chip.
@@ -300,9 +428,12 @@ extern "C" int fl_gemm_tiled_splits(int M, int N, int K) {
 
 // epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up from the
 // N interleaved gate/up rows of w (K is not split then).
-extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace,
-                             int out_dtype, int M, int N, int K, int epilogue, int out_cols,
-                             hipStream_t stream) {
+// epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up from the
+// N interleaved gate/up rows of w (K is not split then).  in_ssq (or null): [M, in_parts] partial sums of
+// squares of the rows that x was made from; every token's results are multiplied by rsqrt(sum / K + eps).
+extern "C" int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* out, float* workspace,
+                                    int out_dtype, int M, int N, int K, int epilogue, int out_cols,
+                                    const float* in_ssq, int in_parts, float eps, hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_tiled: unknown output dtype %d", out_dtype);
@@ -311,6 +442,7 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
              "gemm_tiled: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
              "gemm_tiled: operands must be 16-byte aligned");
+    FL_CHECK(!in_ssq || in_parts > 0, "gemm_tiled: a row scale over %d parts", in_parts);
     if (M == 0) return 0;
     const int n_steps = ceil_div(K, 32);
     const int splits = epilogue ? 1 : fl_gemm_tiled_splits(M, N, K);
@@ -320,13 +452,14 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
     const bf16_t* wb = (const bf16_t*)w_packed;
     const int v = g_tiled_variant;
     const RopeStore none{};
+    const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
     if (epilogue) {
         if (out_dtype == FL_F32)
-            launch_tiled<float, TG_SWIGLU>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, out_cols, none);
+            launch_tiled<float, TG_SWIGLU>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, out_cols, none, fu);
         else
-            launch_tiled<bf16_t, TG_SWIGLU>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, out_cols, none);
+            launch_tiled<bf16_t, TG_SWIGLU>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, out_cols, none, fu);
     } else if (splits > 1) {
-        launch_tiled<float, TG_PLAIN>(v, splits, stream, xb, wb, workspace, M, N, K, n_steps, per, N, none);
+        launch_tiled<float, TG_PLAIN>(v, splits, stream, xb, wb, workspace, M, N, K, n_steps, per, N, none, fu);
         FL_LAUNCH_CHECK();
         const size_t total = (size_t)M * N;
         const unsigned rb = (unsigned)((total + 255) / 256);
@@ -335,10 +468,37 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
         else
             gemm_splitk_reduce_kernel<bf16_t><<<rb, 256, 0, stream>>>(workspace, (bf16_t*)out, total, splits);
     } else if (out_dtype == FL_F32) {
-        launch_tiled<float, TG_PLAIN>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, N, none);
+        launch_tiled<float, TG_PLAIN>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, N, none, fu);
     } else {
-        launch_tiled<bf16_t, TG_PLAIN>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, N, none);
+        launch_tiled<bf16_t, TG_PLAIN>(v, 1, stream, xb, wb, (bf16_t*)out, M, N, K, n_steps, per, N, none, fu);
     }
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace,
+                             int out_dtype, int M, int N, int K, int epilogue, int out_cols,
+                             hipStream_t stream) {
+    return fl_gemm_tiled_scaled(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, stream);
+}
+
+// resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_tiled_parts(M, N)] =
+// the sums of resid^2 over the feature tiles: the factors of the norm that follows.  Only for shapes
+// whose K is not split.
+extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, int M, int N, int K, float* resid,
+                                      const float* g, void* xg, float* out_ssq, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_residual: bad sizes M=%d N=%d K=%d", M, N, K);
+    FL_CHECK(K % 8 == 0, "gemm_tiled_residual: K=%d is no multiple of 8 (16-byte loads)", K);
+    FL_CHECK(N % 4 == 0, "gemm_tiled_residual: N=%d is no multiple of 4 (16-byte accesses to the residual rows)", N);
+    FL_CHECK(resid && g && xg && out_ssq, "gemm_tiled_residual: needs resid, g, xg and out_ssq");
+    FL_CHECK(fl_gemm_tiled_splits(M, N, K) == 1, "gemm_tiled_residual: this shape splits K");
+    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)resid % 16 == 0) &&
+             ((uintptr_t)g % 16 == 0) && ((uintptr_t)xg % 8 == 0), "gemm_tiled_residual: operands must be aligned (16 bytes, xg 8)");
+    if (M == 0) return 0;
+    const int n_steps = ceil_div(K, 32);
+    const TiledFusion fu = {nullptr, 0, 0.f, resid, g, (bf16_t*)xg, out_ssq};
+    launch_tiled<float, TG_RESIDUAL>(g_tiled_variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, resid, M, N, K,
+                                     n_steps, n_steps, N, RopeStore{}, fu);
     FL_LAUNCH_CHECK();
     return 0;
 }
@@ -346,11 +506,12 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
 // The joined q/k/v projection of many rows with its rows in paired order: q is rotated and written to
 // q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens' positions; cs[M,
 // rot / 2, 2] are the step's cosines and sines.  Only for shapes whose K is not split
-// (fl_gemm_tiled_splits == 1).
-extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const int* positions,
-                                  const int* tok_seq, const int* block_table, int max_blocks, const float* cs,
-                                  void* q_out, void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages,
-                                  int rot, int write_cache, hipStream_t stream) {
+// (fl_gemm_tiled_splits == 1).  in_ssq as in fl_gemm_tiled_scaled.
+extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
+                                  int in_parts, float eps, const int* positions, const int* tok_seq,
+                                  const int* block_table, int max_blocks, const float* cs, void* q_out,
+                                  void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages, int rot,
+                                  int write_cache, hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_rope: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled_rope: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(positions && tok_seq && block_table && cs && q_out && cache_base,
@@ -359,12 +520,14 @@ extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, in
              "gemm_tiled_rope: %d features with heads of %d (%d rotated), %d + 2 x %d heads", N, hd, rot, nh, nkv);
     FL_CHECK(fl_gemm_tiled_splits(M, N, K) == 1, "gemm_tiled_rope: this shape splits K");
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0), "gemm_tiled_rope: operands must be 16-byte aligned");
+    FL_CHECK(!in_ssq || in_parts > 0, "gemm_tiled_rope: a row scale over %d parts", in_parts);
     if (M == 0) return 0;
     const RopeStore rs = {positions, tok_seq, block_table, max_blocks, (const float2*)cs, (bf16_t*)q_out,
                           PagedCache{cache_base, nkv, page_size, hd, n_pages}, nh, rot, write_cache};
+    const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
     const int n_steps = ceil_div(K, 32);
     launch_tiled<bf16_t, TG_ROPE>(g_tiled_variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)q_out,
-                                  M, N, K, n_steps, n_steps, N, rs);
+                                  M, N, K, n_steps, n_steps, N, rs, fu);
     FL_LAUNCH_CHECK();
     return 0;
 }

@@ -40,11 +40,53 @@ __device__ __forceinline__ TokenPlace rope_token_place(const RopeStore& rs, int 
     return tp;
 }
 
+// Where the tokens of COUNT lanes-rows go, all look-ups of one kind issued together (one wait for
+// all of them instead of one per token).  toks beyond n_tokens are clamped and get page -1.
+template <int COUNT>
+__device__ __forceinline__ void rope_token_places(const RopeStore& rs, const int (&toks)[COUNT], int n_tokens,
+                                                  TokenPlace (&places)[COUNT]) {
+    const int ps = rs.cache.page_size;
+    int pos[COUNT], seq[COUNT];
+#pragma unroll
+    for (int i = 0; i < COUNT; ++i) {
+        const int t = min(toks[i], n_tokens - 1);
+        pos[i] = rs.positions[t];
+        seq[i] = rs.write_cache ? rs.tok_seq[t] : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < COUNT; ++i) {
+        int page = rs.write_cache ? rs.block_table[(size_t)seq[i] * rs.max_blocks + pos[i] / ps] : -1;
+        if (page >= rs.cache.n_pages || toks[i] >= n_tokens) page = -1;
+        places[i].page = page;
+        places[i].row = pos[i] % ps;
+    }
+}
+
+struct RopeAngles {           // cosine and sine of a lane's four pairs: (c0, s0, c1, s1), (c2, s2, c3, s3)
+    float4 a, b;
+};
+
+// The angles of the four pairs of lane (token, g) at features f0 .. f0 + 3.  The address is clamped
+// into the token's row, so this may be called (and its result ignored) for features that are not
+// rotated; tok must be a valid token and rs.rot at least 8.
+__device__ __forceinline__ RopeAngles rope_angles(const RopeStore& rs, int tok, int f0, int g) {
+    const int hd = rs.cache.head_dim;
+    const int within = f0 % hd, half = rs.rot >> 1;
+    const int pair0 = min(8 * (within >> 4) + 4 * (g & 1), half - 4);
+    const float4* t = (const float4*)(rs.cs + (size_t)tok * half + pair0);
+    RopeAngles an;
+    an.a = t[0];
+    an.b = t[1];
+    return an;
+}
+
 // v: this lane's four features f0 .. f0 + 3 (f0 = 16 * group + 4 g, in paired order) of token tok;
 // every lane of the wave calls this together (the exchange needs all of them), `live` says whether
-// this lane's token and features exist.
+// this lane's token and features exist.  PRELOADED: an holds rope_angles of this lane (else they
+// are read here, where the lane rotates).
+template <bool PRELOADED = false>
 __device__ __forceinline__ void rope_store4(const RopeStore& rs, int tok, const TokenPlace& tp, int f0, int g,
-                                            f32x4 v, bool live) {
+                                            f32x4 v, bool live, RopeAngles an = RopeAngles{}) {
     const int hd = rs.cache.head_dim, nkv = rs.cache.n_kv_heads;
     f32x4 partner;
 #pragma unroll
@@ -58,8 +100,8 @@ __device__ __forceinline__ void rope_store4(const RopeStore& rs, int tok, const 
         const int half = rs.rot >> 1;
         const int pair0 = 8 * (within >> 4) + 4 * (g & 1);          // first of this lane's four pairs
         dim = g < 2 ? pair0 : half + pair0;
-        const float4* t = (const float4*)(rs.cs + (size_t)tok * half + pair0);
-        const float4 cs01 = t[0], cs23 = t[1];
+        if (!PRELOADED) an = rope_angles(rs, tok, f0, g);
+        const float4 cs01 = an.a, cs23 = an.b;
         const float c[4] = {cs01.x, cs01.z, cs23.x, cs23.z}, s[4] = {cs01.y, cs01.w, cs23.y, cs23.w};
 #pragma unroll
         for (int r = 0; r < 4; ++r) o[r] = g < 2 ? v[r] * c[r] - partner[r] * s[r] : v[r] * c[r] + partner[r] * s[r];

@@ -19,7 +19,10 @@ register_signatures({
     "fl_gemm_skinny_fused": [P, P, P, I, I, I, I, I, I, P, I, F, P, P, P, P, P],
     "fl_gemm_skinny_scale_parts": [I, I, I],
     "fl_gemm_skinny_rope": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
-    "fl_gemm_tiled_rope": [P, P, I, I, I, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
+    "fl_gemm_tiled_rope": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
+    "fl_gemm_tiled_scaled": [P, P, P, P, I, I, I, I, I, I, P, I, F, P],
+    "fl_gemm_tiled_residual": [P, P, I, I, I, P, P, P, P, P],
+    "fl_gemm_tiled_parts": [I, I],
     "fl_gemm_mid": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_mid_splits": [I, I, I],
     "fl_gemm_mid_scaled": [P, P, P, P, I, I, I, I, I, I, P, I, F, P],
@@ -172,20 +175,20 @@ def gemm_rope_store(x, w: Weight, store: RopeStore, rt=None) -> bool:
         gemm_skinny_rope(x, w.packed, w.rows, store, row_scale=scale)
         return True
     if M > SKINNY_MAX_ROWS and K % 8 == 0 and gemm_tiled_splits(M, w.rows, K) == 1:
-        if isinstance(x, NormedRows):
-            x = x.materialize(rt)
-        gemm_tiled_rope(x, w.packed, w.rows, store)
+        x, scale = _rows_for(x, w, rt)
+        gemm_tiled_rope(x, w.packed, w.rows, store, row_scale=scale)
         return True
     return False
 
 
-def gemm_tiled_rope(x, w_packed, n_features: int, store: RopeStore):
+def gemm_tiled_rope(x, w_packed, n_features: int, store: RopeStore, row_scale: NormedRows | None = None):
     """``gemm_skinny_rope`` for many rows (shapes whose K is not split)."""
     M, K = x.shape
     if w_packed.numel() != _packed_size(n_features, K):
         raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{n_features}, {K}] matrix packs to {_packed_size(n_features, K)}")
+    ssq, parts, eps = _row_scale_args(row_scale, M, K)
     call("fl_gemm_tiled_rope", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         M, n_features, K, *_rope_args(store, M, n_features), stream_handle())
+         M, n_features, K, ssq, parts, eps, *_rope_args(store, M, n_features), stream_handle())
     return store.q_out
 
 
@@ -241,10 +244,10 @@ def gemm_tiled_splits(M: int, N: int, K: int) -> int:
     return load().fl_gemm_tiled_splits(M, N, K)
 
 
-def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0):
+def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None):
     """``out = x @ w.T`` for many rows of x.  A shape whose grid would not fill the chip splits K
     and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values).  With
-    ``swiglu_rows`` see ``gemm_skinny``."""
+    ``swiglu_rows`` and ``row_scale`` see ``gemm_skinny``."""
     M, K = x.shape
     N = swiglu_rows or out.shape[1]
     if w_packed.numel() != _packed_size(N, K):
@@ -252,11 +255,32 @@ def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0):
     splits = 1 if swiglu_rows else gemm_tiled_splits(M, N, K)
     if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
         raise KernelError(f"gemm_tiled: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
-    call("fl_gemm_tiled", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+    ssq, parts, eps = _row_scale_args(row_scale, M, K)
+    call("fl_gemm_tiled_scaled", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
          _check(out, "gemm.out", None, (M, None)),
          _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], stream_handle())
+         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps, stream_handle())
     return out
+
+
+def tiled_parts(M: int, n_features: int) -> int:
+    """Parts in which ``gemm_tiled_residual`` leaves the sums of squares of its N features."""
+    from .library import load
+    return load().fl_gemm_tiled_parts(M, n_features)
+
+
+def gemm_tiled_residual(x, w_packed, resid, g, xg, ssq, eps: float) -> NormedRows:
+    """``gemm_skinny_residual`` for many rows (shapes whose K is not split): ``ssq[m, p]`` = sums over
+    the tiles of features."""
+    M, K = x.shape
+    N = resid.shape[1]
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    call("fl_gemm_tiled_residual", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         M, N, K, _check(resid, "gemm.resid", torch.float32, (M, N)), _check(g, "gemm.g", torch.float32, (N,)),
+         _check(xg, "gemm.xg", torch.bfloat16, (M, N)), _check(ssq, "gemm.ssq", torch.float32, (M, tiled_parts(M, N))),
+         stream_handle())
+    return NormedRows(xg, ssq, float(eps), resid, g)
 
 
 def _rows_for(x, w: Weight, rt):
@@ -272,6 +296,8 @@ def _rows_for(x, w: Weight, rt):
             return x.xg, x
     if w.packed is not None and FUSED_NORM_MAX_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0 \
             and x.ssq.shape[1] <= MID_SCALE_PARTS:
+        return x.xg, x
+    if w.packed is not None and M > SKINNY_MAX_ROWS and K % 8 == 0:
         return x.xg, x
     return x.materialize(rt), None
 
@@ -299,7 +325,7 @@ def gemm(x, w: Weight, out, rt=None):
         workspace = _split_workspace(rt, splits * M * N, x.device) if splits > 1 else None
         if mid:
             return gemm_mid(x, w.packed, out, workspace, row_scale=scale)
-        return gemm_tiled(x, w.packed, out, workspace)
+        return gemm_tiled(x, w.packed, out, workspace, row_scale=scale)
     if w.rowmajor is None:
         raise KernelError(f"gemm: no kernel for {M} rows of a packed [{w.rows}, {w.cols}] matrix")
     return ops.gemm_plain(x, w.rowmajor, out)
@@ -310,7 +336,7 @@ def gemm_swiglu(x, w: Weight, out, rt):
     x, scale = _rows_for(x, w, rt)
     M, K = x.shape
     if scale is not None and w.swiglu_cols:
-        kernel = gemm_skinny if M <= FUSED_NORM_MAX_ROWS else gemm_mid
+        kernel = gemm_skinny if M <= FUSED_NORM_MAX_ROWS else (gemm_mid if M <= SKINNY_MAX_ROWS else gemm_tiled)
         return kernel(x, w.packed, out, swiglu_rows=w.packed_rows, row_scale=scale)
     if scale is not None:
         x = scale.materialize(rt)

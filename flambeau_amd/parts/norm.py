@@ -26,7 +26,7 @@ class RMSNorm(Norm):
         return ops.rmsnorm(x, self.weight, out, self.eps, delta=delta, store_sum=store_sum, rows=rows)
 
     def after_product(self, rt, resid, product):
-        """For up to 64 rows (a decode step) the product's kernel adds its result to the stream and
+        """Where a kernel for the shape exists the product's kernel adds its result to the stream and
         leaves the norm in factors: x * w in the compute dtype and the sums of squares in parts.
         The product that follows multiplies by rsqrt(mean + eps) itself: no norm kernel runs."""
         if not rt.tuned:
@@ -47,4 +47,8 @@ class RMSNorm(Norm):
             ssq = rt.buffer("normed_ssq_mid", n, tuned.mid_parts(H), torch.float32)
             workspace = tuned._split_workspace(rt, tuned.gemm_mid_splits(n, H, K) * n * H, x.device)
             return tuned.gemm_mid_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps, workspace)
+        if n > tuned.SKINNY_MAX_ROWS and tuned.gemm_tiled_splits(n, H, K) == 1:
+            # many rows (a prompt portion): the tiled product's epilogue does it
+            ssq = rt.buffer("normed_ssq_tiled", n, tuned.tiled_parts(n, H), torch.float32)
+            return tuned.gemm_tiled_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps)
         return None

@@ -124,11 +124,13 @@ def test_gemm_skinny_against_plain(out_dtype, M, N, K):
 
 @pytest.mark.parametrize("M,H,N2,I,eps", [(1, 4096, 6144, 512, 1e-5), (8, 4096, 32768, 14336, 1e-5), (16, 72, 40, 104, 1e-2),
                                             (3, 136, 250, 40, 1e-6), (5, 64, 16, 8, 1e-5),
-                                            (64, 4096, 6144, 14336, 1e-5), (17, 96, 40, 64, 1e-3), (40, 2080, 300, 160, 1e-5)])
+                                            (64, 4096, 6144, 14336, 1e-5), (17, 96, 40, 64, 1e-3), (40, 2080, 300, 160, 1e-5),
+                                            (2048, 4096, 1024, 512, 1e-5), (300, 264, 152, 96, 1e-6), (129, 72, 40, 104, 1e-3)])
 def test_gemm_fused_with_the_norms_around_it(M, H, N2, I, eps):
+    from flambeau_amd.kernels import KernelError
     """resid += a W1^T in the product's epilogue, norm(resid) W2^T through the row scale of the next
     product, against the same chain in float64; and the SwiGLU epilogue after a row scale.  Up to 16
-    rows in the skinny kernel, 17 to 64 in the kernel that shares x through LDS."""
+    rows in the skinny kernel, 17 to 64 in the kernel that shares x through LDS, more in the tiled one."""
     from flambeau_amd.kernels.packing import pack_weight
     a = rnd(M, I, dtype=torch.bfloat16, seed=51)
     w1 = rnd(H, I, dtype=torch.bfloat16, seed=52, scale=0.05)
@@ -140,10 +142,17 @@ def test_gemm_fused_with_the_norms_around_it(M, H, N2, I, eps):
     if M <= 16:
         ssq = torch.full((M, tuned().skinny_parts(H)), float("nan"), dtype=torch.float32, device=DEV)
         rows = tuned().gemm_skinny_residual(a, pack_weight(w1), resid, g, xg, ssq, eps)
-    else:
+    elif M <= 64:
         ssq = torch.full((M, tuned().mid_parts(H)), float("nan"), dtype=torch.float32, device=DEV)
         ws = torch.full((tuned().gemm_mid_splits(M, H, I) * M * H,), float("nan"), dtype=torch.float32, device=DEV)
         rows = tuned().gemm_mid_residual(a, pack_weight(w1), resid, g, xg, ssq, eps, ws)
+    else:
+        if tuned().gemm_tiled_splits(M, H, I) > 1:
+            with pytest.raises(KernelError, match="splits K"):
+                tuned().gemm_tiled_residual(a, pack_weight(w1), resid, g, xg, torch.empty(M, tuned().tiled_parts(M, H), device=DEV), eps)
+            return
+        ssq = torch.full((M, tuned().tiled_parts(M, H)), float("nan"), dtype=torch.float32, device=DEV)
+        rows = tuned().gemm_tiled_residual(a, pack_weight(w1), resid, g, xg, ssq, eps)
     r_ref = resid0.double() + a.double() @ w1.double().T
     assert (resid.double() - r_ref).abs().max() < 1e-5 * r_ref.abs().max()
     assert (ssq.double().sum(1) - (r_ref ** 2).sum(1)).abs().max() < 1e-5 * (r_ref ** 2).sum(1).max()
