@@ -249,3 +249,33 @@ def test_captured_decode_steps_equal_eager_ones(model_dirs, dtype):
     for k in eager:
         assert np.array_equal(eager[k], graphed[k]), k
     rh.compare(graphed, reqs, rh.plain_logits(d, reqs), dtype, "captured steps")
+
+
+@pytest.fixture(scope="module")
+def wide_model_dir(tmp_path_factory):
+    """Two layers with the layer sizes of a 7B model (width 4096, 32 heads in 8 groups of 128,
+    feed-forward 14336, vocabulary 32768), written by the random-weights mode."""
+    import torch
+    from flambeau_amd.weights import write_random_model
+    config = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "hidden_act": "silu",
+              "num_hidden_layers": 2, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8,
+              "intermediate_size": 14336, "vocab_size": 32768, "rope_theta": 1e6, "sliding_window": None,
+              "rms_norm_eps": 1e-5, "max_position_embeddings": 32768, "tie_word_embeddings": False}
+    return write_random_model(config, tmp_path_factory.mktemp("wide") / "model", seed=7, std=0.02, gain_std=0.01,
+                              store_dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cutting_at_real_layer_sizes(wide_model_dir, dtype):
+    """The sizes the kernels are tuned for (and the kernels that only those sizes reach: the tiled
+    products with their fusions, many heads, pages of 16 under long rows), in portions and mixed."""
+    from flambeau_amd.engine import ModelRunner, load_model
+    reqs = rh.make_requests(32768, [150, 40, 90], seed=11)
+    model, _ = load_model(wide_model_dir, dtype=dtype, max_batch_tokens=512)
+    runner = ModelRunner(model, n_pages=24, page_size=16, max_slots=4, max_logit_rows=512)
+    ref = rh.plain_logits(wide_model_dir, reqs)
+    for what, steps in (("portions", rh.trace_portions(reqs, sizes=(2, 70, 3, 17, 2, 130, 31, 4))),
+                        ("mixed", rh.trace_mixed(reqs, seed=3, max_portion=90))):
+        got = rh.run_in_process(runner, steps)
+        assert not runner.manager.live
+        rh.compare(got, reqs, ref, dtype, f"wide {what}")
