@@ -194,13 +194,15 @@ def test_prenorm_block_part(dtype):
 # ---------------------------------------------------------------- toy parts, defined here
 def _register_toys():
     """A mixer with per-request state (a decaying sum of its inputs), a position encoding that is
-    not a rotation (it scales queries and keys by a function of the position), and an
+    not a rotation (it scales queries and keys by a function of the position), a feed-forward
+    that routes every token to one of its experts, a norm that subtracts the mean, and an
     architecture that puts them beside the built-in parts, layer by layer."""
     from dataclasses import dataclass
     from flambeau_amd.config.base import KeyReader
     from flambeau_amd.kernels import ops
     from flambeau_amd.models.decoder import LayerSpec, ModelSpec, RunEntry
-    from flambeau_amd.parts import (MIXERS, POSITION_ENCODINGS, Mixer, PartSpec, PositionEncoding, StateSpec, TensorSpec)
+    from flambeau_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward, Mixer, Norm, PartSpec,
+                                    PositionEncoding, StateSpec, TensorSpec)
     from flambeau_amd.registry import register_architecture
 
     if "toy_decay_sum" in MIXERS.known():
@@ -245,11 +247,71 @@ def _register_toys():
             f = 1.0 + self.rate * torch.cos(positions.float())
             qkv[:, :(n_heads + n_kv_heads) * head_dim] *= f[:, None]
 
+    @FEED_FORWARDS.register("toy_routed")
+    class Routed(FeedForward):
+        """Every token goes to the expert its router scores highest (logits and softmax in 32-bit);
+        delta = p_expert * Down_e silu(Up_e x).  The tokens of an expert are gathered and run
+        through the framework's matrix products."""
+        def __init__(self, hidden_size, inner_size, n_experts):
+            self.H, self.I, self.E = hidden_size, inner_size, n_experts
+
+        def tensors(self):
+            t = {"router.weight": TensorSpec((self.E, self.H))}
+            for e in range(self.E):
+                t[f"e{e}.up.weight"] = TensorSpec((self.I, self.H))
+                t[f"e{e}.down.weight"] = TensorSpec((self.H, self.I))
+            return t
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.router = weights["router.weight"].float()
+            self.up = [rt.prepare_weight(weights[f"e{e}.up.weight"]) for e in range(self.E)]
+            self.down = [rt.prepare_weight(weights[f"e{e}.down.weight"]) for e in range(self.E)]
+
+        def forward(self, x, step):
+            n = x.shape[0]
+            p = torch.softmax(x.float() @ self.router.T, dim=-1)
+            choice = p.argmax(dim=-1)
+            delta = torch.zeros(n, self.H, dtype=torch.float32, device=x.device)
+            for e in range(self.E):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                h = torch.empty(rows.numel(), self.I, dtype=torch.float32, device=x.device)
+                self.rt.gemm(x[rows].contiguous(), self.up[e], h)
+                d = torch.empty(rows.numel(), self.H, dtype=torch.float32, device=x.device)
+                self.rt.gemm((h * torch.sigmoid(h)).to(x.dtype), self.down[e], d)
+                delta[rows] = d * p[rows, e][:, None]
+            return delta
+
+    @NORMS.register("toy_centered_norm")
+    class CenteredNorm(Norm):
+        """y = (x - mean) * rsqrt(var + eps) * w."""
+        def __init__(self, hidden_size, eps):
+            self.hidden_size, self.eps = hidden_size, eps
+
+        def tensors(self):
+            return {"weight": TensorSpec((self.hidden_size,), "vector32")}
+
+        def bind(self, weights, rt):
+            self.rt, self.weight = rt, weights["weight"]
+
+        def forward(self, x, out, delta=None, store_sum=False, rows=None):
+            s = x if delta is None else x + delta
+            if store_sum and delta is not None:
+                x.copy_(s)
+            if rows is not None:
+                s = s[rows.long()]
+            c = s - s.mean(dim=-1, keepdim=True)
+            out.copy_((c * torch.rsqrt((c * c).mean(dim=-1, keepdim=True) + self.eps) * self.weight).to(out.dtype))
+            return out
+
     @dataclass(frozen=True)
     class ToyConfig:
         hidden_size: int
         vocab_size: int
         layer_kinds: tuple
+        ffn_kinds: tuple
         decay: float
         rate: float
         max_position_embeddings: int
@@ -258,12 +320,14 @@ def _register_toys():
         def from_dict(cls, raw, where="config.json"):
             r = KeyReader(raw, where)
             return cls(r.integer("hidden_size"), r.integer("vocab_size"), tuple(raw["layer_kinds"]),
-                       r.number("decay"), r.number("rate"), r.integer("max_position_embeddings"))
+                       tuple(raw["ffn_kinds"]), r.number("decay"), r.number("rate"), r.integer("max_position_embeddings"))
 
     def toy_spec(cfg):
         H = cfg.hidden_size
         norm = PartSpec("rmsnorm", dict(hidden_size=H, eps=1e-5))
-        ffn = PartSpec("swiglu", dict(hidden_size=H, intermediate_size=2 * H))
+        centered = PartSpec("toy_centered_norm", dict(hidden_size=H, eps=1e-3))
+        ffns = {"swiglu": PartSpec("swiglu", dict(hidden_size=H, intermediate_size=2 * H)),
+                "routed": PartSpec("toy_routed", dict(hidden_size=H, inner_size=24, n_experts=3))}
         mixers = {
             "decay": PartSpec("toy_decay_sum", dict(hidden_size=H, decay=cfg.decay)),
             "attn": PartSpec("paged_gqa_attention", dict(hidden_size=H, n_heads=2, n_kv_heads=1, head_dim=16,
@@ -271,11 +335,19 @@ def _register_toys():
         }
         layers = []
         for l, kind in enumerate(cfg.layer_kinds):
-            block = PartSpec("prenorm", dict(mixer=mixers[kind], feed_forward=ffn, norm=norm))
+            routed = cfg.ffn_kinds[l] == "routed"
+            # a routed layer norms with the centered norm, the others with the built-in one
+            block = PartSpec("prenorm", dict(mixer=mixers[kind], feed_forward=ffns[cfg.ffn_kinds[l]],
+                                             norm=centered if routed else norm))
             local = ["w"] if kind == "decay" else ["q", "k", "v", "o"]
             names = {f"mixer.{t}.weight": f"toy.{l}.mix.{t}" for t in local}
-            names.update({"mixer_norm.weight": f"toy.{l}.n1", "ffn_norm.weight": f"toy.{l}.n2",
-                          "ffn.gate.weight": f"toy.{l}.gate", "ffn.up.weight": f"toy.{l}.up", "ffn.down.weight": f"toy.{l}.down"})
+            names.update({"mixer_norm.weight": f"toy.{l}.n1", "ffn_norm.weight": f"toy.{l}.n2"})
+            if routed:
+                names["ffn.router.weight"] = f"toy.{l}.router"
+                for e in range(3):
+                    names.update({f"ffn.e{e}.up.weight": f"toy.{l}.e{e}.up", f"ffn.e{e}.down.weight": f"toy.{l}.e{e}.down"})
+            else:
+                names.update({"ffn.gate.weight": f"toy.{l}.gate", "ffn.up.weight": f"toy.{l}.up", "ffn.down.weight": f"toy.{l}.down"})
             layers.append(LayerSpec(block, names))
         # the order layers run in is data: layer 1 runs twice, its second run reads the first's cache
         order = [RunEntry(l) for l in range(len(layers))]
@@ -295,8 +367,14 @@ def _toy_plain(cfg, w, toks):
     if cfg["layer_kinds"][1] == "attn":
         order.append(1)
     kept = {}            # keys and values a layer's first run stored
+
+    def centered(v, g):
+        c = v - v.mean(axis=-1, keepdims=True)
+        return c / np.sqrt((c * c).mean(axis=-1, keepdims=True) + 1e-3) * g
+
     for l in order:
-        a = pm.rmsnorm(x, w[f"toy.{l}.n1"], 1e-5)
+        routed = cfg["ffn_kinds"][l] == "routed"
+        a = centered(x, w[f"toy.{l}.n1"]) if routed else pm.rmsnorm(x, w[f"toy.{l}.n1"], 1e-5)
         if cfg["layer_kinds"][l] == "decay":
             s, sums = np.zeros(H), []
             for t in range(n):
@@ -314,8 +392,20 @@ def _toy_plain(cfg, w, toks):
                 kept[l] = (k, v)
             d = pm.attention(q, k, v, np.arange(n), 0.25, 0).reshape(n, 32) @ w[f"toy.{l}.mix.o"].T
         x = x + d
-        b = pm.rmsnorm(x, w[f"toy.{l}.n2"], 1e-5)
-        x = x + pm.swiglu_mlp(b, w[f"toy.{l}.gate"], w[f"toy.{l}.up"], w[f"toy.{l}.down"])
+        if routed:
+            b = centered(x, w[f"toy.{l}.n2"])
+            logits = b @ w[f"toy.{l}.router"].T
+            p = np.exp(logits - logits.max(axis=-1, keepdims=True))
+            p = p / p.sum(axis=-1, keepdims=True)
+            d = np.zeros_like(x)
+            for t in range(n):
+                e = int(np.argmax(p[t]))
+                h = w[f"toy.{l}.e{e}.up"] @ b[t]
+                d[t] = p[t, e] * (w[f"toy.{l}.e{e}.down"] @ pm.silu(h))
+            x = x + d
+        else:
+            b = pm.rmsnorm(x, w[f"toy.{l}.n2"], 1e-5)
+            x = x + pm.swiglu_mlp(b, w[f"toy.{l}.gate"], w[f"toy.{l}.up"], w[f"toy.{l}.down"])
     return pm.rmsnorm(x, w["toy.norm"], 1e-5) @ w["toy.head"].T
 
 
@@ -325,10 +415,12 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
     from flambeau_amd.weights import write_random_model
     _register_toys()
     cfg = dict(architectures=["ToyStateLM"], hidden_size=32, vocab_size=90, layer_kinds=["decay", "attn", "decay"],
-               decay=0.8, rate=0.3, max_position_embeddings=128)
+               ffn_kinds=["routed", "swiglu", "routed"], decay=0.8, rate=0.3, max_position_embeddings=128)
     d = write_random_model(cfg, tmp_path / "toy", seed=4, std=0.15, gain_std=0.05, store_dtype=torch.float32)
     model, _ = load_model(d, dtype="float32", max_batch_tokens=128)
     assert [type(b.mixer).__name__ for b in model.blocks] == ["DecaySum", "PagedGQAAttention", "DecaySum"]
+    assert [type(b.ffn).__name__ for b in model.blocks] == ["Routed", "SwiGLU", "Routed"]
+    assert [type(b.ffn_norm).__name__ for b in model.blocks] == ["CenteredNorm", "RMSNorm", "CenteredNorm"]
     runner = ModelRunner(model, n_pages=16, page_size=8, max_slots=3, max_logit_rows=128)
     assert not runner.decode_graphs                                    # a mixer with state of its own never replays
     assert len(runner.storage.states) == 2 and len(runner.storage.pools) == 1
