@@ -36,11 +36,11 @@
 __device__ __forceinline__ int pf_key_of_row(int i, int ab) { return 8 * (i >> 2) + 4 * ab + (i & 3); }
 
 template <int HDP, int QT, int NS>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+__global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, PagedCache cache,
     const int* __restrict__ tiles, const int* __restrict__ positions,
     const int* __restrict__ block_table, int max_blocks, int nh, float scale_log2e, int window,
-    int log2_ps) {
+    int log2_ps, int mirror_from) {
     constexpr int QS = HDP / 32;              // k-steps of the score product
     constexpr int DT = HDP / 16;              // tiles of head dims in the output
     constexpr int KT = 4 * QS;                // 1 KB tiles of a K stage: [chunk (2)][a/b (2)][k-step]
@@ -49,14 +49,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     extern __shared__ __attribute__((aligned(16))) bf16_t ring[];       // [NS][KT + VT][512], then the pages
     int* s_pages = (int*)(ring + (size_t)NS * (KT + VT) * 512);         // [max_blocks]
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);          // the same for the whole wave: branches on it are scalar
     const int j = lane & 15, g = lane >> 4;
     const int hd = cache.head_dim, ps = cache.page_size;
     const int G = nh / cache.n_kv_heads;
     const int hgroups = G / QT;
     const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
-    // tiles late in a prompt have the most keys: they are started first
-    const int tile = gridDim.x - 1 - blockIdx.x;
+    // Tiles late in a prompt have the most keys: they are started first.  When the whole grid is on
+    // the chip at once (two blocks per compute unit, the second half of the grid beside the first),
+    // the second half runs the other way round, so that a long tile shares its unit with a short one.
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    const int tile = lin < mirror_from ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
     const int seq = tiles[3 * tile], row0 = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
     const int* table = block_table + (size_t)seq * max_blocks;
     const bf16_t* kv = (const bf16_t*)cache.base;
@@ -106,13 +110,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 
     // ---- what this wave loads per stage: tiles tl = wave + 4 u of [K tiles | V tiles]; per lane the
     // key offset inside the stage and the offset inside the (page, head) block are fixed
+    // (KT is a multiple of 4, so load u of every wave is a K tile for u < QS and a V tile from there on)
     int key_off[LPW], blk_off[LPW];
-    const size_t head_k = (size_t)kvh * ps * hd, head_v = ((size_t)cache.n_kv_heads + kvh) * ps * hd;
-    const size_t page_stride = (size_t)2 * cache.n_kv_heads * ps * hd;
+    const int head_k = kvh * ps * hd, head_v = (cache.n_kv_heads + kvh) * ps * hd;      // inside a page: below 2^31
+    const unsigned page_stride = 2u * cache.n_kv_heads * ps * hd;
 #pragma unroll
     for (int u = 0; u < LPW; ++u) {
         const int tl = wave + 4 * u;
-        if (tl < KT) {                                         // K tile: chunk, a/b, k-step
+        if (u < QS) {                                          // K tile: chunk, a/b, k-step
             // the four lanes of a quad copy 64 consecutive bytes of one key row (a quad spread over
             // four rows costs four cache lookups); the pieces of a row are exchanged by (row / 2) % 4
             // so that the operand reads meet no bank twice (see gemm_tiled.hip)
@@ -120,14 +125,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             key_off[u] = 32 * c2 + pf_key_of_row(lane >> 2, ab);
             int d = 32 * s + 8 * ((lane & 3) ^ ((lane >> 3) & 3));
             if (d + 8 > hd) d = 0;                             // padding dims: any finite data (Q is zero there)
-            blk_off[u] = d;                                    // + row * hd, row known per stage
+            blk_off[u] = head_k + d;                           // + row * hd, row known per stage
         } else {                                               // V tile: chunk, dim tile
             const int tv = tl - KT;
             const int c2 = tv / DT, dt = tv % DT;
             key_off[u] = 32 * c2 + 8 * g;
             int d = 16 * dt + j;
             if (d >= hd) d = 0;                                // padding dims are never stored
-            blk_off[u] = d * ps;                               // + row
+            blk_off[u] = head_v + d * ps;                      // + row
         }
     }
     // operand lane (key row j, k-piece g) finds its 16 bytes of a K tile here
@@ -143,12 +148,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             // keys outside [lo, p_last] are masked: read any valid one instead.  A value piece is a run
             // of 8 keys and keeps its place if any of its keys is needed (its page is alive then)
             int t = t0 + key_off[u];
-            if (tl < KT) t = min(max(t, lo), p_last);
+            if (u < QS) t = min(max(t, lo), p_last);
             else if (t + 7 < lo || t > p_last) t = p_last & ~7;
-            const int page = s_pages[(t >> log2_ps) - page0];
+            const unsigned page = (unsigned)s_pages[(t >> log2_ps) - page0];
             const int row = t & (ps - 1);
-            const bf16_t* src = kv + (size_t)page * page_stride +
-                                (tl < KT ? head_k + (size_t)row * hd + blk_off[u] : head_v + blk_off[u] + row);
+            // 32-bit arithmetic inside the page (24-bit factors: one full-rate multiply), one 32 x 32 -> 64
+            // multiply for the page
+            const int in_page = blk_off[u] + (u < QS ? __mul24(row, hd) : row);
+            const bf16_t* src = kv + (uint64_t)page * page_stride + in_page;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                              (__attribute__((address_space(3))) void*)(slot + tl * 512), 16, 0, 0);
         }
@@ -284,6 +291,17 @@ template <int HDP, int QT, int NS>
 static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                                const int* tiles, const int* positions, const int* block_table, int max_blocks,
                                int nh, float scale_log2e, int window, int log2_ps) {
+    // blocks that the chip holds at one time: one or two per compute unit
+    static int units = 0;
+    if (!units) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || units <= 0)
+            units = 256;
+    }
+    const int total = (int)(grid.x * grid.y);
+    const int resident = units * (QT * HDP <= 256 ? 2 : 1);
+    // (whole rows of the grid: every tile of a head group is taken exactly once either way)
+    const int mirror_from = (QT * HDP <= 256 && total <= resident && total > units) ? (int)((grid.y / 2) * grid.x) : total;
     constexpr int RING = NS * (4 * (HDP / 32) + 2 * (HDP / 16)) * 1024;
     static bool configured = false;
     auto kern = attn_prefill_kernel<HDP, QT, NS>;
@@ -292,7 +310,7 @@ static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, b
                                   RING + PF_MAX_PAGES * (int)sizeof(int));
         configured = true;
     }
-    kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
+    kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from);
 }
 
 static int g_pf_stages = 0;              // ring stages: 0 = two (two blocks fit a compute unit), 3 for experiments
@@ -318,6 +336,7 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "attn_prefill: head size %d must be a multiple of 8 up to 256", hd);
     FL_CHECK(page_size >= 8 && (page_size & (page_size - 1)) == 0,
              "attn_prefill: page size %d must be a power of two, at least 8", page_size);
+    FL_CHECK((long long)2 * nkv * page_size * hd < (1ll << 31), "attn_prefill: a page of %d heads x %d keys x %d is too large (2^31 values)", nkv, page_size, hd);
     FL_CHECK(max_blocks <= PF_MAX_PAGES, "attn_prefill: %d pages per request, at most %d", max_blocks, PF_MAX_PAGES);
     FL_CHECK(window >= 0, "attn_prefill: negative window");
     FL_CHECK(scale > 0.f, "attn_prefill: the score scale must be positive");
@@ -327,9 +346,11 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     const int hdp = ceil_div(hd, 32) * 32;
     int log2_ps = 0;
     while ((1 << log2_ps) < page_size) ++log2_ps;
-    // query heads per wave: a divisor of the group size, as many as the registers hold
+    // query heads per wave: a divisor of the group size; as many as leave room for two blocks per
+    // compute unit (two waves per SIMD hide each other's waits: measured 906 against 1314 us at 8192
+    // tokens with 2 heads instead of 4 at head size 128)
     int qt = (G % 4 == 0) ? 4 : (G % 2 == 0 ? 2 : 1);
-    const int qt_max = hdp <= 128 ? 4 : 2;
+    const int qt_max = hdp <= 64 ? 4 : 2;
     while (qt > qt_max) qt /= 2;
     if (qt_hint == 1 || qt_hint == 2 || qt_hint == 4)
         while (qt > qt_hint) qt /= 2;
