@@ -35,6 +35,8 @@
 // 16-byte run of a row of the transposed values: the value operand needs no gathering.
 __device__ __forceinline__ int pf_key_of_row(int i, int ab) { return 8 * (i >> 2) + 4 * ab + (i & 3); }
 
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+
 template <int HDP, int QT, int NS>
 __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, PagedCache cache,
@@ -98,12 +100,15 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
         }
     }
     f32x4 o[QT][DT];
-    float m[QT], l[QT], thr[QT];              // base of the exponents, sum, and the score that moves the base
+    f32x4 l[QT];                              // sums of the exponentials: every row of the tile holds the column's sum
+    float m[QT], thr[QT];                     // base of the exponents and the score that moves the base
+    const bf16_t one = (bf16_t)1.0f;
+    const bf16x8 ones8 = {one, one, one, one, one, one, one, one};
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
         m[t] = -INFINITY;
         thr[t] = -INFINITY;
-        l[t] = 0.f;
+        l[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int d = 0; d < DT; ++d) o[t][d] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
@@ -142,9 +147,12 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     auto issue = [&](int i) {
         const int t0 = t_base + i * PF_STAGE;
         bf16_t* slot = ring + (size_t)(i % NS) * (KT + VT) * 512;
+        // first every load's page is looked up (the compiler keeps an LDS read behind a copy into
+        // LDS that precedes it: looked up one by one, each would wait for its own read), then the
+        // copies are started
+        const bf16_t* src[LPW];
 #pragma unroll
         for (int u = 0; u < LPW; ++u) {
-            const int tl = wave + 4 * u;
             // keys outside [lo, p_last] are masked: read any valid one instead.  A value piece is a run
             // of 8 keys and keeps its place if any of its keys is needed (its page is alive then)
             int t = t0 + key_off[u];
@@ -155,10 +163,12 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
             // 32-bit arithmetic inside the page (24-bit factors: one full-rate multiply), one 32 x 32 -> 64
             // multiply for the page
             const int in_page = blk_off[u] + (u < QS ? __mul24(row, hd) : row);
-            const bf16_t* src = kv + (uint64_t)page * page_stride + in_page;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)(slot + tl * 512), 16, 0, 0);
+            src[u] = kv + (uint64_t)page * page_stride + in_page;
         }
+#pragma unroll
+        for (int u = 0; u < LPW; ++u)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src[u],
+                                             (__attribute__((address_space(3))) void*)(slot + (wave + 4 * u) * 512), 16, 0, 0);
     };
     __syncthreads();                                            // s_pages is complete
 #pragma unroll
@@ -174,25 +184,43 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
         asm volatile("s_barrier" ::: "memory");
         if (i + NS - 1 < n_stage) issue(i + NS - 1);
         const bf16_t* slot = ring + (size_t)(i % NS) * (KT + VT) * 512;
+        // The scores of both halves of the stage go to the matrix cores first: the softmax of the
+        // first half (vector unit) then runs while the second half's products are still in flight,
+        // and the second softmax beside the first half's value products.
+        bool act[2];
+        f32x4 sa[2][QT], sb[2][QT];
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             const int t0 = t_base + i * PF_STAGE + 32 * half;
             // wave-uniform: does any query of this wave see any key of this chunk?
-            if (!wave_on || t0 > wp_last || t0 + 31 < w_lo) continue;
-            const bool need_mask = (t0 + 31 > wp_first) || (t0 < (window > 0 ? max(0, wp_last - window + 1) : 0));
-            // ---- scores
-            f32x4 sa[QT], sb[QT];
+            act[half] = wave_on && t0 <= wp_last && t0 + 31 >= w_lo;
+            if (!act[half]) continue;
 #pragma unroll
-            for (int t = 0; t < QT; ++t) { sa[t] = (f32x4){0.f, 0.f, 0.f, 0.f}; sb[t] = sa[t]; }
+            for (int t = 0; t < QT; ++t) { sa[half][t] = (f32x4){0.f, 0.f, 0.f, 0.f}; sb[half][t] = sa[half][t]; }
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
                 const bf16x8 ka = *(const bf16x8*)(slot + ((2 * half) * QS + s) * 512 + k_read);
                 const bf16x8 kb = *(const bf16x8*)(slot + ((2 * half + 1) * QS + s) * 512 + k_read);
 #pragma unroll
                 for (int t = 0; t < QT; ++t) {
-                    sa[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[t][s], sa[t], 0, 0, 0);
-                    sb[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[t][s], sb[t], 0, 0, 0);
+                    sa[half][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[t][s], sa[half][t], 0, 0, 0);
+                    sb[half][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[t][s], sb[half][t], 0, 0, 0);
                 }
+            }
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            if (!act[half]) continue;
+            const int t0 = t_base + i * PF_STAGE + 32 * half;
+            const bool need_mask = (t0 + 31 > wp_first) || (t0 < (window > 0 ? max(0, wp_last - window + 1) : 0));
+            // the value tiles of this half are asked for now and arrive during the softmax (where
+            // the registers allow it)
+            constexpr bool EARLY_V = QT * HDP <= 256;
+            bf16x8 vt[EARLY_V ? DT : 1];
+            if (EARLY_V) {
+#pragma unroll
+                for (int d = 0; d < DT; ++d) vt[EARLY_V ? d : 0] = *(const bf16x8*)(slot + (KT + half * DT + d) * 512 + lane * 8);
+                __builtin_amdgcn_sched_barrier(0);
             }
             // ---- softmax per query column; this lane holds keys t0 + 8 g + r (a) and + 4 + r (b).
             // m holds the raw (unscaled) score that the exponents are taken against.  It follows the
@@ -208,16 +236,16 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int ka = t0 + 8 * g + r, kb = ka + 4;
-                        sa[t][r] = (ka > p || ka < my_lo) ? -INFINITY : sa[t][r];
-                        sb[t][r] = (kb > p || kb < my_lo) ? -INFINITY : sb[t][r];
+                        sa[half][t][r] = (ka > p || ka < my_lo) ? -INFINITY : sa[half][t][r];
+                        sb[half][t][r] = (kb > p || kb < my_lo) ? -INFINITY : sb[half][t][r];
                     }
             }
             float mx[QT];
             bool above = false;
 #pragma unroll
             for (int t = 0; t < QT; ++t) {
-                mx[t] = fmaxf(fmaxf(fmaxf(sa[t][0], sa[t][1]), fmaxf(sa[t][2], sa[t][3])),
-                              fmaxf(fmaxf(sb[t][0], sb[t][1]), fmaxf(sb[t][2], sb[t][3])));
+                const f32x4 a = sa[half][t], b = sb[half][t];
+                mx[t] = max3(max3(a[0], a[1], a[2]), max3(a[3], b[0], b[1]), fmaxf(b[2], b[3]));
                 above = above || mx[t] > thr[t];
             }
             if (__any(above)) {
@@ -243,24 +271,22 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
                 // column that has seen no key yet keeps m = -inf: its base is 0 then (its scores
                 // are all -inf, their exponentials 0)
                 const float base = m[t] == -INFINITY ? 0.f : m[t] * scale_log2e;
-                float ls = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float ea = __builtin_amdgcn_exp2f(fmaf(sa[t][r], scale_log2e, -base));
-                    const float eb = __builtin_amdgcn_exp2f(fmaf(sb[t][r], scale_log2e, -base));
-                    ls += ea + eb;
-                    pmat[t][r] = (bf16_t)ea;
-                    pmat[t][4 + r] = (bf16_t)eb;
+                    pmat[t][r] = (bf16_t)__builtin_amdgcn_exp2f(fmaf(sa[half][t][r], scale_log2e, -base));
+                    pmat[t][4 + r] = (bf16_t)__builtin_amdgcn_exp2f(fmaf(sb[half][t][r], scale_log2e, -base));
                 }
-                l[t] += ls;
+                // the column's sum of exponentials (of the rounded ones, which are what the values
+                // are weighted with) comes from the matrix cores too: a value tile of ones
+                l[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones8, pmat[t], l[t], 0, 0, 0);
             }
             // ---- O^T += V^T P^T
 #pragma unroll
             for (int d = 0; d < DT; ++d) {
-                const bf16x8 vt = *(const bf16x8*)(slot + (KT + half * DT + d) * 512 + lane * 8);
+                const bf16x8 vd = EARLY_V ? vt[EARLY_V ? d : 0] : *(const bf16x8*)(slot + (KT + half * DT + d) * 512 + lane * 8);
 #pragma unroll
                 for (int t = 0; t < QT; ++t)
-                    o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pmat[t], o[t][d], 0, 0, 0);
+                    o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vd, pmat[t], o[t][d], 0, 0, 0);
             }
         }
     }
@@ -269,9 +295,7 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     if (!q_ok) return;
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
-        float ll = l[t];
-        ll += __shfl_xor(ll, 16, 64);
-        ll += __shfl_xor(ll, 32, 64);
+        const float ll = l[t][0];
         const float inv = ll > 0.f ? 1.0f / ll : 0.f;
         const int head = kvh * G + hg * QT + t;
         bf16_t* orow = out + ((size_t)(row0 + qtok) * nh + head) * hd;
