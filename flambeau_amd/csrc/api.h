@@ -25,7 +25,7 @@ int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int* positions
                      const int* tok_seq, const int* block_table, int max_blocks, void* q_out,
                      void* cache_base, int dtype, int n, int nh, int nkv, int hd, int page_size,
                      int n_pages, int rot, float theta, int write_cache, const float* cs, int paired,
-                     hipStream_t stream);
+                     int n_parts, long part_stride, hipStream_t stream);
 // cs[n][rot / 2][2]: cosine and sine of every (token, rotation pair) of a step
 int fl_rope_table(const int* positions, int n, int rot, float theta, float* cs, hipStream_t stream);
 int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
@@ -67,6 +67,8 @@ int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out, float* wo
                        float eps, hipStream_t stream);
 int fl_gemm_mid_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
                          float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream);
+int fl_gemm_mid_partials(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                         const float* in_ssq, int in_parts, float eps, hipStream_t stream);
 int fl_gemm_mid_parts(int N);
 
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,

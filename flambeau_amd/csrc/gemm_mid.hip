@@ -383,6 +383,23 @@ extern "C" int fl_gemm_mid(const void* x, const void* w_packed, void* out, float
     return fl_gemm_mid_scaled(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, stream);
 }
 
+// The K-splits of x w^T left apart: workspace[s][M][N] for s < fl_gemm_mid_splits(M, N, K) (one "split"
+// if K is not split), for a kernel that adds them itself (fl_rope_kv_write).  in_ssq as in
+// fl_gemm_mid_scaled: every part is scaled, so their sum is.
+extern "C" int fl_gemm_mid_partials(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                                    const float* in_ssq, int in_parts, float eps, hipStream_t stream) {
+    if (mid_checks(x, w_packed, M, N, K)) return -1;
+    FL_CHECK(workspace && (uintptr_t)workspace % 16 == 0, "gemm_mid_partials: needs a 16-byte aligned workspace");
+    FL_CHECK(!in_ssq || (in_parts > 0 && in_parts <= GM_SCALE_PARTS), "gemm_mid: a row scale over %d parts (at most %d)",
+             in_parts, GM_SCALE_PARTS);
+    if (M == 0) return 0;
+    const MidScale sc = {in_ssq, in_parts, eps};
+    launch_mid_mt<float, false>(ceil_div(M, 16), (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
+                                fl_gemm_mid_splits(M, N, K), N, sc, stream);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+
 // resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_mid_parts(N)] =
 // sums of resid^2 over 4096 columns each: the factors of the norm that follows.  The workspace holds
 // fl_gemm_mid_splits(M, N, K) * M * N floats (also when K is not split).

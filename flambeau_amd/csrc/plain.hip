@@ -285,12 +285,18 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const TIn* __restrict__ qkv, int ld, const int* __restrict__ positions,
     const int* __restrict__ tok_seq, const int* __restrict__ block_table, int max_blocks,
     T* __restrict__ q_out, PagedCache cache, int nh, int hd, int rot, float theta, int write_cache,
-    const float2* __restrict__ cs, int paired) {
+    const float2* __restrict__ cs, int paired, int n_parts, size_t part_stride) {
     const int token = blockIdx.x;
     const int head = blockIdx.y;
     const int nkv = cache.n_kv_heads;
     const int pos = positions[token];
     const TIn* src = qkv + (size_t)token * ld + (size_t)head * hd;
+    // the projection may arrive as n_parts partial sums (a product that split K): added here, in rising order
+    auto value = [&](int i) {
+        float v = to_f32(src[i]);
+        for (int part = 1; part < n_parts; ++part) v += to_f32(src[(size_t)part * part_stride + i]);
+        return v;
+    };
     T* dst;
     size_t stride = 1;      // distance between consecutive head dims at the destination
     bool rotate;
@@ -326,13 +332,13 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
                 c = cosf(angle); s = sinf(angle);
             }
             const int at = paired ? 16 * (i >> 3) + (i & 7) : i;
-            const float x0 = to_f32(src[at]), x1 = to_f32(src[paired ? at + 8 : i + half]);
+            const float x0 = value(at), x1 = value(paired ? at + 8 : i + half);
             dst[i] = from_f32<T>(x0 * c - x1 * s);
             dst[i + half] = from_f32<T>(x0 * s + x1 * c);
         }
-        for (int i = rot + threadIdx.x; i < hd; i += 64) dst[i] = from_f32<T>(to_f32(src[i]));
+        for (int i = rot + threadIdx.x; i < hd; i += 64) dst[i] = from_f32<T>(value(i));
     } else {
-        for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * stride] = from_f32<T>(to_f32(src[i]));
+        for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * stride] = from_f32<T>(value(i));
     }
 }
 
@@ -340,8 +346,10 @@ extern "C" int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int
                                 const int* tok_seq, const int* block_table, int max_blocks,
                                 void* q_out, void* cache_base, int dtype, int n, int nh, int nkv,
                                 int hd, int page_size, int n_pages, int rot, float theta,
-                                int write_cache, const float* cs, int paired, hipStream_t stream) {
+                                int write_cache, const float* cs, int paired, int n_parts, long part_stride,
+                                hipStream_t stream) {
     FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && hd > 0 && page_size > 0, "rope_kv_write: bad sizes");
+    FL_CHECK(n_parts >= 1 && (n_parts == 1 || part_stride >= (long)n * ld), "rope_kv_write: %d parts %ld values apart", n_parts, part_stride);
     FL_CHECK(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotated dims %d of head %d", rot, hd);
     FL_CHECK(ld >= (nh + 2 * nkv) * hd, "rope_kv_write: row stride %d too small", ld);
     FL_CHECK(!paired || (rot % 16 == 0 && hd % 16 == 0), "rope_kv_write: the paired order needs rotated dims and head size in steps of 16 (%d of %d)", rot, hd);
@@ -351,7 +359,7 @@ extern "C" int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int
 #define FL_ROPE(TIN, TT)                                                                       \
     rope_kv_write_kernel<TIN, TT><<<grid, 64, 0, stream>>>((const TIN*)qkv, ld, positions, tok_seq, \
                                                            block_table, max_blocks, (TT*)q_out, c, \
-                                                           nh, hd, rot, theta, write_cache, (const float2*)cs, paired)
+                                                           nh, hd, rot, theta, write_cache, (const float2*)cs, paired, n_parts, (size_t)part_stride)
     if (in_dtype == FL_F32 && dtype == FL_F32) FL_ROPE(float, float);
     else if (in_dtype == FL_F32 && dtype == FL_BF16) FL_ROPE(float, bf16_t);
     else if (in_dtype == FL_BF16 && dtype == FL_BF16) FL_ROPE(bf16_t, bf16_t);

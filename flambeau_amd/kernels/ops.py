@@ -110,11 +110,19 @@ def rope_table(positions, rotated_dims, theta, out):
 
 
 def rope_kv_write(qkv, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads,
-                  rotated_dims, theta, write_cache=True, table=None, paired=False):
+                  rotated_dims, theta, write_cache=True, table=None, paired=False, parts: int = 1):
     """Rotate q and k, store q and the cache rows.  ``table``: the step's ``rope_table`` (else the
     angles are computed here); ``paired``: the projection's rows come in the order of
-    ``rotary_paired_rows``."""
-    n, ld = qkv.shape
+    ``rotary_paired_rows``.  With ``parts`` > 1 ``qkv`` is ``[parts, n, ld]``: partial sums of a
+    product that split K, added here."""
+    if parts > 1 or qkv.dim() == 3:
+        if qkv.dim() != 3 or qkv.shape[0] != parts or not qkv.is_contiguous():
+            raise KernelError(f"rope_kv_write: {parts} parts want a contiguous [{parts}, n, ld] tensor")
+        part_stride = qkv.shape[1] * qkv.shape[2]
+        n, ld = qkv.shape[1:]
+    else:
+        part_stride = 0
+        n, ld = qkv.shape
     nkv, hd = cache.n_kv_heads, cache.head_dim
     if ld != (n_heads + 2 * nkv) * hd:
         raise KernelError(f"rope_kv_write: row of {ld} values, expected {(n_heads + 2 * nkv) * hd}")
@@ -126,7 +134,7 @@ def rope_kv_write(qkv, positions, tok_seq, block_table, q_out, cache: PagedLayer
          _check(cache.pool, "rope.cache"), dtype_code(cache.pool.dtype), n, n_heads, nkv, hd,
          cache.page_size, cache.n_pages, int(rotated_dims), float(theta), int(bool(write_cache)),
          _check(table, "rope.table", torch.float32, (n, rotated_dims // 2, 2)) if table is not None and rotated_dims else None,
-         int(bool(paired)), stream_handle())
+         int(bool(paired)), int(parts), int(part_stride), stream_handle())
     return q_out
 
 

@@ -28,6 +28,7 @@ register_signatures({
     "fl_gemm_mid_scaled": [P, P, P, P, I, I, I, I, I, I, P, I, F, P],
     "fl_gemm_mid_residual": [P, P, P, I, I, I, P, P, P, P, P],
     "fl_gemm_mid_parts": [I],
+    "fl_gemm_mid_partials": [P, P, P, I, I, I, P, I, F, P],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
@@ -178,6 +179,15 @@ def gemm_rope_store(x, w: Weight, store: RopeStore, rt=None) -> bool:
         x, scale = _rows_for(x, w, rt)
         gemm_tiled_rope(x, w.packed, w.rows, store, row_scale=scale)
         return True
+    if FUSED_NORM_MAX_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0:
+        # 17 to 64 rows: the product leaves its K-splits apart and the rotation kernel adds them
+        x, scale = _rows_for(x, w, rt)
+        N = w.rows
+        splits = gemm_mid_splits(M, N, K)
+        parts = gemm_mid_partials(x, w.packed, _split_workspace(rt, splits * M * N, x.device), N, row_scale=scale)
+        ops.rope_kv_write(parts, store.positions, store.tok_seq, store.block_table, store.q_out, store.cache, store.n_heads,
+                          store.rotated_dims, 0.0, write_cache=store.write_cache, table=store.angles, paired=True, parts=splits)
+        return True
     return False
 
 
@@ -215,6 +225,22 @@ def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: 
          _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
          dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps, stream_handle())
     return out
+
+
+def gemm_mid_partials(x, w_packed, workspace, n_features: int, row_scale: NormedRows | None = None):
+    """The K-splits of ``x @ w.T`` (17 to 64 rows) left apart: returns ``[splits, M, N]`` float32 (a
+    view of ``workspace``) for a kernel that adds them itself."""
+    M, K = x.shape
+    N = n_features
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    splits = gemm_mid_splits(M, N, K)
+    if workspace is None or workspace.numel() < splits * M * N:
+        raise KernelError(f"gemm_mid_partials: needs a workspace of {splits * M * N} floats")
+    ssq, parts, eps = _row_scale_args(row_scale, M, K)
+    call("fl_gemm_mid_partials", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(workspace, "gemm.workspace", torch.float32), M, N, K, ssq, parts, eps, stream_handle())
+    return workspace[:splits * M * N].view(splits, M, N)
 
 
 def mid_parts(n_features: int) -> int:

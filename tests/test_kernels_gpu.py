@@ -529,10 +529,13 @@ def test_gemm_mid_refuses_what_it_cannot_do():
 
 @pytest.mark.parametrize("M,nh,nkv,hd,rot,ps,H", [(1, 32, 8, 128, 128, 16, 4096), (8, 4, 2, 16, 16, 8, 64), (16, 5, 5, 32, 16, 16, 80),
                                                   (300, 6, 2, 64, 64, 16, 96), (2048, 32, 8, 128, 128, 16, 512),
-                                                  (130, 3, 1, 48, 32, 32, 72), (70, 8, 8, 16, 16, 8, 40)])
+                                                  (130, 3, 1, 48, 32, 32, 72), (70, 8, 8, 16, 16, 8, 40),
+                                                  (64, 32, 8, 128, 128, 16, 4096), (17, 6, 2, 64, 32, 16, 96), (40, 5, 5, 32, 16, 8, 2048),
+                                                  (33, 4, 2, 16, 16, 8, 40)])
 def test_gemm_with_rotation_and_stores_in_its_kernel(M, nh, nkv, hd, rot, ps, H):
     """The joined q/k/v projection with rows in paired order, rotated and stored by the product's own
-    kernel (few rows: skinny; many rows: tiled), against product + rotation kernel apart and float64."""
+    kernel (few rows: skinny; many rows: tiled) or, for 17 to 64 rows, by a rotation kernel that adds
+    the product's K-splits itself; against product + rotation kernel apart and float64."""
     from flambeau_amd.kernels.packing import rotary_paired_rows
     theta = 1e4
     N = (nh + 2 * nkv) * hd
@@ -570,7 +573,7 @@ def test_gemm_with_rotation_and_stores_in_its_kernel(M, nh, nkv, hd, rot, ps, H)
     cache_b = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
     q_b = torch.full((M, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     store = tuned().RopeStore(pos_d, seq_d, table, angles, q_b, cache_b, nh, rot, True)
-    if 16 < M <= 64 or (M > 64 and tuned().gemm_tiled_splits(M, N, H) > 1):
+    if (16 < M <= 64 and H % 32) or (M > 64 and tuned().gemm_tiled_splits(M, N, H) > 1):
         assert not tuned().gemm_rope_store(x, W, store)
         return
     assert tuned().gemm_rope_store(x, W, store)
