@@ -471,6 +471,46 @@ def test_gemm_tiled_against_plain(out_dtype, M, N, K):
     assert (got.double() - ref).abs().max() < tol * scale
 
 
+@pytest.mark.parametrize("variant", [3, 6])
+@pytest.mark.parametrize("M,N,K", [(300, 520, 72), (129, 264, 96), (1100, 640, 256)])
+def test_gemm_tiled_block_shapes(variant, M, N, K):
+    """Both block shapes of the tiled product (256 x 128 and 128 x 256), whichever the sizes would
+    choose, through the plain epilogue, the row scale and the add-to-the-stream epilogue."""
+    from flambeau_amd.kernels.library import load
+    from flambeau_amd.kernels.packing import pack_weight
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=23), rnd(N, K, dtype=torch.bfloat16, seed=24, scale=0.05)
+    g = 1 + rnd(N, seed=25, scale=0.1)
+    resid0 = rnd(M, N, seed=26)
+    load().fl_gemm_tiled_set_variant(variant)
+    try:
+        splits = tuned().gemm_tiled_splits(M, N, K)
+        ws = torch.empty(splits * M * N, dtype=torch.float32, device=DEV) if splits > 1 else None
+        got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+        tuned().gemm_tiled(x, pack_weight(w), got, ws)
+        ref = x.double() @ w.double().T
+        assert (got.double() - ref).abs().max() < 1e-5 * ref.abs().max()
+        if splits == 1:
+            resid = resid0.clone()
+            xg = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ssq = torch.full((M, tuned().tiled_parts(M, N)), float("nan"), dtype=torch.float32, device=DEV)
+            rows = tuned().gemm_tiled_residual(x, pack_weight(w), resid, g, xg, ssq, 1e-5)
+            want = resid0.double() + ref
+            assert (resid.double() - want).abs().max() < 1e-5 * want.abs().max()
+            assert (xg.double() - want * g.double()).abs().max() < 5e-3 * (want * g.double()).abs().max()
+            assert (ssq.double().sum(dim=1) - (want * want).sum(dim=1)).abs().max() < 1e-4 * (want * want).sum(dim=1).max()
+            # the rows in factors feed a product that scales by the norm itself
+            w2 = rnd(200, N, dtype=torch.bfloat16, seed=27, scale=0.05)
+            out2 = torch.full((M, 200), float("nan"), dtype=torch.float32, device=DEV)
+            sp2 = tuned().gemm_tiled_splits(M, 200, N)
+            ws2 = torch.empty(sp2 * M * 200, dtype=torch.float32, device=DEV) if sp2 > 1 else None
+            tuned().gemm_tiled(rows.xg, pack_weight(w2), out2, ws2, row_scale=rows)
+            normed = want * g.double() * torch.rsqrt((want * want).mean(dim=1, keepdim=True) + 1e-5)
+            ref2 = normed @ w2.double().T
+            assert (out2.double() - ref2).abs().max() < 1e-2 * ref2.abs().max()
+    finally:
+        load().fl_gemm_tiled_set_variant(0)
+
+
 def test_gemm_tiled_splits_k_for_small_grids():
     assert tuned().gemm_tiled_splits(2048, 4096, 4096) == 1
     assert tuned().gemm_tiled_splits(128, 4096, 4096) > 1
