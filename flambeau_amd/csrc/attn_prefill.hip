@@ -144,26 +144,50 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     const int k_read = 32 * j + 8 * (g ^ ((j >> 1) & 3));
     const int n_stage = (p_last / PF_STAGE) - (lo / PF_STAGE) + 1;
     const int t_base = (lo / PF_STAGE) * PF_STAGE;
+    // A stage whose 64 keys all lie in [lo, p_last] needs no clamping, and then little arithmetic:
+    // the keys of a load sit in one of the stage's two chunks of 32, at a row of its page that is
+    // the same in every stage (pages divide 64 or are multiples of it), and the page a lane needs
+    // within a chunk depends on lane / 16 only (keys 8 (lane / 16) .. + 7 of the chunk, for K and V
+    // tiles alike).  So two look-ups and two multiplications per stage serve all loads.
+    int in_page_c[LPW];
+    bool second_chunk[LPW];
+#pragma unroll
+    for (int u = 0; u < LPW; ++u) {
+        const int r = key_off[u] & (ps - 1);
+        in_page_c[u] = blk_off[u] + (u < QS ? __mul24(r, hd) : r);
+        second_chunk[u] = (u < QS ? (wave + 4 * u) / (2 * QS) : (wave + 4 * u - KT) / DT) != 0;      // the same for the wave
+    }
+    const int lane_pg = (8 * g) >> log2_ps;
     auto issue = [&](int i) {
         const int t0 = t_base + i * PF_STAGE;
         bf16_t* slot = ring + (size_t)(i % NS) * (KT + VT) * 512;
-        // first every load's page is looked up (the compiler keeps an LDS read behind a copy into
-        // LDS that precedes it: looked up one by one, each would wait for its own read), then the
-        // copies are started
         const bf16_t* src[LPW];
+        if (t0 >= lo && t0 + PF_STAGE - 1 <= p_last) {
+            const bf16_t* base0 = kv + (uint64_t)(unsigned)s_pages[(t0 >> log2_ps) - page0 + lane_pg] * page_stride;
+            const bf16_t* base1 = kv + (uint64_t)(unsigned)s_pages[((t0 + 32) >> log2_ps) - page0 + lane_pg] * page_stride;
+            const int row_shift = t0 & (ps - 1);              // pages longer than a stage: where the stage begins in its page
+            const int shift_k = row_shift * hd;
 #pragma unroll
-        for (int u = 0; u < LPW; ++u) {
-            // keys outside [lo, p_last] are masked: read any valid one instead.  A value piece is a run
-            // of 8 keys and keeps its place if any of its keys is needed (its page is alive then)
-            int t = t0 + key_off[u];
-            if (u < QS) t = min(max(t, lo), p_last);
-            else if (t + 7 < lo || t > p_last) t = p_last & ~7;
-            const unsigned page = (unsigned)s_pages[(t >> log2_ps) - page0];
-            const int row = t & (ps - 1);
-            // 32-bit arithmetic inside the page (24-bit factors: one full-rate multiply), one 32 x 32 -> 64
-            // multiply for the page
-            const int in_page = blk_off[u] + (u < QS ? __mul24(row, hd) : row);
-            src[u] = kv + (uint64_t)page * page_stride + in_page;
+            for (int u = 0; u < LPW; ++u)
+                src[u] = (second_chunk[u] ? base1 : base0) + (in_page_c[u] + (u < QS ? shift_k : row_shift));
+        } else {
+            // first every load's page is looked up (the compiler keeps an LDS read behind a copy into
+            // LDS that precedes it: looked up one by one, each would wait for its own read), then the
+            // copies are started
+#pragma unroll
+            for (int u = 0; u < LPW; ++u) {
+                // keys outside [lo, p_last] are masked: read any valid one instead.  A value piece is a run
+                // of 8 keys and keeps its place if any of its keys is needed (its page is alive then)
+                int t = t0 + key_off[u];
+                if (u < QS) t = min(max(t, lo), p_last);
+                else if (t + 7 < lo || t > p_last) t = p_last & ~7;
+                const unsigned page = (unsigned)s_pages[(t >> log2_ps) - page0];
+                const int row = t & (ps - 1);
+                // 32-bit arithmetic inside the page (24-bit factors: one full-rate multiply), one 32 x 32 -> 64
+                // multiply for the page
+                const int in_page = blk_off[u] + (u < QS ? __mul24(row, hd) : row);
+                src[u] = kv + (uint64_t)page * page_stride + in_page;
+            }
         }
 #pragma unroll
         for (int u = 0; u < LPW; ++u)
@@ -197,14 +221,19 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
             if (!act[half]) continue;
 #pragma unroll
             for (int t = 0; t < QT; ++t) { sa[half][t] = (f32x4){0.f, 0.f, 0.f, 0.f}; sb[half][t] = sa[half][t]; }
+            // all key tiles of the half are asked for at once: the later ones arrive behind the first products
+            bf16x8 ka[QS], kb[QS];
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
-                const bf16x8 ka = *(const bf16x8*)(slot + ((2 * half) * QS + s) * 512 + k_read);
-                const bf16x8 kb = *(const bf16x8*)(slot + ((2 * half + 1) * QS + s) * 512 + k_read);
+                ka[s] = *(const bf16x8*)(slot + ((2 * half) * QS + s) * 512 + k_read);
+                kb[s] = *(const bf16x8*)(slot + ((2 * half + 1) * QS + s) * 512 + k_read);
+            }
+#pragma unroll
+            for (int s = 0; s < QS; ++s) {
 #pragma unroll
                 for (int t = 0; t < QT; ++t) {
-                    sa[half][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[t][s], sa[half][t], 0, 0, 0);
-                    sb[half][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[t][s], sb[half][t], 0, 0, 0);
+                    sa[half][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[s], qreg[t][s], sa[half][t], 0, 0, 0);
+                    sb[half][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[s], qreg[t][s], sb[half][t], 0, 0, 0);
                 }
             }
         }
@@ -215,7 +244,7 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
             const bool need_mask = (t0 + 31 > wp_first) || (t0 < (window > 0 ? max(0, wp_last - window + 1) : 0));
             // the value tiles of this half are asked for now and arrive during the softmax (where
             // the registers allow it)
-            constexpr bool EARLY_V = QT * HDP <= 256;
+            constexpr bool EARLY_V = QT * HDP <= 256 && QT <= 2;
             bf16x8 vt[EARLY_V ? DT : 1];
             if (EARLY_V) {
 #pragma unroll
@@ -349,9 +378,13 @@ template <int HDP, int NS>
 static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                            const int* tiles, const int* positions, const int* block_table, int max_blocks, int nh,
                            float scale_log2e, int window, int log2_ps) {
-    if (qt == 4)
-        launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
-    else if (qt == 2)
+    if constexpr (HDP <= 64) {            // four heads per wave only where two blocks still fit a compute unit
+        if (qt == 4) {
+            launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
+            return;
+        }
+    }
+    if (qt >= 2)
         launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
     else
         launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
