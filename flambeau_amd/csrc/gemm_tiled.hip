@@ -10,16 +10,22 @@
 //  * LDS is a ring of NS stages of one k-step (32 values of k); one bare s_barrier per stage;
 //  * the w tile is the A operand and the x tile the B operand: C[feature][token] leaves each
 //    lane with four consecutive features of one token, one 16-byte store;
-//  * two shapes: 256 features x 128 tokens per block (a wave computes 8 x 4 tiles: 12 operand
-//    reads feed 32 products) when that grid fills the chip, else 128 x 128 (4 x 4 tiles, deeper
-//    ring);
+//  * two shapes: 256 features x 128 tokens per block (four waves, a wave computes 8 x 4 tiles: 12
+//    operand reads feed 32 products; ring of 3; two blocks per compute unit) when that grid fills
+//    the chip, else 128 x 256 (eight waves of 4 x 4 tiles, ring of 4, one block per unit); blocks
+//    are handed to the eight dies in turn, each die working on a compact patch of tiles;
 //  * with few rows and a narrow matrix even that grid is small: K is then split over
 //    blockIdx.z, the parts are written as float partial sums and a second kernel adds them in
 //    a fixed order;
-//  * optional SwiGLU epilogue over gate/up rows interleaved in fours.
+//  * epilogues: plain; SwiGLU over gate/up rows interleaved in fours; rotate and store q and the
+//    cache rows (rope_store.h); add to the residual stream and leave the next norm in factors.
+//    Every one can scale a token's results by the factor of a norm left that way (TiledFusion).
 //
-// Measured on the 7B shapes at 2,048 rows: 0.73 to 0.88 PFLOP/s.  What bounds it is the delivery
-// of operand tiles into LDS (the same kernel without loads runs at 1.2 to 1.6 PFLOP/s).
+// Measured on the 7B shapes: 0.78 to 1.09 PFLOP/s at 2,048 rows, 1.1 to 1.2 at 4,096.  What bounds
+// it is the delivery of operand tiles into LDS: for 28672 x 4096 x 4096 the matrix cores alone take
+// 555 us, with the operand reads 583, with the barrier 637, the whole kernel 871, and the stream
+// of copies alone 700 (about 14 TB/s out of the L2s, whatever the tile shape, ring depth, order of
+// issue or row stride).
 //
 // The reference's nearest kernel multiplies a 64 x 8 tile per 64-thread block without matrix
 // cores (crates/kernels-hip/src/kernels/mmq_f16_tile.cu:33-107).
