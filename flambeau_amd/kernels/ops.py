@@ -66,6 +66,11 @@ def embed(table, tokens, out):
     return out
 
 
+def gather_rows(src, rows, out):
+    """``out[r] = src[rows[r]]`` for a float32 ``src`` (the embedding kernel over a table of rows)."""
+    return embed(src, rows, out)
+
+
 def rmsnorm(x, weight, out, eps, delta=None, store_sum=False, rows=None):
     """``out = rmsnorm(x (+ delta)) * weight``; ``store_sum`` writes x + delta back into x;
     ``rows`` (int32) picks the rows of x that are normed, one output row each."""

@@ -14,6 +14,7 @@ from dataclasses import dataclass, field
 
 import torch
 
+from ..kernels import ops
 from ..parts import BLOCKS, NORMS, OutputHead, PartSpec, ResidualStream, TokenEmbedding
 
 
@@ -130,6 +131,9 @@ class DecoderModel:
             # same kernels whatever is wanted), and the wanted ones are picked afterwards
             x = stream.normed(self.final_norm, name="final", lazy=True)
             logits = self.head.forward(x, max(max_logit_rows, step.n_tokens))
-            return logits if every_row else torch.index_select(logits, 0, step.logit_rows)
+            if every_row:
+                return logits
+            picked = rt.buffer("logits_picked", step.logit_rows.shape[0], logits.shape[1], torch.float32, max_rows=max_logit_rows)
+            return ops.gather_rows(logits, step.logit_rows, picked)
         x = stream.normed(self.final_norm, rows=step.logit_rows, name="final")
         return self.head.forward(x, max_logit_rows)
