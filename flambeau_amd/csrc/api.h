@@ -70,6 +70,9 @@ int fl_gemm_mid_residual(const void* x, const void* w_packed, float* workspace, 
 int fl_gemm_mid_partials(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
                          const float* in_ssq, int in_parts, float eps, hipStream_t stream);
 int fl_gemm_mid_parts(int N);
+// The adding half of fl_gemm_mid_residual for any number of rows: part[splits][M][N] -> resid, xg, out_ssq.
+int fl_reduce_residual(const float* part, float* resid, const float* g, void* xg, float* out_ssq, int M, int N,
+                       int splits, hipStream_t stream);
 
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
@@ -86,14 +89,15 @@ int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K,
                        const int* block_table, int max_blocks, const float* cs, void* q_out, void* cache_base,
                        int nh, int nkv, int hd, int page_size, int n_pages, int rot, int write_cache,
                        hipStream_t stream);
-// The tiled product fused with the norms around it, as fl_gemm_skinny_fused (shapes whose K is not split for
-// the residual form; out_ssq[M, fl_gemm_tiled_parts(M, N)]).
+// The tiled product fused with the norms around it, as fl_gemm_skinny_fused.  The residual form leaves
+// out_ssq[M, fl_gemm_tiled_residual_parts(M, N, K)] and needs a workspace of splits * M * N floats where K is split.
 int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                          int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
                          float eps, hipStream_t stream);
-int fl_gemm_tiled_residual(const void* x, const void* w_packed, int M, int N, int K, float* resid,
+int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K, float* resid,
                            const float* g, void* xg, float* out_ssq, hipStream_t stream);
 int fl_gemm_tiled_parts(int M, int N);
+int fl_gemm_tiled_residual_parts(int M, int N, int K);
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                    const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
                    int n_pages, float scale, int window, int n_split, hipStream_t stream);

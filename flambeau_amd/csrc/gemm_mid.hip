@@ -422,3 +422,19 @@ extern "C" int fl_gemm_mid_residual(const void* x, const void* w_packed, float* 
 }
 
 extern "C" int fl_gemm_mid_parts(int N) { return ceil_div(N, GM_RED_COLS); }
+
+// The second half of fl_gemm_mid_residual on its own, for any number of rows: part[splits][M][N] are
+// partial sums of a product; resid += their sum, xg = bf16(resid * g), out_ssq[M, fl_gemm_mid_parts(N)].
+extern "C" int fl_reduce_residual(const float* part, float* resid, const float* g, void* xg, float* out_ssq, int M,
+                                  int N, int splits, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && splits >= 1, "reduce_residual: bad sizes M=%d N=%d splits=%d", M, N, splits);
+    FL_CHECK(part && resid && g && xg && out_ssq, "reduce_residual: needs part, resid, g, xg and out_ssq");
+    FL_CHECK(((uintptr_t)part % 16 == 0) && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)g % 16 == 0) &&
+             ((uintptr_t)xg % 8 == 0), "reduce_residual: part, resid and g must be 16-byte aligned, xg 8-byte");
+    FL_CHECK(M <= 65535, "reduce_residual: %d rows, at most 65535", M);
+    if (M == 0) return 0;
+    dim3 grid(ceil_div(N, GM_RED_COLS), M);
+    gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(part, resid, g, (bf16_t*)xg, out_ssq, M, N, splits);
+    FL_LAUNCH_CHECK();
+    return 0;
+}

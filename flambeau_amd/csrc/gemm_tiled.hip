@@ -488,25 +488,39 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
     return fl_gemm_tiled_scaled(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, stream);
 }
 
-// resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_tiled_parts(M, N)] =
-// the sums of resid^2 over the feature tiles: the factors of the norm that follows.  Only for shapes
-// whose K is not split.
-extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, int M, int N, int K, float* resid,
-                                      const float* g, void* xg, float* out_ssq, hipStream_t stream) {
+// resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_tiled_residual_parts(M, N, K)]
+// = the sums of resid^2 in parts: the factors of the norm that follows.  Where K is not split the
+// product's epilogue does it (one part per tile of features); where it is, the partial sums go to
+// the workspace (fl_gemm_tiled_splits(M, N, K) * M * N floats) and the kernel that adds them does it
+// (one part per 4096 features, fl_reduce_residual).
+extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                                      float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_residual: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled_residual: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(N % 4 == 0, "gemm_tiled_residual: N=%d is no multiple of 4 (16-byte accesses to the residual rows)", N);
     FL_CHECK(resid && g && xg && out_ssq, "gemm_tiled_residual: needs resid, g, xg and out_ssq");
-    FL_CHECK(fl_gemm_tiled_splits(M, N, K) == 1, "gemm_tiled_residual: this shape splits K");
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)resid % 16 == 0) &&
              ((uintptr_t)g % 16 == 0) && ((uintptr_t)xg % 8 == 0), "gemm_tiled_residual: operands must be aligned (16 bytes, xg 8)");
     if (M == 0) return 0;
     const int n_steps = ceil_div(K, 32);
+    const int splits = fl_gemm_tiled_splits(M, N, K);
+    if (splits > 1) {
+        FL_CHECK(workspace && (uintptr_t)workspace % 16 == 0, "gemm_tiled_residual: this shape splits K %d ways and needs a workspace", splits);
+        launch_tiled<float, TG_PLAIN>(g_tiled_variant, splits, stream, (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
+                                      n_steps, ceil_div(n_steps, splits), N, RopeStore{});
+        FL_LAUNCH_CHECK();
+        return fl_reduce_residual(workspace, resid, g, xg, out_ssq, M, N, splits, stream);
+    }
     const TiledFusion fu = {nullptr, 0, 0.f, resid, g, (bf16_t*)xg, out_ssq};
     launch_tiled<float, TG_RESIDUAL>(g_tiled_variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, resid, M, N, K,
                                      n_steps, n_steps, N, RopeStore{}, fu);
     FL_LAUNCH_CHECK();
     return 0;
+}
+
+// Parts in which fl_gemm_tiled_residual leaves a token's sum of squares.
+extern "C" int fl_gemm_tiled_residual_parts(int M, int N, int K) {
+    return fl_gemm_tiled_splits(M, N, K) > 1 ? fl_gemm_mid_parts(N) : fl_gemm_tiled_parts(M, N);
 }
 
 // The joined q/k/v projection of many rows with its rows in paired order: q is rotated and written to

@@ -21,8 +21,9 @@ register_signatures({
     "fl_gemm_skinny_rope": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
     "fl_gemm_tiled_rope": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
     "fl_gemm_tiled_scaled": [P, P, P, P, I, I, I, I, I, I, P, I, F, P],
-    "fl_gemm_tiled_residual": [P, P, I, I, I, P, P, P, P, P],
+    "fl_gemm_tiled_residual": [P, P, P, I, I, I, P, P, P, P, P],
     "fl_gemm_tiled_parts": [I, I],
+    "fl_gemm_tiled_residual_parts": [I, I, I],
     "fl_gemm_mid": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_mid_splits": [I, I, I],
     "fl_gemm_mid_scaled": [P, P, P, P, I, I, I, I, I, I, P, I, F, P],
@@ -289,22 +290,27 @@ def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale
     return out
 
 
-def tiled_parts(M: int, n_features: int) -> int:
+def tiled_parts(M: int, n_features: int, K: int) -> int:
     """Parts in which ``gemm_tiled_residual`` leaves the sums of squares of its N features."""
     from .library import load
-    return load().fl_gemm_tiled_parts(M, n_features)
+    return load().fl_gemm_tiled_residual_parts(M, n_features, K)
 
 
-def gemm_tiled_residual(x, w_packed, resid, g, xg, ssq, eps: float) -> NormedRows:
-    """``gemm_skinny_residual`` for many rows (shapes whose K is not split): ``ssq[m, p]`` = sums over
-    the tiles of features."""
+def gemm_tiled_residual(x, w_packed, resid, g, xg, ssq, eps: float, workspace=None) -> NormedRows:
+    """``gemm_skinny_residual`` for many rows: ``ssq[m, p]`` = sums over the tiles of features where K
+    is not split, else over 4096 features each (the kernel that adds the K-splits does it then and
+    needs ``workspace``: float32, ``gemm_tiled_splits(M, N, K) * M * N`` values)."""
     M, K = x.shape
     N = resid.shape[1]
     if w_packed.numel() != _packed_size(N, K):
         raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    splits = gemm_tiled_splits(M, N, K)
+    if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
+        raise KernelError(f"gemm_tiled_residual: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
     call("fl_gemm_tiled_residual", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
          M, N, K, _check(resid, "gemm.resid", torch.float32, (M, N)), _check(g, "gemm.g", torch.float32, (N,)),
-         _check(xg, "gemm.xg", torch.bfloat16, (M, N)), _check(ssq, "gemm.ssq", torch.float32, (M, tiled_parts(M, N))),
+         _check(xg, "gemm.xg", torch.bfloat16, (M, N)), _check(ssq, "gemm.ssq", torch.float32, (M, tiled_parts(M, N, K))),
          stream_handle())
     return NormedRows(xg, ssq, float(eps), resid, g)
 

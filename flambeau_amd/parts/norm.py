@@ -47,8 +47,10 @@ class RMSNorm(Norm):
             ssq = rt.buffer("normed_ssq_mid", n, tuned.mid_parts(H), torch.float32)
             workspace = tuned._split_workspace(rt, tuned.gemm_mid_splits(n, H, K) * n * H, x.device)
             return tuned.gemm_mid_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps, workspace)
-        if n > tuned.SKINNY_MAX_ROWS and tuned.gemm_tiled_splits(n, H, K) == 1:
-            # many rows (a prompt portion): the tiled product's epilogue does it
-            ssq = rt.buffer("normed_ssq_tiled", n, tuned.tiled_parts(n, H), torch.float32)
-            return tuned.gemm_tiled_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps)
+        if n > tuned.SKINNY_MAX_ROWS and H % 4 == 0:
+            # many rows (a prompt portion): the tiled product's epilogue does it, or the kernel that adds its K-splits
+            ssq = rt.buffer("normed_ssq_tiled", n, tuned.tiled_parts(n, H, K), torch.float32)
+            splits = tuned.gemm_tiled_splits(n, H, K)
+            workspace = tuned._split_workspace(rt, splits * n * H, x.device) if splits > 1 else None
+            return tuned.gemm_tiled_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps, workspace)
         return None

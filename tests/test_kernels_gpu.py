@@ -125,7 +125,8 @@ def test_gemm_skinny_against_plain(out_dtype, M, N, K):
 @pytest.mark.parametrize("M,H,N2,I,eps", [(1, 4096, 6144, 512, 1e-5), (8, 4096, 32768, 14336, 1e-5), (16, 72, 40, 104, 1e-2),
                                             (3, 136, 250, 40, 1e-6), (5, 64, 16, 8, 1e-5),
                                             (64, 4096, 6144, 14336, 1e-5), (17, 96, 40, 64, 1e-3), (40, 2080, 300, 160, 1e-5),
-                                            (2048, 4096, 1024, 512, 1e-5), (300, 264, 152, 96, 1e-6), (129, 72, 40, 104, 1e-3)])
+                                            (2048, 4096, 1024, 512, 1e-5), (300, 264, 152, 96, 1e-6), (129, 72, 40, 104, 1e-3),
+                                            (128, 4096, 6144, 4096, 1e-5), (100, 520, 64, 2048, 1e-5), (512, 5120, 256, 1024, 1e-5)])
 def test_gemm_fused_with_the_norms_around_it(M, H, N2, I, eps):
     from flambeau_amd.kernels import KernelError
     """resid += a W1^T in the product's epilogue, norm(resid) W2^T through the row scale of the next
@@ -147,12 +148,13 @@ def test_gemm_fused_with_the_norms_around_it(M, H, N2, I, eps):
         ws = torch.full((tuned().gemm_mid_splits(M, H, I) * M * H,), float("nan"), dtype=torch.float32, device=DEV)
         rows = tuned().gemm_mid_residual(a, pack_weight(w1), resid, g, xg, ssq, eps, ws)
     else:
-        if tuned().gemm_tiled_splits(M, H, I) > 1:
-            with pytest.raises(KernelError, match="splits K"):
-                tuned().gemm_tiled_residual(a, pack_weight(w1), resid, g, xg, torch.empty(M, tuned().tiled_parts(M, H), device=DEV), eps)
-            return
-        ssq = torch.full((M, tuned().tiled_parts(M, H)), float("nan"), dtype=torch.float32, device=DEV)
-        rows = tuned().gemm_tiled_residual(a, pack_weight(w1), resid, g, xg, ssq, eps)
+        splits = tuned().gemm_tiled_splits(M, H, I)
+        ws = torch.full((splits * M * H,), float("nan"), dtype=torch.float32, device=DEV) if splits > 1 else None
+        if splits > 1:
+            with pytest.raises(KernelError, match="workspace"):
+                tuned().gemm_tiled_residual(a, pack_weight(w1), resid, g, xg, torch.empty(M, tuned().tiled_parts(M, H, I), device=DEV), eps)
+        ssq = torch.full((M, tuned().tiled_parts(M, H, I)), float("nan"), dtype=torch.float32, device=DEV)
+        rows = tuned().gemm_tiled_residual(a, pack_weight(w1), resid, g, xg, ssq, eps, ws)
     r_ref = resid0.double() + a.double() @ w1.double().T
     assert (resid.double() - r_ref).abs().max() < 1e-5 * r_ref.abs().max()
     assert (ssq.double().sum(1) - (r_ref ** 2).sum(1)).abs().max() < 1e-5 * (r_ref ** 2).sum(1).max()
@@ -492,7 +494,7 @@ def test_gemm_tiled_block_shapes(variant, M, N, K):
         if splits == 1:
             resid = resid0.clone()
             xg = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
-            ssq = torch.full((M, tuned().tiled_parts(M, N)), float("nan"), dtype=torch.float32, device=DEV)
+            ssq = torch.full((M, tuned().tiled_parts(M, N, K)), float("nan"), dtype=torch.float32, device=DEV)
             rows = tuned().gemm_tiled_residual(x, pack_weight(w), resid, g, xg, ssq, 1e-5)
             want = resid0.double() + ref
             assert (resid.double() - want).abs().max() < 1e-5 * want.abs().max()
