@@ -102,9 +102,11 @@ int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, cons
                    const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
                    int n_pages, float scale, int window, int n_split, hipStream_t stream);
 int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int* tiles, int n_tiles,
-                    const int* positions, const int* block_table, int max_blocks, int nh, int nkv,
-                    int hd, int page_size, int n_pages, float scale, int window, int qt_hint,
-                    hipStream_t stream);
+                    const int* positions, const int* block_table, int max_blocks, int nh, int nkv, int hd,
+                    int page_size, int n_pages, float scale, int window, int qt_hint, float* part_o, float* part_ml,
+                    int n_split, hipStream_t stream);
+int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int max_keys);
+int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 
 #ifdef __cplusplus

@@ -25,6 +25,7 @@
 // attention_decode_f16_splitk.cu:31-256 (partials and merge).
 #include "common.h"
 #include "api.h"
+#include "attn_merge.h"
 
 #define DEC_WAVES 4
 #define DEC_CHUNK 32
@@ -259,56 +260,16 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
     }
 }
 
-// Merge of the splits: one block per (item, head).  The splits' (max, sum) pairs are read by one
-// thread each; then every thread owns head dims and adds the splits' partial outputs, loads issued
-// eight at a time.  The order of the sum is fixed (rising split).
+// Merge of the splits: one block per (item, head) (attn_merge.h).
 __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __restrict__ part_o,
                                                                 const float* __restrict__ part_ml,
                                                                 bf16_t* __restrict__ out,
                                                                 const int4* __restrict__ items, int nh,
                                                                 int hd, int hdp, int n_split) {
-    __shared__ float s_f[256];       // exp(m_s - m_max) per split (n_split <= 256)
-    __shared__ float s_inv;
     const int item = blockIdx.x, head = blockIdx.y;
     const int token = items[item].x;
-    const size_t base = ((size_t)item * nh + head) * n_split;
-    const int t = threadIdx.x;
-    float ms = -INFINITY, ls = 0.f;
-    if (t < n_split) {
-        ms = part_ml[(base + t) * 2];
-        ls = part_ml[(base + t) * 2 + 1];
-    }
-    s_f[t] = ms;
-    __syncthreads();
-    float mm = -INFINITY;
-    for (int s = 0; s < n_split; ++s) mm = fmaxf(mm, s_f[s]);
-    __syncthreads();
-    const float f = ms == -INFINITY ? 0.f : expf(ms - mm);
-    s_f[t] = f;
-    // sum of l_s f_s in rising s, by thread 0 after everyone has written its factor
-    __shared__ float s_l[256];
-    s_l[t] = ls * f;
-    __syncthreads();
-    if (t == 0) {
-        float ll = 0.f;
-        for (int s = 0; s < n_split; ++s) ll += s_l[s];
-        s_inv = ll > 0.f ? 1.0f / ll : 0.f;
-    }
-    __syncthreads();
-    const float inv = s_inv;
-    for (int d = t; d < hd; d += blockDim.x) {
-        float acc = 0.f;
-        int s = 0;
-        for (; s + 8 <= n_split; s += 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = part_o[(base + s + u) * hdp + d];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) acc += v[u] * s_f[s + u];
-        }
-        for (; s < n_split; ++s) acc += part_o[(base + s) * hdp + d] * s_f[s];
-        out[((size_t)token * nh + head) * hd + d] = (bf16_t)(acc * inv);
-    }
+    attn_merge_splits(part_o, part_ml, out + ((size_t)token * nh + head) * hd, ((size_t)item * nh + head) * n_split, hd, hdp,
+                      n_split);
 }
 
 extern "C" int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats,

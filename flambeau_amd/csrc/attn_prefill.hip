@@ -24,6 +24,7 @@
 // prefill, 4 query rows per tile), attention_prefill_f16_paged.cu:50-150 (paged addressing).
 #include "common.h"
 #include "api.h"
+#include "attn_merge.h"
 
 #define PF_TOKENS 64          // query tokens per block
 #define PF_STAGE 64           // keys per LDS stage
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, PagedCache cache,
     const int* __restrict__ tiles, const int* __restrict__ positions,
     const int* __restrict__ block_table, int max_blocks, int nh, float scale_log2e, int window,
-    int log2_ps, int mirror_from) {
+    int log2_ps, int mirror_from, float* __restrict__ part_o, float* __restrict__ part_ml) {
     constexpr int QS = HDP / 32;              // k-steps of the score product
     constexpr int DT = HDP / 16;              // tiles of head dims in the output
     constexpr int KT = 4 * QS;                // 1 KB tiles of a K stage: [chunk (2)][a/b (2)][k-step]
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     // the second half runs the other way round, so that a long tile shares its unit with a short one.
     const int lin = blockIdx.y * gridDim.x + blockIdx.x;
     const int tile = lin < mirror_from ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
-    const int seq = tiles[3 * tile], row0 = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
+    const int seq = tiles[4 * tile], row0 = tiles[4 * tile + 1], cnt = tiles[4 * tile + 2], item0 = tiles[4 * tile + 3];
     const int* table = block_table + (size_t)seq * max_blocks;
     const bf16_t* kv = (const bf16_t*)cache.base;
 
@@ -142,8 +143,14 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     }
     // operand lane (key row j, k-piece g) finds its 16 bytes of a K tile here
     const int k_read = 32 * j + 8 * (g ^ ((j >> 1) & 3));
-    const int n_stage = (p_last / PF_STAGE) - (lo / PF_STAGE) + 1;
-    const int t_base = (lo / PF_STAGE) * PF_STAGE;
+    // the keys are walked in stages of 64; with gridDim.z > 1 this block takes one part of the stages
+    // and leaves its result unnormalised for the merge (a short portion behind a long context gives
+    // few tiles, and splitting the keys is what fills the chip then)
+    const int all_stages = (p_last / PF_STAGE) - (lo / PF_STAGE) + 1;
+    const int per_split = (all_stages + gridDim.z - 1) / gridDim.z;
+    const int first_stage = min(all_stages, (int)blockIdx.z * per_split);
+    const int n_stage = min(all_stages, first_stage + per_split) - first_stage;
+    const int t_base = (lo / PF_STAGE) * PF_STAGE + first_stage * PF_STAGE;
     // A stage whose 64 keys all lie in [lo, p_last] needs no clamping, and then little arithmetic:
     // the keys of a load sit in one of the stage's two chunks of 32, at a row of its page that is
     // the same in every stage (pages divide 64 or are multiples of it), and the page a lane needs
@@ -320,8 +327,25 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
         }
     }
 
-    // ---- normalise and store: lane (query j, g) holds dims 16 d + 4 g + r
     if (!q_ok) return;
+    if (gridDim.z > 1) {
+        // ---- one part of the keys: the unnormalised output, the base of its exponents (in natural-log
+        // units, as the merge wants it) and its sum go to the workspace
+#pragma unroll
+        for (int t = 0; t < QT; ++t) {
+            const int head = kvh * G + hg * QT + t;
+            const size_t at = ((size_t)(item0 + qtok) * nh + head) * gridDim.z + blockIdx.z;
+            float* prow = part_o + at * HDP;
+#pragma unroll
+            for (int d = 0; d < DT; ++d) *(f32x4*)(prow + 16 * d + 4 * g) = o[t][d];
+            if (g == 0) {
+                part_ml[at * 2] = m[t] * scale_log2e * 0.6931471805599453f;
+                part_ml[at * 2 + 1] = l[t][0];
+            }
+        }
+        return;
+    }
+    // ---- normalise and store: lane (query j, g) holds dims 16 d + 4 g + r
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
         const float ll = l[t][0];
@@ -353,13 +377,13 @@ static int pf_units() {                  // compute units of the device
 template <int HDP, int QT, int NS>
 static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                                const int* tiles, const int* positions, const int* block_table, int max_blocks,
-                               int nh, float scale_log2e, int window, int log2_ps) {
+                               int nh, float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml) {
     // blocks that the chip holds at one time: one or two per compute unit
     const int units = pf_units();
-    const int total = (int)(grid.x * grid.y);
+    const int total = (int)(grid.x * grid.y * grid.z);
     const int resident = units * (QT * HDP <= 256 ? 2 : 1);
     // (whole rows of the grid: every tile of a head group is taken exactly once either way)
-    const int mirror_from = (QT * HDP <= 256 && total <= resident && total > units) ? (int)((grid.y / 2) * grid.x) : total;
+    const int mirror_from = (QT * HDP <= 256 && grid.z == 1 && total <= resident && total > units) ? (int)((grid.y / 2) * grid.x) : (int)(grid.x * grid.y);
     constexpr int RING = NS * (4 * (HDP / 32) + 2 * (HDP / 16)) * 1024;
     static bool configured = false;
     auto kern = attn_prefill_kernel<HDP, QT, NS>;
@@ -368,7 +392,7 @@ static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, b
                                   RING + PF_MAX_PAGES * (int)sizeof(int));
         configured = true;
     }
-    kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from);
+    kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from, part_o, part_ml);
 }
 
 static int g_pf_stages = 0;              // ring stages: 0 = two (two blocks fit a compute unit), 3 for experiments
@@ -377,23 +401,74 @@ extern "C" int fl_attn_prefill_set_stages(int n) { g_pf_stages = n; return 0; }
 template <int HDP, int NS>
 static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                            const int* tiles, const int* positions, const int* block_table, int max_blocks, int nh,
-                           float scale_log2e, int window, int log2_ps) {
+                           float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml) {
     if constexpr (HDP <= 64) {            // four heads per wave only where two blocks still fit a compute unit
         if (qt == 4) {
-            launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
+            launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml);
             return;
         }
     }
     if (qt >= 2)
-        launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
+        launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml);
     else
-        launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps);
+        launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml);
 }
 
+// query heads per wave: a divisor of the group size; as many as leave room for two blocks per
+// compute unit (two waves per SIMD hide each other's waits: measured 906 against 1314 us at 8192
+// tokens with 2 heads instead of 4 at head size 128), and few enough that the grid has more blocks
+// than the chip has units (a short portion: measured 176 against 217 us for 512 tokens behind 7,680
+// with 1 head instead of 2)
+static int pf_heads_per_wave(int n_tiles, int nh, int nkv, int hd, int qt_hint) {
+    const int G = nh / nkv;
+    const int hdp = ceil_div(hd, 32) * 32;
+    int qt = (G % 4 == 0) ? 4 : (G % 2 == 0 ? 2 : 1);
+    const int qt_max = hdp <= 64 ? 4 : 2;
+    while (qt > qt_max) qt /= 2;
+    while (qt > 1 && n_tiles * nkv * (G / qt) <= pf_units()) qt /= 2;
+    if (qt_hint == 1 || qt_hint == 2 || qt_hint == 4)
+        while (qt > qt_hint) qt /= 2;
+    return qt;
+}
+
+// Into how many parts the keys are split: 1 unless the tiles are so few that the chip stays mostly
+// empty and the longest context (max_keys) gives every part at least 8 stages of 64 keys.
+extern "C" int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int max_keys) {
+    if (n_tiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv) return 1;
+    const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, 0);
+    const int blocks = n_tiles * nkv * ((nh / nkv) / qt);
+    const int want = (2 * pf_units()) / max(blocks, 1);
+    const int by_keys = ceil_div(max(max_keys, 1), PF_STAGE) / 8;
+    return max(1, min(min(want, by_keys), 16));
+}
+
+// Workspace of the split form, in floats: part_o and part_ml for n_rows rows of tiles.
+extern "C" int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split, long* o_floats, long* ml_floats) {
+    const int hdp = ceil_div(hd, 32) * 32;
+    *o_floats = (long)n_rows * nh * n_split * hdp;
+    *ml_floats = (long)n_rows * nh * n_split * 2;
+    return 0;
+}
+
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16_t* __restrict__ out, const int* __restrict__ tiles,
+                                                                 int nh, int hd, int hdp, int n_split) {
+    const int tile = blockIdx.x / PF_TOKENS, qtok = blockIdx.x % PF_TOKENS, head = blockIdx.y;
+    const int row0 = tiles[4 * tile + 1], cnt = tiles[4 * tile + 2], item0 = tiles[4 * tile + 3];
+    if (qtok >= cnt) return;                                       // (the whole block leaves)
+    attn_merge_splits(part_o, part_ml, out + ((size_t)(row0 + qtok) * nh + head) * hd,
+                      ((size_t)(item0 + qtok) * nh + head) * n_split, hd, hdp, n_split);
+}
+
+// tiles[n_tiles][4] = (row of the request in the block table, first row, rows (at most 64), index of
+// the first row among all rows of tiles).  n_split > 1 (fl_attn_prefill_splits): the keys are split,
+// part_o and part_ml hold fl_attn_prefill_workspace floats.
 extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int* tiles,
                                int n_tiles, const int* positions, const int* block_table,
                                int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
-                               float scale, int window, int qt_hint, hipStream_t stream) {
+                               float scale, int window, int qt_hint, float* part_o, float* part_ml, int n_split,
+                               hipStream_t stream) {
     FL_CHECK(n_tiles >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_prefill: bad head counts %d/%d", nh, nkv);
     FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "attn_prefill: head size %d must be a multiple of 8 up to 256", hd);
     FL_CHECK(page_size >= 8 && (page_size & (page_size - 1)) == 0,
@@ -402,32 +477,25 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     FL_CHECK(max_blocks <= PF_MAX_PAGES, "attn_prefill: %d pages per request, at most %d", max_blocks, PF_MAX_PAGES);
     FL_CHECK(window >= 0, "attn_prefill: negative window");
     FL_CHECK(scale > 0.f, "attn_prefill: the score scale must be positive");
+    FL_CHECK(n_split >= 1 && n_split <= 256, "attn_prefill: %d splits", n_split);
+    FL_CHECK(n_split == 1 || (part_o && part_ml && (uintptr_t)part_o % 16 == 0), "attn_prefill: splits need a 16-byte aligned workspace");
+    FL_CHECK(n_tiles <= 65535 / PF_TOKENS || n_split == 1, "attn_prefill: %d tiles are too many to split", n_tiles);
     if (n_tiles == 0) return 0;
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
     const int G = nh / nkv;
     const int hdp = ceil_div(hd, 32) * 32;
     int log2_ps = 0;
     while ((1 << log2_ps) < page_size) ++log2_ps;
-    // query heads per wave: a divisor of the group size; as many as leave room for two blocks per
-    // compute unit (two waves per SIMD hide each other's waits: measured 906 against 1314 us at 8192
-    // tokens with 2 heads instead of 4 at head size 128)
-    int qt = (G % 4 == 0) ? 4 : (G % 2 == 0 ? 2 : 1);
-    const int qt_max = hdp <= 64 ? 4 : 2;
-    while (qt > qt_max) qt /= 2;
-    // ... and few enough that the grid has more blocks than the chip has units (a short portion:
-    // measured 176 against 217 us for 512 tokens behind 7,680 with 1 head instead of 2)
-    while (qt > 1 && n_tiles * nkv * (G / qt) <= pf_units()) qt /= 2;
-    if (qt_hint == 1 || qt_hint == 2 || qt_hint == 4)
-        while (qt > qt_hint) qt /= 2;
-    dim3 grid(n_tiles, nkv * (G / qt));
+    const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, qt_hint);
+    dim3 grid(n_tiles, nkv * (G / qt), n_split);
     const float sl = scale * 1.4426950408889634f;
 #define FL_PF(HDP_, NS_)                                                                                       \
     if (NS_ == 3 && g_pf_stages == 3)                                                                          \
         launch_prefill<HDP_, NS_>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                                  max_blocks, nh, sl, window, log2_ps);                                        \
+                                  max_blocks, nh, sl, window, log2_ps, part_o, part_ml);                       \
     else                                                                                                       \
         launch_prefill<HDP_, 2>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                                max_blocks, nh, sl, window, log2_ps)
+                                max_blocks, nh, sl, window, log2_ps, part_o, part_ml)
     switch (hdp) {
         case 32: FL_PF(32, 3); break;
         case 64: FL_PF(64, 3); break;
@@ -440,5 +508,10 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     }
 #undef FL_PF
     FL_LAUNCH_CHECK();
+    if (n_split > 1) {
+        dim3 mg(n_tiles * PF_TOKENS, nh);
+        attn_prefill_merge_kernel<<<mg, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, tiles, nh, hd, hdp, n_split);
+        FL_LAUNCH_CHECK();
+    }
     return 0;
 }

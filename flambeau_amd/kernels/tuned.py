@@ -32,7 +32,8 @@ register_signatures({
     "fl_gemm_mid_partials": [P, P, P, I, I, I, P, I, F, P],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
-    "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
+    "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, P, I, P],
+    "fl_attn_prefill_splits": [I, I, I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
 })
 
@@ -413,17 +414,21 @@ PREFILL_TILE = 64        # query tokens per block of the tiled kernel
 def attention_metadata(batch) -> dict:
     """Work lists for the attention kernels of one batch: ``attn_rows`` = (row, position, request,
     0) of the rows that run as single queries (decode rows and rows of short portions);
-    ``attn_tiles`` = (request, first row, rows) for every 64 rows of the longer portions."""
+    ``attn_tiles`` = (request, first row, rows, index of the first row among all rows of tiles) for
+    every 64 rows of the longer portions."""
     import numpy as np
     rows, tiles = [], []
+    n_tile_rows = 0
     for s, (q0, ql, p0) in enumerate(zip(batch.q_starts, batch.q_lens, batch.start_pos)):
         if ql <= SHORT_PORTION:
             rows += [(q0 + i, p0 + i, s, 0) for i in range(ql)]
         else:
             for off in range(0, ql, PREFILL_TILE):
-                tiles.append((s, q0 + off, min(PREFILL_TILE, ql - off)))
+                cnt = min(PREFILL_TILE, ql - off)
+                tiles.append((s, q0 + off, cnt, n_tile_rows))
+                n_tile_rows += cnt
     return {"attn_rows": np.asarray(rows, dtype=np.int32).reshape(-1, 4),
-            "attn_tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 3)}
+            "attn_tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 4)}
 
 
 def decode_splits(n_items: int, n_kv_heads: int, group: int, max_ctx: int) -> int:
@@ -456,16 +461,37 @@ def attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, par
     return out
 
 
-def attn_prefill(q, out, cache, tiles, positions, table, n_heads, scale, window, heads_per_wave: int = 0):
+def attn_prefill_splits(n_tiles: int, n_heads: int, n_kv_heads: int, head_dim: int, max_keys: int) -> int:
+    """Into how many parts the tiled kernel wants the keys split for a batch of this shape (1: not
+    at all; more when few tiles face a long context)."""
+    from .library import load
+    return load().fl_attn_prefill_splits(n_tiles, n_heads, n_kv_heads, head_dim, max_keys)
+
+
+def attn_prefill(q, out, cache, tiles, positions, table, n_heads, scale, window, heads_per_wave: int = 0,
+                 n_split: int = 1, part_o=None, part_ml=None):
+    """Attention of the longer portions; ``tiles[i] = (request's row in ``table``, first row, rows,
+    index of the first row among all rows of tiles)``.  With ``n_split`` > 1 the keys are split and
+    merged; ``part_o`` / ``part_ml``: float32 workspaces of rows x heads x n_split x (head_dim rounded
+    up to 32, and 2) values, rows = all rows of tiles."""
     n = q.shape[0]
     hd = cache.head_dim
     n_tiles = tiles.shape[0]
+    if n_split > 1:
+        n_rows = int(tiles[-1, 2] + tiles[-1, 3]) if isinstance(tiles, torch.Tensor) and not tiles.is_cuda else None
+        hdp = -(-hd // 32) * 32
+        if part_o is None or part_ml is None:
+            raise KernelError("attn_prefill: splits need a workspace")
+        if n_rows is not None and (part_o.numel() < n_rows * n_heads * n_split * hdp or part_ml.numel() < n_rows * n_heads * n_split * 2):
+            raise KernelError("attn_prefill: workspace too small for the splits")
     call("fl_attn_prefill", _check(q, "attn.q", torch.bfloat16, (n, n_heads * hd)),
          _check(out, "attn.out", torch.bfloat16, (n, n_heads * hd)), _check(cache.pool, "attn.cache", torch.bfloat16),
-         _check(tiles, "attn.tiles", torch.int32, (n_tiles, 3)), n_tiles,
+         _check(tiles, "attn.tiles", torch.int32, (n_tiles, 4)), n_tiles,
          _check(positions, "attn.positions", torch.int32, (n,)),
          _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads, hd,
-         cache.page_size, cache.n_pages, float(scale), int(window), int(heads_per_wave), stream_handle())
+         cache.page_size, cache.n_pages, float(scale), int(window), int(heads_per_wave),
+         _check(part_o, "attn.part_o", torch.float32) if part_o is not None else None,
+         _check(part_ml, "attn.part_ml", torch.float32) if part_ml is not None else None, int(n_split), stream_handle())
     return out
 
 
@@ -491,7 +517,16 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
     if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table)):
         return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
     if tiles.shape[0]:
-        attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window)
+        # few tiles before a long context: the keys are split too, so that the chip has blocks enough
+        longest = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + PREFILL_TILE)
+        p_split = attn_prefill_splits(tiles.shape[0], n_heads, cache.n_kv_heads, cache.head_dim, longest)
+        p_o = p_ml = None
+        if p_split > 1:
+            n_rows = sum(ql for ql in batch.q_lens if ql > SHORT_PORTION)
+            hdp = -(-cache.head_dim // 32) * 32
+            p_o = rt.buffer("attn_tile_part_o", n_rows * n_heads * p_split, hdp, torch.float32, max_rows=1 << 24)
+            p_ml = rt.buffer("attn_tile_part_ml", n_rows * n_heads * p_split, 2, torch.float32, max_rows=1 << 24)
+        attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window, n_split=p_split, part_o=p_o, part_ml=p_ml)
     if rows.shape[0]:
         group = n_heads // cache.n_kv_heads
         max_ctx = batch.ctx_bound or batch.max_ctx_len

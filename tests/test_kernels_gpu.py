@@ -653,16 +653,22 @@ def tiles_for(seqs, tile=64):
     rows, at = [], 0
     for s, (_, ql) in enumerate(seqs):
         for off in range(0, ql, tile):
-            rows.append((s, at + off, min(tile, ql - off)))
+            rows.append((s, at + off, min(tile, ql - off), at + off))         # every row is a row of a tile here
         at += ql
-    return torch.tensor(rows, dtype=torch.int32, device=DEV).reshape(-1, 3)
+    return torch.tensor(rows, dtype=torch.int32, device=DEV).reshape(-1, 4)
 
 
-@pytest.mark.parametrize("heads_per_wave", [0, 1])
+def split_workspace(n_rows, nh, hd, n_split):
+    hdp = -(-hd // 32) * 32
+    return (torch.full((n_rows * nh * n_split * hdp,), float("nan"), dtype=torch.float32, device=DEV),
+            torch.full((n_rows * nh * n_split * 2,), float("nan"), dtype=torch.float32, device=DEV))
+
+
+@pytest.mark.parametrize("heads_per_wave,n_split", [(0, 1), (1, 1), (0, 3), (2, 7)])
 @pytest.mark.parametrize("nh,nkv,hd,ps,window", [(32, 8, 128, 16, 0), (4, 2, 16, 8, 16), (6, 1, 24, 16, 0),
                                                 (5, 5, 32, 16, 24), (8, 4, 64, 8, 0), (4, 2, 256, 32, 100),
                                                 (6, 3, 40, 64, 37), (2, 1, 160, 128, 0), (8, 2, 96, 16, 70)])
-def test_attn_prefill_against_plain_and_reference(nh, nkv, hd, ps, window, heads_per_wave):
+def test_attn_prefill_against_plain_and_reference(nh, nkv, hd, ps, window, heads_per_wave, n_split):
     # (context, queries): a whole prompt, a portion deep in a context, one that starts mid-page,
     # a portion that is no multiple of the tile, a short one
     seqs = [(200, 200), (300, 70), (ps * 5 + 3, 9), (131, 130), (64, 64), (17, 16)]
@@ -671,8 +677,10 @@ def test_attn_prefill_against_plain_and_reference(nh, nkv, hd, ps, window, heads
     scale = 1 / math.sqrt(hd)
     q2 = case["q"].reshape(n, nh * hd)
     out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    # with n_split > 1 the keys of every tile are split (some parts are empty: 7 parts of 1 to 5 stages) and merged
+    part_o, part_ml = split_workspace(n, nh, hd, n_split) if n_split > 1 else (None, None)
     tuned().attn_prefill(q2, out, case["cache"], tiles_for(seqs), case["pos_d"], case["table"], nh, scale, window,
-                         heads_per_wave)
+                         heads_per_wave, n_split=n_split, part_o=part_o, part_ml=part_ml)
     plain = torch.empty_like(out)
     ops().attn_plain(q2, plain, case["cache"], case["pos_d"], case["seq_d"], case["table"], nh, scale, window)
     ref = attention_case_ref(case, scale, window)
@@ -709,12 +717,14 @@ def test_attn_prefill_peaked_scores_find_single_keys():
         t = [lo, i, (i // ps) * ps if (i // ps) * ps >= lo else lo, min(i, lo + 15)][i % 4]
         targets.append(t)
         q[i] = (K[t, 0] / K[t, 0].norm() * 60.0).to(torch.bfloat16)          # all heads alike
-    out = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
-    tuned().attn_prefill(q.reshape(n, nh * hd), out, case["cache"], tiles_for(seqs), case["pos_d"], case["table"], nh,
-                         1.0, window)
     case["q"] = q
     ref = attention_case_ref(case, 1.0, window)
-    assert (out.double().reshape(n, nh, hd) - ref).abs().max() < 2e-2 * ref.abs().max()
+    for n_split in (1, 2):          # whole, and with the keys of every tile in two parts
+        out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        part_o, part_ml = split_workspace(n, nh, hd, n_split) if n_split > 1 else (None, None)
+        tuned().attn_prefill(q.reshape(n, nh * hd), out, case["cache"], tiles_for(seqs), case["pos_d"], case["table"], nh,
+                             1.0, window, n_split=n_split, part_o=part_o, part_ml=part_ml)
+        assert (out.double().reshape(n, nh, hd) - ref).abs().max() < 2e-2 * ref.abs().max()
     # and the reference indeed picks single keys
     V = case["V"][0]
     hits = sum(float((ref[i, 0] - V[targets[i], 0]).abs().max()) < 0.05 for i in range(n))

@@ -57,7 +57,7 @@ def step_for(rt, seqs, page_size, n_pages, shuffle_seed=0):
     batch = HostBatch(q_starts, q_lens, starts, list(range(len(seqs))), at, 0)
     i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=DEV)
     extra = {k: i32(v) for k, v in tuned.attention_metadata(batch).items()}
-    extra["attn_tiles"] = extra["attn_tiles"].reshape(-1, 3)
+    extra["attn_tiles"] = extra["attn_tiles"].reshape(-1, 4)
     extra["attn_rows"] = extra["attn_rows"].reshape(-1, 4)
     return StepState(n_tokens=at, n_seqs=len(seqs), tokens=i32([0] * at), positions=i32(pos), tok_seq=i32(tok_seq),
                      seq_slots=i32(range(len(seqs))), seq_q_start=i32(q_starts), seq_q_len=i32(q_lens),
