@@ -12,6 +12,7 @@ from tiny_configs import TINY, write_sharpened
 pytestmark = pytest.mark.gpu
 
 STORE = {"float32": "float32", "bfloat16": "bfloat16"}
+STORE_DTYPE = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 LENGTHS = {"A": [5, 12, 23, 40, 70, 97], "B": [1, 31, 97, 64, 129], "C": [3, 50, 33, 150, 81]}
 
 
@@ -279,3 +280,26 @@ def test_cutting_at_real_layer_sizes(wide_model_dir, dtype):
         got = rh.run_in_process(runner, steps)
         assert not runner.manager.live
         rh.compare(got, reqs, ref, dtype, f"wide {what}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_short_portions_behind_a_long_context(tmp_path_factory, dtype):
+    """A request of 1,500 tokens in portions that shrink: the late portions give the tiled attention
+    few tiles with many keys, which it then splits over blocks and merges."""
+    import torch
+    from flambeau_amd.engine import ModelRunner, load_model
+    from flambeau_amd.kernels import tuned
+    from flambeau_amd.weights import write_random_model
+    config = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "hidden_act": "silu",
+              "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2,
+              "intermediate_size": 96, "vocab_size": 150, "rope_theta": 1e4, "sliding_window": None,
+              "rms_norm_eps": 1e-5, "max_position_embeddings": 2048, "tie_word_embeddings": False}
+    d = write_random_model(config, tmp_path_factory.mktemp("long") / "model", seed=12, std=0.08, gain_std=0.02,
+                           store_dtype=STORE_DTYPE[dtype])
+    assert tuned.attn_prefill_splits(2, 4, 2, 16, 1400) > 1
+    reqs = rh.make_requests(150, [1500], seed=9)
+    model, _ = load_model(d, dtype=dtype, max_batch_tokens=1024)
+    runner = ModelRunner(model, n_pages=100, page_size=16, max_slots=2, max_logit_rows=1024)
+    steps = rh.trace_portions(reqs, sizes=(700, 500, 100, 64, 9, 70, 30, 27))
+    got = rh.run_in_process(runner, steps)
+    rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, "long context")
