@@ -30,6 +30,7 @@ class Runtime:
         self.tuned = bool(tuned) and dtype == torch.bfloat16
         self.max_batch_tokens = int(max_batch_tokens)
         self._buffers: dict = {}
+        self._views: dict = {}
         self._scope = ""
 
     # ------------------------------------------------------------ buffers
@@ -41,12 +42,18 @@ class Runtime:
         if rows > cap:
             raise KernelError(f"buffer '{name}': {rows} rows asked, at most {cap} allowed")
         key = (self._scope, name, cols, dtype)
+        view = self._views.get((key, rows))             # (slicing a tensor costs a microsecond or two, a step asks 400 times)
+        if view is not None:
+            return view
         buf = self._buffers.get(key)
         if buf is None or buf.shape[0] < rows:
             size = min(cap, max(16, 1 << max(rows - 1, 0).bit_length()))
             buf = torch.empty((size, cols), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-        return buf[:rows]
+            for k in [k for k in self._views if k[0] == key]:
+                del self._views[k]
+        view = self._views[(key, rows)] = buf[:rows]
+        return view
 
     def scope(self, name: str):
         """Buffers asked for inside ``with rt.scope(name)`` are separate from all others (a

@@ -64,8 +64,13 @@ def register_signatures(extra: dict) -> None:
             fn.restype = c_int
 
 
+_functions: dict = {}
+
+
 def call(name: str, *args) -> None:
-    lib = load()
-    rc = getattr(lib, name)(*args)
+    fn = _functions.get(name)
+    if fn is None:
+        fn = _functions[name] = getattr(load(), name)
+    rc = fn(*args)
     if rc != 0:
-        raise KernelError(f"{name}: {lib.fl_last_error().decode(errors='replace')} (code {rc})")
+        raise KernelError(f"{name}: {load().fl_last_error().decode(errors='replace')} (code {rc})")

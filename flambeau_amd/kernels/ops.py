@@ -23,8 +23,27 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise KernelError(f"unsupported dtype {dtype}: the kernels take float32 and bfloat16") from None
 
 
+_pinned_stream = None
+
+
 def stream_handle() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The stream kernels are launched on: torch's current one, or the one pinned for a forward pass."""
+    return _pinned_stream if _pinned_stream is not None else torch.cuda.current_stream().cuda_stream
+
+
+class pinned_stream:
+    """``with pinned_stream():`` every launch inside goes to the stream that is current on entry.
+    Asking torch for its current stream at each of a step's two hundred launches costs more than
+    the launches; nothing inside a forward pass changes the stream."""
+
+    def __enter__(self):
+        global _pinned_stream
+        self.prev = _pinned_stream
+        _pinned_stream = torch.cuda.current_stream().cuda_stream
+
+    def __exit__(self, *exc):
+        global _pinned_stream
+        _pinned_stream = self.prev
 
 
 def _check(t: torch.Tensor, name: str, dtype=None, shape=None):
@@ -37,8 +56,15 @@ def _check(t: torch.Tensor, name: str, dtype=None, shape=None):
     if dtype is not None and t.dtype != dtype:
         raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
     if shape is not None:
-        if t.dim() != len(shape) or any(e is not None and e != s for s, e in zip(t.shape, shape)):
-            raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        have = t.shape
+        ok = len(have) == len(shape)
+        if ok:
+            for s, e in zip(have, shape):
+                if e is not None and e != s:
+                    ok = False
+                    break
+        if not ok:
+            raise KernelError(f"{name}: shape {tuple(have)}, expected {tuple(shape)}")
     return t.data_ptr()
 
 

@@ -113,6 +113,10 @@ class DecoderModel:
 
     # ------------------------------------------------------------ the forward pass of one batch
     def forward(self, step, caches, max_logit_rows: int):
+        with ops.pinned_stream():             # one look-up of torch's current stream for all launches of the pass
+            return self._forward(step, caches, max_logit_rows)
+
+    def _forward(self, step, caches, max_logit_rows: int):
         """Logits ``[R, vocab]`` (float32) at ``step.logit_rows``; ``caches[i]`` belongs to
         run-order entry ``i``."""
         rt = self.rt
