@@ -181,8 +181,11 @@ extern "C" int fl_add_inplace(float* x, const float* delta, long n, hipStream_t 
 
 // ------------------------------------------------------------------ plain GEMM
 // out[m, n] = sum_k x[m,k] * w[n,k]; 64x64 tile per block, 4x4 per thread, k in steps of 16.
-// Each output element is one float accumulator fed in rising k: the result of a row does not
-// depend on how many rows the call has.
+// Each output element is summed in a fixed order (rising k): the result of a row does not depend on
+// how many rows the call has.  The 16 products of a step are added in a chain of their own and the
+// steps' sums with a compensated (Kahan) addition, still all in float: over K = 14336 a single
+// chain loses about sqrt(K) roundings, which is what showed in the 32-bit path's logits (6.6e-5 at
+// 7B layer sizes against a float64 reference, against a bound of 1e-4).
 template <typename TIn, typename TOut>
 __global__ __launch_bounds__(256) void gemm_plain_kernel(const TIn* __restrict__ x,
                                                          const TIn* __restrict__ w,
@@ -192,11 +195,11 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(const TIn* __restrict__
     __shared__ float ws[16][68];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
-    float acc[4][4];
+    float acc[4][4], lost[4][4];              // the running sums and what their roundings have lost so far
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+        for (int j = 0; j < 4; ++j) { acc[i][j] = 0.f; lost[i][j] = 0.f; }
     for (int k0 = 0; k0 < K; k0 += 16) {
         for (int e = threadIdx.x; e < 1024; e += 256) {
             const int row = e >> 4, kk = e & 15;
@@ -206,6 +209,11 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(const TIn* __restrict__
             ws[kk][row] = (gn < N && gk < K) ? to_f32(w[(size_t)gn * K + gk]) : 0.f;
         }
         __syncthreads();
+        float part[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < 16; ++kk) {
             float a[4], b[4];
@@ -216,8 +224,17 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(const TIn* __restrict__
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
         }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float y = part[i][j] - lost[i][j];
+                const float t = acc[i][j] + y;
+                lost[i][j] = (t - acc[i][j]) - y;
+                acc[i][j] = t;
+            }
         __syncthreads();
     }
 #pragma unroll
@@ -255,12 +272,14 @@ extern "C" int fl_gemm_plain(const void* x, const void* w, void* out, int in_dty
 __global__ __launch_bounds__(64) void rope_table_kernel(const int* __restrict__ positions, int rot, float theta,
                                                         float2* __restrict__ cs) {
     const int token = blockIdx.x, half = rot >> 1;
-    const float pos = (float)positions[token];
+    // The angle is formed in double: in float a position of some thousands times a frequency near 1
+    // is already off by 1e-4 rad, which is the largest error left in the 32-bit path's logits; the
+    // table itself is float.
+    const double pos = (double)positions[token];
     for (int i = threadIdx.x; i < half; i += 64) {
-        const float exponent = 2.0f * (float)i / (float)rot;
-        const float inv_freq = 1.0f / powf(theta, exponent);
-        const float angle = pos * inv_freq;
-        cs[(size_t)token * half + i] = make_float2(cosf(angle), sinf(angle));
+        const double inv_freq = pow((double)theta, -2.0 * (double)i / (double)rot);
+        const double angle = pos * inv_freq;
+        cs[(size_t)token * half + i] = make_float2((float)cos(angle), (float)sin(angle));
     }
 }
 
@@ -326,10 +345,9 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
                 const float2 v = cs[(size_t)token * half + i];
                 c = v.x; s = v.y;
             } else {
-                const float exponent = 2.0f * (float)i / (float)rot;
-                const float inv_freq = 1.0f / powf(theta, exponent);
-                const float angle = (float)pos * inv_freq;
-                c = cosf(angle); s = sinf(angle);
+                // (in double, as in rope_table_kernel)
+                const double angle = (double)pos * pow((double)theta, -2.0 * (double)i / (double)rot);
+                c = (float)cos(angle); s = (float)sin(angle);
             }
             const int at = paired ? 16 * (i >> 3) + (i & 7) : i;
             const float x0 = value(at), x1 = value(paired ? at + 8 : i + half);
