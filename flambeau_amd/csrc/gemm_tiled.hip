@@ -423,17 +423,19 @@ static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16
         launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu);
 }
 
+static int g_tiled_splits = 0;           // 0: chosen from the sizes (a fixed number for experiments)
+extern "C" int fl_gemm_tiled_set_splits(int s) { g_tiled_splits = s; return 0; }
+
 // How many ways K is split for a product of this shape: 1 if the grid fills the chip.
 extern "C" int fl_gemm_tiled_splits(int M, int N, int K) {
+    if (g_tiled_splits > 0) return max(1, min(g_tiled_splits, ceil_div(K, 32) / 8));
     const int blocks = ceil_div(M, TG_BM) * ceil_div(N, TG_BN);
     const int steps = ceil_div(K, 32);
     int splits = 1;
-    while (blocks * splits < 384 && splits < 16 && steps / (splits * 2) >= 8) splits *= 2;
+    while (blocks * splits < 288 && splits < 16 && steps / (splits * 2) >= 8) splits *= 2;          // (288: measured on the 7B shapes, 65 to 1,536 rows)
     return splits;
 }
 
-// epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up from the
-// N interleaved gate/up rows of w (K is not split then).
 // epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up from the
 // N interleaved gate/up rows of w (K is not split then).  in_ssq (or null): [M, in_parts] partial sums of
 // squares of the rows that x was made from; every token's results are multiplied by rsqrt(sum / K + eps).
