@@ -87,7 +87,8 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
     __shared__ float s_scale[NTT * 16];                               // row scale of the block's tokens
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // the same for the whole wave: LDS addresses of its copies are scalars
     const int wf = wave & 1, wt = wave >> 1;
     // Which tile: blocks go to the eight dies of the chip in turn (block b to die b % 8), each die
     // with an L2 of its own.  A die gets one contiguous eighth of the tiles, ordered in groups of 8
