@@ -53,7 +53,8 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
     const int G = nh / cache.n_kv_heads;
     const int* table = block_table + (size_t)it.z * max_blocks;
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // the same for the whole wave: what depends on it is scalar
     const int li = lane & 15, g = lane >> 4;
     const bf16_t* kv = (const bf16_t*)cache.base;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};

@@ -66,7 +66,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     constexpr bool SWIGLU = EPI == EPI_SWIGLU;
     extern __shared__ float red[];               // [NW][MT][64][4], then [NW * 4][16] for the row scale
     const int nw = blockDim.x >> 6;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // the same for the whole wave: what depends on it is scalar
     const int li = lane & 15, g = lane >> 4;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     // tiles of this row group: [n_steps][64 lanes][8 values]
