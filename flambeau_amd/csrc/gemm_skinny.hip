@@ -136,9 +136,15 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
         }
     }
 
-    // epilogue 3: where this token's key and value go (two dependent loads, early)
+    // epilogue 3: where this token's key and value go (two dependent loads) and the angles of this
+    // lane's pairs, all asked for now
     TokenPlace place = {-1, 0};
-    if (EPI == EPI_ROPE && MT == 1 && wave == 0 && li < M) place = rope_token_place(rs, li);
+    RopeAngles angles = {};
+    const bool angles_early = EPI == EPI_ROPE && MT == 1 && rs.rot >= 8;
+    if (EPI == EPI_ROPE && MT == 1 && wave == 0 && li < M) {
+        place = rope_token_place(rs, li);
+        if (angles_early) angles = rope_angles(rs, li, blockIdx.x * 16 + 4 * g, g);
+    }
 
     int s = s0;
     // iterations of U steps: every load of the iteration is issued before the first product needs
@@ -197,7 +203,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
             }
             if (EPI == EPI_ROPE) {
                 const int f0 = blockIdx.x * 16 + 4 * g;
-                rope_store4(rs, tok, place, f0, g, sum, MT == 1 && tok < M && f0 < N);
+                if (angles_early) rope_store4<true>(rs, tok, place, f0, g, sum, MT == 1 && tok < M && f0 < N, angles);
+                else rope_store4(rs, tok, place, f0, g, sum, MT == 1 && tok < M && f0 < N);
             } else if (EPI == EPI_RESIDUAL) {
                 const int f0 = blockIdx.x * 16 + 4 * g;
                 f32x4 nr;
