@@ -160,7 +160,8 @@ class ModelRunner:
         if pad_to is not None:
             rows = list(range(pad_to))          # a fixed-shape step computes every row's logits
         batch = HostBatch(q_starts, q_lens, starts, slots, n + n_pad, len(rows),
-                          ctx_bound=self.max_seq_len if pad_to is not None else None)
+                          ctx_bound=self.max_seq_len if pad_to is not None else None,
+                          every_row=rows == list(range(n + n_pad)))
         if pad_to is not None:
             width = mgr.max_blocks
         else:
@@ -298,7 +299,7 @@ class ModelRunner:
         elif gs.feedback != feedback:
             raise StepError("the token feedback buffer must be set before the first captured step")
         gs.graph.replay()
-        wanted = [i for i, e in enumerate(entries) if e.want]
+        wanted = [i for i, e in enumerate(entries) for _ in e.want]     # one row per wanted place
         if not wanted:
             return None
         if wanted == list(range(len(wanted))):

@@ -129,7 +129,7 @@ class DecoderModel:
         if step.logit_rows.shape[0] == 0:
             stream.flush()
             return None
-        every_row = step.host.n_logit_rows == step.n_tokens          # a decode step: rows 0 .. n - 1 in order
+        every_row = step.host.every_row          # rows 0 .. n - 1 in order (a decode step, a whole prompt)
         if every_row or step.n_tokens <= SMALL_STEP:
             # a few rows cost what one row costs: all of them take the path of a decode step (the
             # same kernels whatever is wanted), and the wanted ones are picked afterwards

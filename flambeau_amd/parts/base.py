@@ -93,6 +93,7 @@ class HostBatch:
     n_tokens: int
     n_logit_rows: int
     ctx_bound: int | None = None   # set for a fixed-shape batch (graph replay): longest context it may ever hold
+    every_row: bool = False        # the wanted rows are exactly rows 0 .. n_tokens - 1, in that order
 
     @property
     def n_seqs(self): return len(self.q_lens)

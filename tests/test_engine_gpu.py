@@ -129,6 +129,50 @@ def test_logits_do_not_depend_on_neighbours(model_dirs, runners):
         assert np.array_equal(alone[("r3", p)], together[("r3", p)])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_wanted_rows_come_in_the_order_asked(model_dirs, runners, dtype):
+    """``want`` may name every token of a step out of order, or one place twice: the rows come back in
+    the order of the entries and of their ``want``, in eager steps and in captured decode steps."""
+    name = "A"
+    d = model_dirs[(name, STORE[dtype])]
+    reqs = rh.make_requests(256, [2, 16, 9, 5], seed=31)
+    ref = rh.plain_logits(d, reqs)
+    runner = runners(name, dtype)
+    perm = [int(i) for i in np.random.default_rng(4).permutation(16)]
+    assert perm != sorted(perm)
+    steps = [
+        dict(entries=[dict(id="r0", tokens=reqs["r0"], want=[1, 0])], end=["r0"]),
+        dict(entries=[dict(id="r0", tokens=reqs["r0"], want=[0, 0])], end=["r0"]),
+        dict(entries=[dict(id="r0", tokens=reqs["r0"], want=[1, 1, 0, 1])], end=["r0"]),
+        dict(entries=[dict(id="r1", tokens=reqs["r1"], want=perm)], end=["r1"]),
+        # two requests whose wanted rows together cover every row of the step, out of order
+        dict(entries=[dict(id="r2", tokens=reqs["r2"][:3], want=[2, 1, 0]), dict(id="r3", tokens=reqs["r3"][:2], want=[0, 1])], end=[]),
+        # decode steps (captured): a place wanted twice, beside a request that wants nothing
+        dict(entries=[dict(id="r2", tokens=[reqs["r2"][3]], want=[0, 0]), dict(id="r3", tokens=[reqs["r3"][2]], want=[])], end=[]),
+        dict(entries=[dict(id="r3", tokens=[reqs["r3"][3]], want=[0, 0, 0]), dict(id="r2", tokens=[reqs["r2"][4]], want=[0])], end=["r2", "r3"]),
+    ]
+    from flambeau_amd.engine import StepEntry
+    tol = rh.tolerance(dtype, max(float(np.abs(r).max()) for r in ref.values()))
+    pos = {}
+    for s in steps:
+        entries = []
+        for e in s["entries"]:
+            if e["id"] not in runner.manager.live:
+                assert runner.begin(e["id"])
+                pos[e["id"]] = 0
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+        rows = runner.step(entries).cpu().double().numpy()
+        expect = [(e["id"], pos[e["id"]] + w) for e in s["entries"] for w in e["want"]]
+        assert rows.shape[0] == len(expect)
+        for row, (rid, p) in zip(rows, expect):
+            assert np.abs(row - ref[rid][p]).max() <= tol, (s, rid, p)
+        for e in s["entries"]:
+            pos[e["id"]] += len(e["tokens"])
+        for rid in s["end"]:
+            runner.end(rid)
+    assert not runner.manager.live
+
+
 def test_step_refuses_bad_batches(model_dirs, runners):
     from flambeau_amd.cache import CacheError
     from flambeau_amd.engine import StepEntry, StepError

@@ -34,23 +34,30 @@ def test_replay_details(model_dirs, tmp_path):
     """A request may sit out a step; a step may want nothing (no file) or hold no entries; files
     are little-endian float32 [wanted, vocab] in the order of entries and of want."""
     d = model_dirs[("A", "float32")]
-    reqs = rh.make_requests(256, [10, 6], seed=8)
-    a, b = reqs["r0"], reqs["r1"]
+    reqs = rh.make_requests(256, [10, 6, 2], seed=8)
+    a, b, c = reqs["r0"], reqs["r1"], reqs["r2"]
     steps = [
         dict(entries=[dict(id="r0", tokens=a[:4], want=[])], end=[]),
         dict(entries=[dict(id="r1", tokens=b[:3], want=[2, 0])], end=[]),
         dict(entries=[], end=[]),
         dict(entries=[dict(id="r1", tokens=b[3:], want=[2]), dict(id="r0", tokens=a[4:], want=[5, 0])], end=["r0", "r1"]),
+        # every token of the step wanted, out of order; then one place twice
+        dict(entries=[dict(id="r2", tokens=c, want=[1, 0])], end=["r2"]),
+        dict(entries=[dict(id="r2", tokens=c, want=[0, 0])], end=["r2"]),
     ]
     lines = "".join(json.dumps(dict(step=10 + i, **s)) + "\n" for i, s in enumerate(steps))
     out = tmp_path / "o"
     r = subprocess.run([sys.executable, str(rh.ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", "float32",
                         "--out", str(out), "--max-tokens", "128"], input=lines, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-3000:]
-    assert r.stdout.split() == ["done", "10", "done", "11", "done", "12", "done", "13"]
-    assert sorted(p.name for p in out.iterdir()) == ["11.f32", "13.f32"]
+    assert r.stdout.split() == ["done", "10", "done", "11", "done", "12", "done", "13", "done", "14", "done", "15"]
+    assert sorted(p.name for p in out.iterdir()) == ["11.f32", "13.f32", "14.f32", "15.f32"]
     ref = rh.plain_logits(d, reqs)
     s11 = np.fromfile(out / "11.f32", dtype="<f4").reshape(2, 256)
     s13 = np.fromfile(out / "13.f32", dtype="<f4").reshape(3, 256)
-    for row, (rid, p) in zip(list(s11) + list(s13), [("r1", 2), ("r1", 0), ("r1", 5), ("r0", 9), ("r0", 4)]):
+    s14 = np.fromfile(out / "14.f32", dtype="<f4").reshape(2, 256)
+    s15 = np.fromfile(out / "15.f32", dtype="<f4").reshape(2, 256)
+    assert np.abs(ref["r2"][0] - ref["r2"][1]).max() > 1e-3          # the two rows can be told apart
+    for row, (rid, p) in zip(list(s11) + list(s13) + list(s14) + list(s15),
+                             [("r1", 2), ("r1", 0), ("r1", 5), ("r0", 9), ("r0", 4), ("r2", 1), ("r2", 0), ("r2", 0), ("r2", 0)]):
         assert np.abs(row - ref[rid][p]).max() < 1e-4
