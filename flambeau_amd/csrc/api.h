@@ -101,6 +101,19 @@ int fl_gemm_tiled_residual_parts(int M, int N, int K);
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                    const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
                    int n_pages, float scale, int window, int n_split, hipStream_t stream);
+// fl_attn_decode for callers that cannot allocate device memory (code under graph capture, tight
+// serving loops, harnesses that forbid it).  It has no counterpart in the reference.  The splits'
+// partial results, which fl_attn_decode takes as part_o / part_ml, go to an array of
+// FL_ATTN_DECODE_STATIC_FLOATS floats (8 MiB) that is part of the library's image on every GPU it
+// runs on; the call allocates and frees nothing.  It refuses n_items * nh * n_split * (hd rounded
+// up to 32, + 2) floats beyond that size.  Every call on a GPU uses that GPU's one array: calls
+// that overlap on one GPU (two streams, two threads) race; calls on one stream do not.  Nothing in
+// the array has to start at zero: every slot a call reads was written by the same call before.
+#define FL_ATTN_DECODE_STATIC_FLOATS (2u << 20)
+int fl_attn_decode_static(const void* q, void* out, const void* cache_base, const int* items, int n_items,
+                          const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
+                          int n_pages, float scale, int window, int n_split, hipStream_t stream);
+long fl_attn_decode_static_capacity(void);
 int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int* tiles, int n_tiles,
                     const int* positions, const int* block_table, int max_blocks, int nh, int nkv, int hd,
                     int page_size, int n_pages, float scale, int window, int qt_hint, float* part_o, float* part_ml,

@@ -26,6 +26,7 @@
 #include "common.h"
 #include "api.h"
 #include "attn_merge.h"
+#include <mutex>
 
 #define DEC_WAVES 4
 #define DEC_CHUNK 32
@@ -281,17 +282,17 @@ extern "C" int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split
     return 0;
 }
 
-extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml,
+static int attn_decode_launch(const char* who, const void* q, void* out, float* part_o, float* part_ml,
                               const void* cache_base, const int* items, int n_items, const int* block_table,
                               int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
                               float scale, int window, int n_split, hipStream_t stream) {
-    FL_CHECK(n_items >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_decode: bad head counts %d/%d", nh, nkv);
-    FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "attn_decode: head size %d must be a multiple of 8 up to 256", hd);
-    FL_CHECK(page_size % 8 == 0, "attn_decode: page size %d must be a multiple of 8", page_size);
-    FL_CHECK(n_split >= 1 && n_split <= 256, "attn_decode: %d splits", n_split);
-    FL_CHECK(n_split == 1 || (part_o && part_ml), "attn_decode: splits need a workspace");
-    FL_CHECK(window >= 0, "attn_decode: negative window");
-    FL_CHECK((uintptr_t)items % 16 == 0, "attn_decode: the items must be 16-byte aligned");
+    FL_CHECK(n_items >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "%s: bad head counts %d/%d", who, nh, nkv);
+    FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "%s: head size %d must be a multiple of 8 up to 256", who, hd);
+    FL_CHECK(page_size % 8 == 0, "%s: page size %d must be a multiple of 8", who, page_size);
+    FL_CHECK(n_split >= 1 && n_split <= 256, "%s: %d splits", who, n_split);
+    FL_CHECK(n_split == 1 || (part_o && part_ml), "%s: splits need a workspace", who);
+    FL_CHECK(window >= 0, "%s: negative window", who);
+    FL_CHECK((uintptr_t)items % 16 == 0, "%s: the items must be 16-byte aligned", who);
     if (n_items == 0) return 0;
     int ps_shift = -1;
     if ((page_size & (page_size - 1)) == 0)
@@ -324,4 +325,65 @@ extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* pa
         FL_LAUNCH_CHECK();
     }
     return 0;
+}
+
+extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml,
+                              const void* cache_base, const int* items, int n_items, const int* block_table,
+                              int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
+                              float scale, int window, int n_split, hipStream_t stream) {
+    return attn_decode_launch("attn_decode", q, out, part_o, part_ml, cache_base, items, n_items, block_table, max_blocks,
+                              nh, nkv, hd, page_size, n_pages, scale, window, n_split, stream);
+}
+
+// ---- the same without any allocation: the splits' partial results go to an array that is part of
+// the library's image on every GPU.  `scratch` is a host-side stand-in for that array, not a device
+// address; its address on the current device is asked for once per device and kept.
+static __device__ __align__(256) float scratch[FL_ATTN_DECODE_STATIC_FLOATS];
+
+#define FL_MAX_DEVICES 64
+static float* g_scratch_ptr[FL_MAX_DEVICES];       // per device: where `scratch` lies there
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    FL_CHECK(e == hipSuccess, "attn_decode_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    FL_CHECK(dev >= 0 && dev < FL_MAX_DEVICES, "attn_decode_static: device %d, at most %d are known", dev, FL_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        FL_CHECK(e == hipSuccess && p, "attn_decode_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                 hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" long fl_attn_decode_static_capacity(void) { return (long)FL_ATTN_DECODE_STATIC_FLOATS; }
+
+extern "C" int fl_attn_decode_static(const void* q, void* out, const void* cache_base, const int* items, int n_items,
+                                     const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,
+                                     int n_pages, float scale, int window, int n_split, hipStream_t stream) {
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    if (n_split > 1 && n_items > 0) {
+        FL_CHECK(nh > 0 && hd > 0 && hd <= 256 && n_split <= 256, "attn_decode_static: bad sizes (%d heads, head size %d, %d splits)",
+                 nh, hd, n_split);
+        const long hdp = ceil_div(hd, 32) * 32;
+        const long slots = (long)n_items * nh * n_split;
+        const long o_floats = (slots * hdp + 63) / 64 * 64;          // the pairs start 256-byte aligned
+        const long need = o_floats + slots * 2;
+        FL_CHECK(need <= (long)FL_ATTN_DECODE_STATIC_FLOATS,
+                 "attn_decode_static: %d rows x %d heads x %d splits need %ld floats of scratch, the static array holds %ld "
+                 "(use fl_attn_decode with a workspace, or fewer splits)",
+                 n_items, nh, n_split, need, (long)FL_ATTN_DECODE_STATIC_FLOATS);
+        float* base = nullptr;
+        if (static_scratch(&base) != 0) return -1;
+        part_o = base;
+        part_ml = base + o_floats;
+    }
+    return attn_decode_launch("attn_decode_static", q, out, part_o, part_ml, cache_base, items, n_items, block_table,
+                              max_blocks, nh, nkv, hd, page_size, n_pages, scale, window, n_split, stream);
 }
