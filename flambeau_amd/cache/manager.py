@@ -37,6 +37,7 @@ class PagePool:
         self.n_pages = n_pages
         self._free = deque(range(n_pages))
         self._is_free = [True] * n_pages
+        self.n_acquired = 0                     # pages handed out so far (more than n_pages: pages were used again)
 
     @property
     def n_free(self) -> int:
@@ -47,6 +48,7 @@ class PagePool:
             return None
         p = self._free.popleft()
         self._is_free[p] = False
+        self.n_acquired += 1
         return p
 
     def release(self, page: int) -> None:

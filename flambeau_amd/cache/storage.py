@@ -70,6 +70,12 @@ class CacheStorage:
         for t in self.states.values():
             t.index_fill_(0, idx, 0)
 
+    def fill(self, value: float) -> None:
+        """Overwrite every page of every pool (a debugging aid: with NaN, a read of a row that was
+        never written, or of a stale one that should have been masked, shows in the logits)."""
+        for p in self.pools:
+            p.fill_(value)
+
     def bytes_per_token(self) -> int:
         return sum(p.shape[0] * 2 * p.shape[3] * p.shape[5] * p.element_size() for p in self.pools)
 

@@ -316,10 +316,22 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
                 // are weighted with) comes from the matrix cores too: a value tile of ones
                 l[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones8, pmat[t], l[t], 0, 0, 0);
             }
-            // ---- O^T += V^T P^T
+            // ---- O^T += V^T P^T.  In a chunk at an end of [lo, p_last] the values of keys outside it
+            // (rows of a page that were never written, or belong to whoever holds the page now) are
+            // zeroed: their weights are 0, but 0 * NaN would not be
+            const bool edge = t0 < lo || t0 + 31 > p_last;             // the same for the whole block
+            u32x4 keep = {~0u, ~0u, ~0u, ~0u};
+            if (edge) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int k0 = t0 + 8 * g + 2 * e;
+                    keep[e] = ((k0 >= lo && k0 <= p_last) ? 0x0000FFFFu : 0u) | ((k0 + 1 >= lo && k0 + 1 <= p_last) ? 0xFFFF0000u : 0u);
+                }
+            }
 #pragma unroll
             for (int d = 0; d < DT; ++d) {
-                const bf16x8 vd = EARLY_V ? vt[EARLY_V ? d : 0] : *(const bf16x8*)(slot + (KT + half * DT + d) * 512 + lane * 8);
+                bf16x8 vd = EARLY_V ? vt[EARLY_V ? d : 0] : *(const bf16x8*)(slot + (KT + half * DT + d) * 512 + lane * 8);
+                if (edge) vd = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, vd) & keep);
 #pragma unroll
                 for (int t = 0; t < QT; ++t)
                     o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vd, pmat[t], o[t][d], 0, 0, 0);

@@ -26,6 +26,9 @@ def build_parser():
     ap.add_argument("--max-slots", type=int, default=64, help="most requests live at a time")
     ap.add_argument("--plain-kernels", action="store_true",
                     help="run the plain kernels in bfloat16 too (float32 always does)")
+    ap.add_argument("--poison-cache", action="store_true",
+                    help="fill the cache with NaN before the first step: a read of a row that was never "
+                         "written then shows in the logits")
     return ap
 
 
@@ -46,6 +49,8 @@ def main(argv=None) -> int:
                           tuned=not args.plain_kernels)
     runner = ModelRunner(model, n_pages=max_tokens // args.page_size, page_size=args.page_size,
                          max_slots=args.max_slots, max_logit_rows=max_tokens)
+    if args.poison_cache:
+        runner.storage.fill(float("nan"))
 
     for line in sys.stdin:
         line = line.strip()
@@ -71,4 +76,7 @@ def main(argv=None) -> int:
             if rid in runner.manager.live:
                 runner.end(rid)
         print(f"done {step_no}", flush=True)
+    pools = runner.manager.pools
+    print(f"trace_run: {sum(p.n_pages for p in pools)} pages in the pool, {sum(p.n_acquired for p in pools)} handed out",
+          file=sys.stderr)
     return 0

@@ -130,8 +130,9 @@ def run_in_process(runner, steps):
     return out
 
 
-def run_program(model_dir, dtype, steps, out_dir, max_tokens, vocab, extra=(), timeout=600):
-    """The same through ``bin/trace_run`` as a child process."""
+def run_program(model_dir, dtype, steps, out_dir, max_tokens, vocab, extra=(), timeout=600, stats=None):
+    """The same through ``bin/trace_run`` as a child process.  ``stats`` (a dict) receives the pool's
+    size and the number of pages handed out, which the program reports when its input ends."""
     lines = "".join(json.dumps(dict(step=i, **s)) + "\n" for i, s in enumerate(steps))
     cmd = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype,
            "--out", str(out_dir), "--max-tokens", str(max_tokens), *extra]
@@ -139,6 +140,11 @@ def run_program(model_dir, dtype, steps, out_dir, max_tokens, vocab, extra=(), t
     assert r.returncode == 0, f"trace_run failed ({r.returncode}):\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
     done = [l for l in r.stdout.splitlines() if l.startswith("done ")]
     assert done == [f"done {i}" for i in range(len(steps))], r.stdout[-2000:]
+    if stats is not None:
+        import re
+        m = re.search(r"trace_run: (\d+) pages in the pool, (\d+) handed out", r.stderr)
+        assert m, r.stderr[-2000:]
+        stats["pool"], stats["handed_out"] = int(m.group(1)), int(m.group(2))
     out, pos = {}, {}
     for i, s in enumerate(steps):
         n_want = sum(len(e["want"]) for e in s["entries"])
