@@ -50,13 +50,15 @@ class LLMEngine:
                                   decode_graphs=opt.decode_graphs)
         self.scheduler = Scheduler(self.runner.manager, max_batch_tokens=model.rt.max_batch_tokens,
                                    prefill_chunk_tokens=opt.prefill_chunk_tokens,
-                                   max_queue_depth=opt.max_queue_depth, eos_token_id=spec.eos_token_id,
+                                   max_queue_depth=opt.max_queue_depth,
+                                   eos_token_id=getattr(spec, "eos_token_ids", ()) or spec.eos_token_id,
                                    default_seed=opt.seed)
         self.sampler = DeviceSampler(model.rt.device, max(opt.inflight_slots, 1))
         # tokens drawn on the device are fed to the next step on the device: the host enqueues
         # step i + 1 while step i runs and reads step i's tokens afterwards
         self.runner.token_feedback = self.sampler.ids
         self._in_flight = None            # (scheduled, sampler handle) of the step the host has not read yet
+        self._pick_host = self._pick_dev = None
         self._next_id = 0
 
     @classmethod
@@ -129,15 +131,43 @@ class LLMEngine:
             finished += self.flush()                  # the step before; this one is running meanwhile
             self._in_flight = (sched, handle) if rows else None
             return finished
-        # penalties, bias or filters: the logits go to the host sampler, nothing stays in flight
+        # Some request wants penalties, a bias or filters: its logits go to the host sampler and nothing
+        # stays in flight.  Rows that the device can draw are still drawn there (by the same kernel,
+        # from the same numbers of their own generators), so a request's tokens do not depend on
+        # what its neighbours ask for.
         finished += self.flush()
-        host = logits.to("cpu").numpy() if rows else None
         sampled = {}
-        for i, s in enumerate(rows):
-            r = s.request
-            if r.status != "finished":            # (a stop token of the step before may just have ended it)
+        live = [i for i, s in enumerate(rows) if s.request.status != "finished"]   # (a stop token of the step before may just have ended one)
+        on_dev = [i for i in live if self.options.gpu_sampler and rows[i].request.params.device_ok]
+        if on_dev:
+            params = [rows[i].request.params for i in on_dev]
+            inv_t = [0.0 if p.is_greedy else 1.0 / p.temperature for p in params]
+            us = [0.0 if p.is_greedy else rows[i].request.rng.next_f32() for i, p in zip(on_dev, params)]
+            picked = logits if on_dev == list(range(logits.shape[0])) else self._pick_rows(logits, on_dev)
+            for i, t in zip(on_dev, self.sampler.sample(picked, inv_t, us)):
+                sampled[rows[i].request.request_id] = t
+        on_host = [i for i in live if i not in on_dev]
+        if on_host:
+            host = logits.to("cpu").numpy()
+            for i in on_host:
+                r = rows[i].request
                 sampled[r.request_id] = sample_host(host[i], r.params, r.output, r.rng)
         return finished + self.scheduler.commit(sched, sampled)
+
+    def _pick_rows(self, logits, idx):
+        """Rows ``idx`` of the step's logits, gathered on the device for the device sampler."""
+        from ..kernels import ops
+        n = len(idx)
+        if self._pick_host is None:
+            cap = max(self.options.inflight_slots, 1)
+            self._pick_host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self._pick_dev = torch.empty(cap, dtype=torch.int32, device=self.model.rt.device)
+        torch.cuda.current_stream().synchronize()          # the copy of the call before has left the pinned buffer
+        self._pick_host[:n] = torch.tensor(idx, dtype=torch.int32)
+        self._pick_dev[:n].copy_(self._pick_host[:n], non_blocking=True)
+        out = self.model.rt.buffer("logits_for_device_sampler", n, logits.shape[1], torch.float32,
+                                   max_rows=max(self.options.inflight_slots, 1))
+        return ops.gather_rows(logits, self._pick_dev[:n], out)
 
     # ------------------------------------------------------------ whole generations
     def generate(self, prompts, params=None) -> list:

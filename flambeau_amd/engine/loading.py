@@ -35,9 +35,12 @@ def load_model(model_dir, dtype="bfloat16", device="cuda:0", max_batch_tokens: i
 
 
 def random_model(config: dict, seed: int, dtype="bfloat16", device="cuda:0", max_batch_tokens: int = 2048,
-                 tuned: bool = True, std: float = 0.02, gain_std: float = 0.0, n_layers: int | None = None):
-    """A model with seeded random weights made on the device, without a folder.  ``n_layers``
-    keeps only the first layers of the configuration (for measurements that say so)."""
+                 tuned: bool = True, std: float = 0.02, gain_std: float = 0.0, n_layers: int | None = None,
+                 generate_on: str = "device"):
+    """A model with seeded random weights, without a folder.  ``n_layers`` keeps only the first layers
+    of the configuration (for measurements that say so).  ``generate_on``: "device" makes the
+    tensors with the GPU's generator (fast; its values are its own), "cpu" with the host's, which
+    gives the values that ``write_random_model`` writes for the same seed."""
     arch, cfg = config_from_dict(config, "config")
     rt = Runtime(device, parse_dtype(dtype), max_batch_tokens, tuned)
     spec = arch.build_spec(cfg)
@@ -45,6 +48,9 @@ def random_model(config: dict, seed: int, dtype="bfloat16", device="cuda:0", max
         spec.layers = spec.layers[:n_layers]
         spec.run_order = [e for e in spec.run_order if e.layer < n_layers]
     model = DecoderModel(spec, rt)
-    src = RandomSource(model.manifest(), seed, std, gain_std, rt.dtype, device=rt.device)
+    if generate_on not in ("device", "cpu"):
+        raise ValueError(f"generate_on must be 'device' or 'cpu', got {generate_on!r}")
+    src = RandomSource(model.manifest(), seed, std, gain_std, rt.dtype,
+                       device=rt.device if generate_on == "device" else "cpu")
     load_weights(model, src)
     return model, cfg

@@ -60,6 +60,20 @@ class Request:
     def tokens(self) -> list:
         return self.prompt + self.output
 
+    def token_at(self, i: int):
+        """Token ``i`` of prompt + output, without joining the two lists."""
+        n = len(self.prompt)
+        return self.prompt[i] if i < n else self.output[i - n]
+
+    def token_slice(self, a: int, b: int) -> list:
+        """Tokens ``[a, b)`` of prompt + output; copies only what it returns."""
+        n = len(self.prompt)
+        if b <= n:
+            return self.prompt[a:b]
+        if a >= n:
+            return self.output[a - n:b - n]
+        return self.prompt[a:] + self.output[:b - n]
+
     @property
     def n_pending(self) -> int:
         return len(self.prompt) + len(self.output) - self.n_computed
@@ -74,14 +88,20 @@ class Scheduled:
 
 class Scheduler:
     def __init__(self, manager: CacheManager, *, max_batch_tokens: int, prefill_chunk_tokens: int = 512,
-                 max_queue_depth: int = 0, eos_token_id: int | None = None, default_seed: int = 0):
+                 max_queue_depth: int = 0, eos_token_id=None, default_seed: int = 0):
         if max_batch_tokens < 1 or prefill_chunk_tokens < 1:
             raise ValueError("token budgets must be positive")
         self.manager = manager
         self.max_batch_tokens = max_batch_tokens
         self.prefill_chunk_tokens = prefill_chunk_tokens
         self.max_queue_depth = max_queue_depth      # 0: no limit (routes.rs:481 "0 disables")
-        self.eos_token_id = eos_token_id
+        # one id or several: any of them ends a request
+        if eos_token_id is None:
+            self.eos_token_ids = frozenset()
+        elif isinstance(eos_token_id, int):
+            self.eos_token_ids = frozenset([eos_token_id])
+        else:
+            self.eos_token_ids = frozenset(int(t) for t in eos_token_id)
         self.default_seed = default_seed
         self.waiting: deque[Request] = deque()
         self.running: list[Request] = []            # in order of admission
@@ -182,7 +202,7 @@ class Scheduler:
                 continue
             upto = r.n_computed + 1
             if self._fits(planned, r, upto):
-                out.append(Scheduled(r, [r.tokens[r.n_computed]], True))
+                out.append(Scheduled(r, [r.token_at(r.n_computed)], True))
                 planned.append((r, upto))
                 budget -= 1
                 i += 1
@@ -205,7 +225,7 @@ class Scheduler:
             k = self._portion(planned, r, min(r.n_pending, budget, self.prefill_chunk_tokens))
             if k <= 0:
                 continue
-            out.append(Scheduled(r, r.tokens[r.n_computed:r.n_computed + k], k == r.n_pending))
+            out.append(Scheduled(r, r.token_slice(r.n_computed, r.n_computed + k), k == r.n_pending))
             planned.append((r, r.n_computed + k))
             budget -= k
 
@@ -220,7 +240,7 @@ class Scheduler:
             self.waiting.popleft()
             r.status = "running"
             self.running.append(r)
-            out.append(Scheduled(r, r.tokens[:k], k == r.n_pending))
+            out.append(Scheduled(r, r.token_slice(0, k), k == r.n_pending))
             planned.append((r, k))
             budget -= k
 
@@ -287,8 +307,7 @@ class Scheduler:
             r.output[at] = tok
             if r.pending_row is not None and PENDING not in r.output:
                 r.pending_row = None
-            stop = (not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id) \
-                or tok in r.params.stop_token_ids
+            stop = (not r.params.ignore_eos and tok in self.eos_token_ids) or tok in r.params.stop_token_ids
             if stop:
                 del r.output[at + 1:]
                 r.pending_row = None

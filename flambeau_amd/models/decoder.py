@@ -43,6 +43,8 @@ class ModelSpec:
     tied_head: bool = False
     eos_token_id: int | None = None
     bos_token_id: int | None = None
+    eos_token_ids: tuple = ()         # every id that ends a sequence (eos_token_id is the first)
+    ignored_tensors: tuple = ()       # name patterns (fnmatch) of tensors a file may hold and the model does not read
 
 
 SMALL_STEP = 16      # up to this many rows the output head runs on every row of a step

@@ -18,16 +18,19 @@ from .decoder import LayerSpec, ModelSpec, RunEntry
 def mistral_spec(cfg: MistralConfig) -> ModelSpec:
     norm = PartSpec("rmsnorm", dict(hidden_size=cfg.hidden_size, eps=cfg.rms_norm_eps))
     position = PartSpec("rope_neox", dict(head_dim=cfg.head_dim, theta=cfg.rope_theta))
-    mixer = PartSpec("paged_gqa_attention", dict(
-        hidden_size=cfg.hidden_size, n_heads=cfg.num_attention_heads,
-        n_kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim,
-        window=cfg.sliding_window, position=position))
     ffn = PartSpec("swiglu", dict(hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size))
-    block = PartSpec("prenorm", dict(mixer=mixer, feed_forward=ffn, norm=norm))
+
+    def block(window):
+        mixer = PartSpec("paged_gqa_attention", dict(
+            hidden_size=cfg.hidden_size, n_heads=cfg.num_attention_heads,
+            n_kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim,
+            window=window, position=position))
+        return PartSpec("prenorm", dict(mixer=mixer, feed_forward=ffn, norm=norm))
+
     layers = []
     for l in range(cfg.num_hidden_layers):
         p = f"model.layers.{l}."
-        layers.append(LayerSpec(block, {
+        layers.append(LayerSpec(block(cfg.window_of_layer(l)), {
             "mixer_norm.weight": p + "input_layernorm.weight",
             "mixer.q.weight": p + "self_attn.q_proj.weight",
             "mixer.k.weight": p + "self_attn.k_proj.weight",
@@ -52,6 +55,9 @@ def mistral_spec(cfg: MistralConfig) -> ModelSpec:
         tied_head=cfg.tie_word_embeddings,
         eos_token_id=cfg.eos_token_id,
         bos_token_id=cfg.bos_token_id,
+        eos_token_ids=cfg.eos_token_ids,
+        # tensors that files of this architecture may hold and the model does not read
+        ignored_tensors=("*.rotary_emb.inv_freq",) + (("lm_head.weight",) if cfg.tie_word_embeddings else ()),
     )
 
 

@@ -14,7 +14,9 @@ tensor (crates/forward/src/loader/primitives.rs:158-163).
 """
 from __future__ import annotations
 
+import fnmatch
 import json
+import warnings
 from pathlib import Path
 
 import torch
@@ -93,11 +95,19 @@ class SafetensorsDir:
             f.close()
 
 
-def check_against_manifest(manifest: dict, source) -> None:
+def check_against_manifest(manifest: dict, source, ignored=()) -> list:
+    """Raises ONE ``WeightError`` for everything that does not fit.  ``ignored``: name patterns
+    (``fnmatch``) of tensors the architecture says a file may hold without the model reading them;
+    those are skipped with a warning and returned."""
     have = set(source.names())
     want = set(manifest)
     missing = want - have
     unexpected = have - want
+    skipped = sorted(n for n in unexpected if any(fnmatch.fnmatchcase(n, pat) for pat in ignored))
+    unexpected -= set(skipped)
+    if skipped:
+        warnings.warn(f"{source.description}: {len(skipped)} tensors are not read by this model: "
+                      + ", ".join(skipped[:8]) + (" ..." if len(skipped) > 8 else ""), stacklevel=2)
     wrong_shape, wrong_dtype = [], []
     for name in want & have:
         shape, tag = source.info(name)
@@ -109,12 +119,13 @@ def check_against_manifest(manifest: dict, source) -> None:
             wrong_dtype.append((name, tag))
     if missing or unexpected or wrong_shape or wrong_dtype:
         raise WeightError(source.description, missing, unexpected, wrong_shape, wrong_dtype)
+    return skipped
 
 
 def load_weights(model, source, progress=None) -> None:
     """Check, move to the device, bind."""
     manifest = model.manifest()
-    check_against_manifest(manifest, source)
+    check_against_manifest(manifest, source, getattr(model.spec, "ignored_tensors", ()))
     tensors = {}
     for i, (name, (_, _, tspec)) in enumerate(manifest.items()):
         tensors[name] = model.rt.to_device(source.read(name), tspec.role)

@@ -180,6 +180,12 @@ def swiglu_mlp(x, w_gate, w_up, w_down):
     return linear(silu(linear(x, w_gate)) * linear(x, w_up), w_down)
 
 
+def default_scale(hd: int) -> float:
+    """Score scale when the weights give none: 1 / sqrt(head_dim).
+    crates/forward/src/core/composites/standard_attn.rs:418-420 ((head_dim as f32).sqrt().recip())."""
+    return 1.0 / math.sqrt(hd)
+
+
 def attention_mixer(x, w, prefix, positions, nh, nkv, hd, theta, window):
     """Q/K/V projections, rotation of Q and K (not V), attention, output projection.
 
@@ -192,7 +198,7 @@ def attention_mixer(x, w, prefix, positions, nh, nkv, hd, theta, window):
     v = linear(x, w[prefix + "v_proj.weight"]).reshape(n, nkv, hd)
     q = rope_neox(q, positions, theta)
     k = rope_neox(k, positions, theta)
-    o = attention(q, k, v, positions, 1.0 / math.sqrt(hd), window)
+    o = attention(q, k, v, positions, default_scale(hd), window)
     return linear(o.reshape(n, nh * hd), w[prefix + "o_proj.weight"])
 
 
@@ -204,9 +210,21 @@ def config_numbers(cfg: dict) -> dict:
         nkv=cfg.get("num_key_value_heads") or nh,
         hd=cfg.get("head_dim") or cfg["hidden_size"] // nh,
         I=cfg["intermediate_size"], V=cfg["vocab_size"], eps=cfg["rms_norm_eps"],
-        theta=cfg.get("rope_theta", 10000.0), window=cfg.get("sliding_window") or 0,
+        theta=(cfg.get("rope_parameters") or {}).get("rope_theta") or cfg.get("rope_theta", 10000.0),
+        window=cfg.get("sliding_window") or 0,
         tied=bool(cfg.get("tie_word_embeddings", False)),
+        layer_types=cfg.get("layer_types"),
     )
+
+
+def layer_window(c: dict, layer: int) -> int:
+    """The window of one layer: ``sliding_window`` everywhere, unless ``layer_types`` names the layer
+    "full_attention" (a per-layer switch as in crates/models/gemma4-v2/src/config.rs:124-138, where a
+    per-layer pattern says which layers have the window)."""
+    lt = c["layer_types"]
+    if lt is None or lt[layer] == "sliding_attention":
+        return c["window"]
+    return 0
 
 
 def forward(cfg: dict, w: dict, tokens, positions=None, keep_layers=None) -> np.ndarray:
@@ -227,7 +245,7 @@ def forward(cfg: dict, w: dict, tokens, positions=None, keep_layers=None) -> np.
         p = f"model.layers.{l}."
         a = rmsnorm(x, w[p + "input_layernorm.weight"], c["eps"])
         x = x + attention_mixer(a, w, p + "self_attn.", positions, c["nh"], c["nkv"], c["hd"],
-                                c["theta"], c["window"])
+                                c["theta"], layer_window(c, l))
         b = rmsnorm(x, w[p + "post_attention_layernorm.weight"], c["eps"])
         x = x + swiglu_mlp(b, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                            w[p + "mlp.down_proj.weight"])

@@ -17,13 +17,18 @@ def test_every_number_comes_from_the_file():
         assert cfg.hidden_size == raw["hidden_size"] and cfg.num_hidden_layers == raw["num_hidden_layers"]
         assert cfg.num_key_value_heads == raw["num_key_value_heads"]
         assert cfg.head_dim == raw.get("head_dim", raw["hidden_size"] // raw["num_attention_heads"])
-        assert cfg.rms_norm_eps == raw["rms_norm_eps"] and cfg.rope_theta == raw["rope_theta"]
+        theta = raw["rope_theta"] if "rope_theta" in raw else raw["rope_parameters"]["rope_theta"]
+        assert cfg.rms_norm_eps == raw["rms_norm_eps"] and cfg.rope_theta == theta
         assert cfg.sliding_window == (raw["sliding_window"] or 0)
         assert cfg.vocab_size == raw["vocab_size"] and cfg.tie_word_embeddings == raw["tie_word_embeddings"]
         spec = arch.build_spec(cfg)
         assert len(spec.layers) == raw["num_hidden_layers"] and len(spec.run_order) == raw["num_hidden_layers"]
         mixer = spec.layers[0].block.params["mixer"].params
         assert mixer["head_dim"] == cfg.head_dim and mixer["window"] == cfg.sliding_window
+        types = raw.get("layer_types")
+        for l, layer in enumerate(spec.layers):
+            window = layer.block.params["mixer"].params["window"]
+            assert window == (cfg.sliding_window if types is None or types[l] == "sliding_attention" else 0)
         assert mixer["position"].params["theta"] == cfg.rope_theta
         assert spec.layers[0].block.params["norm"].params["eps"] == cfg.rms_norm_eps
 
@@ -68,6 +73,41 @@ def test_bad_values_are_refused():
         raw.update(patch)
         with pytest.raises(ConfigError, match=pattern):
             config_from_dict(raw)
+
+
+def test_keys_that_change_the_arithmetic_are_read_or_refused():
+    base = TINY["A"]["config"]
+    for patch, pattern in [
+        ({"rope_scaling": {"rope_type": "linear", "factor": 2.0}}, "rotation scaling of type 'linear'"),
+        ({"rope_scaling": {"type": "yarn", "factor": 4.0}}, "yarn"),
+        ({"rope_parameters": {"rope_type": "llama3", "rope_theta": 1e4}}, "llama3"),
+        ({"rope_scaling": {"rope_type": "default", "factor": 8.0}}, "factor"),
+        ({"rope_scaling": "linear"}, "must be an object"),
+        ({"rope_parameters": {"rope_type": "default", "rope_theta": 5e5}}, "differ"),      # base says 1e4
+        ({"attention_bias": True}, "attention_bias"),
+        ({"mlp_bias": True}, "mlp_bias"),
+        ({"mlp_bias": "yes"}, "true or false"),
+        ({"layer_types": ["sliding_attention"]}, "layer_types"),
+        ({"layer_types": ["sliding_attention", "chunked"]}, "layer_types"),
+        ({"sliding_window": None, "layer_types": ["sliding_attention", "full_attention"]}, "sliding_window"),
+        ({"eos_token_id": [2, "x"]}, "eos_token_id"),
+    ]:
+        raw = dict(base)
+        raw.update(patch)
+        with pytest.raises(ConfigError, match=pattern):
+            config_from_dict(raw)
+    # the harmless forms are read
+    raw = dict(base, rope_scaling=None, attention_bias=False, mlp_bias=False, eos_token_id=[2, 9, 5])
+    del raw["rope_theta"]
+    raw["rope_parameters"] = {"rope_type": "default", "rope_theta": 7.5e5}
+    _, cfg = config_from_dict(raw)
+    assert cfg.rope_theta == 7.5e5 and cfg.eos_token_ids == (2, 9, 5) and cfg.eos_token_id == 2
+    arch, _ = config_from_dict(raw)
+    assert arch.build_spec(cfg).eos_token_ids == (2, 9, 5)
+    _, cfg = config_from_dict(dict(base, eos_token_id=3))
+    assert cfg.eos_token_ids == (3,)
+    _, cfg = config_from_dict(TINY["D"]["config"])
+    assert [cfg.window_of_layer(l) for l in range(4)] == [20, 0, 0, 20]
 
 
 def test_unknown_architecture_lists_the_known_ones():

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 STORE = {"float32": "float32", "bfloat16": "bfloat16"}
 STORE_DTYPE = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-LENGTHS = {"A": [5, 12, 23, 40, 70, 97], "B": [1, 31, 97, 64, 129], "C": [3, 50, 33, 150, 81]}
+LENGTHS = {"A": [5, 12, 23, 40, 70, 97], "B": [1, 31, 97, 64, 129], "C": [3, 50, 33, 150, 81], "D": [4, 45, 100, 29, 160]}
 
 
 def make_runner(model_dir, dtype, name, n_tokens, max_slots=8, page_size=None, tuned=True):
@@ -43,7 +43,7 @@ def runners(model_dirs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_cutting(model_dirs, runners, name, dtype, mode):
     d = model_dirs[(name, STORE[dtype])]
@@ -199,7 +199,7 @@ def test_step_refuses_bad_batches(model_dirs, runners):
 
 
 # ---------------------------------------------------------------- generation through the entry point
-def _plain_generate(d, prompt, n_new, temperature=0.0, seed=0):
+def _plain_generate(d, prompt, n_new, temperature=0.0, seed=0, stop=(), **filters):
     cfg, w = pm.read_model_dir(d)
     rng = pm.Xoshiro(seed)
     toks, margins = list(prompt), []
@@ -207,7 +207,9 @@ def _plain_generate(d, prompt, n_new, temperature=0.0, seed=0):
         logits = pm.forward(cfg, w, toks)[-1].astype(np.float32)
         s = np.sort(logits)
         margins.append(float(s[-1] - s[-2]))
-        toks.append(pm.sample(logits, rng, temperature=temperature))
+        toks.append(pm.sample(logits, rng, temperature=temperature, **filters))
+        if toks[-1] in stop:
+            break
     return toks[len(prompt):], margins
 
 
@@ -246,8 +248,69 @@ def test_temperature_generation_through_the_entry_point(model_dirs):
         assert out == want
     # the host sampler (filters) takes the same path through the scheduler
     outs2 = eng.generate(prompts[:2], [SamplingParams(temperature=0.8, top_k=384, seed=s, max_tokens=8) for s in seeds[:2]])
-    assert all(len(o) == 8 for o in outs2)
+    for prompt, out, s in zip(prompts, outs2, seeds):
+        assert out == _plain_generate(d, prompt, 8, temperature=0.8, seed=s, top_k=384)[0]
     assert not eng.runner.manager.live and eng.runner.manager.free_pages() == [24]
+
+
+def test_a_request_s_tokens_do_not_depend_on_what_its_neighbours_ask_for(model_dirs):
+    """A seeded temperature request beside a neighbour with a filter (whose logits go to the host
+    sampler) draws the tokens it draws alone, and the plain sampler's."""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    d = model_dirs[("B", "float32")]
+    prompts = list(rh.make_requests(384, [9, 14, 20], seed=23).values())
+    eng = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", page_size=16, inflight_slots=3, prefill_chunk_tokens=32))
+    mine = SamplingParams(temperature=0.8, seed=500, max_tokens=20)
+    alone = eng.generate(prompts[:1], mine)[0]
+    assert alone == _plain_generate(d, prompts[0], 20, temperature=0.8, seed=500)[0]
+    beside = eng.generate(prompts, [mine, SamplingParams(temperature=0.9, top_k=7, seed=501, max_tokens=20),
+                                    SamplingParams(temperature=0.0, repetition_penalty=1.3, max_tokens=12)])
+    assert beside[0] == alone
+    assert beside[1] == _plain_generate(d, prompts[1], 20, temperature=0.9, seed=501, top_k=7)[0]
+    # and with the device sampler switched off everything goes through the host sampler
+    host = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", page_size=16, inflight_slots=3, prefill_chunk_tokens=32,
+                                                    gpu_sampler=False))
+    greedy = SamplingParams(max_tokens=10)
+    assert host.generate(prompts[:2], greedy) == eng.generate(prompts[:2], greedy)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_stop_tokens_end_requests_while_the_next_step_is_in_flight(model_dirs, dtype):
+    """The engine runs one step ahead of the host: when a stop id (or one of several end-of-sequence
+    ids) arrives, the step after it is already enqueued.  Its token is dropped, the pages come back,
+    and the other requests' tokens are what they are alone.  Pages are so few that requests are
+    pre-empted on the way."""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    d = model_dirs[("D", STORE[dtype])]          # config.json names the end-of-sequence ids 7 and 11
+    prompts = list(rh.make_requests(210, [6, 17, 30, 11], seed=41).values())
+    n_new = 24
+    free = [_plain_generate(d, p, n_new)[0] for p in prompts]
+    # stop ids: a token the first request emits in the middle, one the third emits early
+    stops = (free[0][9], free[2][3])
+    want = []
+    for out in free:
+        cut = next((i for i, t in enumerate(out) if t in stops or t in (7, 11)), len(out) - 1)
+        want.append(out[:cut + 1])
+    assert any(len(w) < n_new for w in want)
+    eng = LLMEngine.from_dir(str(d), EngineOptions(dtype=dtype, page_size=8, inflight_slots=3, prefill_chunk_tokens=16,
+                                                   paged_kv=7))
+    got = eng.generate(prompts, SamplingParams(max_tokens=n_new, stop_token_ids=stops))
+    if dtype == "float32":
+        assert got == want
+    else:
+        # rounding may move a near-tie, so the tokens are not compared; every output still ends at its
+        # first stop or end-of-sequence id, or at the length
+        for g in got:
+            assert len(g) == n_new or g[-1] in stops or g[-1] in (7, 11)
+            assert not any(t in stops or t in (7, 11) for t in g[:-1])
+    assert not eng.runner.manager.live and eng.runner.manager.free_pages() == [7, 7]
+    eng.runner.manager.check_invariants()
+    if dtype == "float32":
+        assert eng.scheduler.n_preemptions > 0
+        # ignore_eos lets a request run past an end-of-sequence id, not past a stop id
+        again = eng.generate(prompts[:1], SamplingParams(max_tokens=n_new, ignore_eos=True, stop_token_ids=stops))
+        cut = min(i for i, t in enumerate(free[0]) if t in stops)
+        assert again[0] == free[0][:cut + 1]
 
 
 def test_generation_survives_preemption(model_dirs):

@@ -98,7 +98,46 @@ def test_rope_preserves_norms_and_depends_on_distance_only():
     assert abs(other - dots[0]) > 1e-6
 
 
+def test_rope_frequency_ladder_by_hand():
+    """theta = 10^4 and 8 rotated dims give the frequencies 1, 1/10, 1/100, 1/1000 (theta^(-2i/rot):
+    the exponent steps by 2/rot, starts at 0 and stops one step short of 1), so position 1000 turns
+    pair 3 by exactly one radian and position 10 turns pair 1 by one radian.  An exponent i/rot, or
+    2(i+1)/rot, or one taken over the head size instead of the rotated dims, fails."""
+    hd, rot = 12, 8
+    for pair, pos in ((0, 1), (1, 10), (2, 100), (3, 1000)):
+        x = np.zeros((1, 1, hd))
+        x[0, 0, pair] = 1.0
+        y = pm.rope_neox(x, [pos], 1e4, rotated_dims=rot)[0, 0]
+        np.testing.assert_allclose([y[pair], y[pair + rot // 2]], [math.cos(1.0), math.sin(1.0)], atol=1e-9)
+    # measured from the function itself: the angle a pair turns by at position 1 is its frequency
+    theta, rot = 5e5, 24
+    freqs = []
+    for pair in range(rot // 2):
+        x = np.zeros((1, 1, rot))
+        x[0, 0, pair] = 1.0
+        y = pm.rope_neox(x, [1], theta)[0, 0]
+        freqs.append(math.atan2(y[pair + rot // 2], y[pair]))
+    assert freqs[0] == 1.0
+    ratios = np.array(freqs[1:]) / np.array(freqs[:-1])
+    np.testing.assert_allclose(ratios, ratios[0], rtol=1e-9)                      # a geometric ladder
+    np.testing.assert_allclose(freqs[-1] * ratios[0], 1.0 / theta, rtol=1e-9)    # whose next rung would be 1 / theta
+
+
 # ---------------------------------------------------------------- attention
+def test_default_scale_is_the_library_routine_s():
+    """Without rotation, window or grouping, attention with the default scale is torch's
+    scaled_dot_product_attention with ITS default scale (1 / sqrt(head size)) and a causal mask."""
+    import torch
+    rng = np.random.default_rng(12)
+    n, nh, hd = 11, 3, 20
+    q, k, v = (rng.normal(size=(n, nh, hd)) for _ in range(3))
+    got = pm.attention(q, k, v, np.arange(n), pm.default_scale(hd), 0)
+    tq, tk, tv = (torch.from_numpy(a).permute(1, 0, 2)[None] for a in (q, k, v))     # [1, heads, n, hd]
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, is_causal=True)[0].permute(1, 0, 2).numpy()
+    np.testing.assert_allclose(got, want, atol=1e-12)
+    assert abs(pm.default_scale(64) - 0.125) < 1e-15
+
+
 def _library_attention(q, k, v, scale, mask):
     """softmax(Q K^T scale + mask) V with heads already matched."""
     s = np.einsum("ihd,jhd->hij", q, k) * scale + mask[None]
@@ -227,6 +266,22 @@ def test_forward_is_causal_and_shift_invariant():
     full = pm.forward(cfg, w, toks)
     np.testing.assert_allclose(pm.forward(cfg, w, toks[:7]), full[:7], atol=1e-10)
     np.testing.assert_allclose(pm.forward(cfg, w, toks, positions=np.arange(12) + 37), full, atol=1e-9)
+
+
+def test_forward_layer_types_switch_the_window_per_layer():
+    """``layer_types`` names the layers that have the window; all "sliding_attention" is the window
+    everywhere, all "full_attention" is no window, and a mixture differs from both."""
+    rng = np.random.default_rng(8)
+    cfg, w = _random_model(rng, L=3, window=4)
+    toks = list(rng.integers(0, 30, size=14))
+    base = pm.forward(cfg, w, toks)
+    np.testing.assert_array_equal(pm.forward(dict(cfg, layer_types=["sliding_attention"] * 3), w, toks), base)
+    free = pm.forward(dict(cfg, sliding_window=None), w, toks)
+    np.testing.assert_array_equal(pm.forward(dict(cfg, layer_types=["full_attention"] * 3), w, toks), free)
+    mixed = pm.forward(dict(cfg, layer_types=["full_attention", "sliding_attention", "full_attention"]), w, toks)
+    assert np.abs(mixed - base).max() > 1e-6 and np.abs(mixed - free).max() > 1e-6
+    # only the second layer has the window: the same as a model whose other layers see everything
+    np.testing.assert_array_equal(mixed[:4], free[:4])            # (no difference before the window bites)
 
 
 def test_forward_tied_head_uses_the_embedding_table():

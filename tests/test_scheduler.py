@@ -244,3 +244,32 @@ def test_commit_in_two_halves_with_a_step_enqueued_in_between():
     assert s.resolve(s4, {"a": 14}) == [a] and a.output == [11, 12, 13, 14] and a.finish_reason == "length"
     m.check_invariants()
     assert m.free_pages() == [16]
+
+
+def test_any_of_several_end_of_sequence_ids_ends_a_request():
+    m, s = mk(eos_token_id=(7, 11))
+    a = s.add("a", [1, 2, 3], SamplingParams(max_tokens=10))
+    b = s.add("b", [1, 2, 3], SamplingParams(max_tokens=10))
+    c = s.add("c", [1, 2, 3], SamplingParams(max_tokens=4, ignore_eos=True))
+    emits = {"a": [5, 11, 6], "b": [7], "c": [7, 11, 7, 11]}
+    while s.has_work():
+        run_step(m, s, token=lambda r: emits[r.request_id][len(r.output)])
+    assert a.output == [5, 11] and a.finish_reason == "stop"
+    assert b.output == [7] and b.finish_reason == "stop"
+    assert c.output == [7, 11, 7, 11] and c.finish_reason == "length"
+    assert m.free_pages() == [16] and m.n_free_slots == 3
+    # one id, as before
+    m, s = mk(eos_token_id=9)
+    r = s.add("r", [1], SamplingParams(max_tokens=5))
+    while s.has_work():
+        run_step(m, s, token=lambda r: 9)
+    assert r.output == [9]
+
+
+def test_token_access_without_joining_prompt_and_output():
+    from flambeau_amd.engine.scheduler import Request
+    r = Request("x", [10, 11, 12], SamplingParams(), output=[20, 21])
+    assert [r.token_at(i) for i in range(5)] == r.tokens
+    for a in range(6):
+        for b in range(a, 6):
+            assert r.token_slice(a, b) == r.tokens[a:b]

@@ -73,6 +73,7 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     del t["model.layers.1.mlp.up_proj.weight"]
     del t["model.norm.weight"]
     t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    t["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(64)
     t["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(16, 64)       # should be [32, 64]
     t["lm_head.weight"] = torch.zeros(64, 256)                              # transposed
     write_safetensors(d / "model.safetensors", t)
@@ -81,10 +82,14 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         check_against_manifest(_manifest("A"), src)
     e = ei.value
     assert e.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
-    assert e.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert e.unexpected == ["model.layers.0.self_attn.q_proj.bias", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    # tensors the architecture says a file may hold without the model reading them are no error
+    with pytest.warns(UserWarning, match="rotary_emb.inv_freq"), pytest.raises(WeightError) as ei:
+        check_against_manifest(_manifest("A"), src, ignored=("*.rotary_emb.inv_freq",))
+    assert ei.value.unexpected == ["model.layers.0.self_attn.q_proj.bias"]
     assert sorted(n for n, _, _ in e.wrong_shape) == ["lm_head.weight", "model.layers.0.self_attn.k_proj.weight"]
     msg = str(e)
-    for piece in ("missing (2)", "unexpected (1)", "model.norm.weight", "rotary_emb.inv_freq",
+    for piece in ("missing (2)", "unexpected (2)", "model.norm.weight", "rotary_emb.inv_freq",
                   "lm_head.weight is [64, 256], expected [256, 64]"):
         assert piece in msg
 

@@ -1,7 +1,9 @@
 """Tiny configurations of the architecture for the tests.  They differ in every size and
 option: layers, width, head counts and groups (GQA, MQA, MHA), head size (derived, explicit
 and not width/heads), intermediate size, vocabulary (none a power of two but A's), theta,
-window (16, none, 24 = no multiple of a page), eps, tied or untied head, weight scale."""
+window (16, none, 24 = no multiple of a page; D: a window in two of its four layers only, so its
+cache has two groups of layers with pages of their own), eps, tied or untied head, weight scale,
+one or several end-of-sequence ids."""
 import torch
 
 from flambeau_amd.weights import write_random_model
@@ -31,6 +33,13 @@ TINY = {
                     sliding_window=24, rms_norm_eps=1e-4, max_position_embeddings=640,
                     tie_word_embeddings=True),
         seed=5, std=0.04, gain_std=0.02, page_size=16),
+    "D": dict(
+        config=_cfg(num_hidden_layers=4, hidden_size=48, num_attention_heads=3, num_key_value_heads=1,
+                    head_dim=16, intermediate_size=72, vocab_size=210, rope_parameters={"rope_type": "default", "rope_theta": 2.5e4},
+                    sliding_window=20, layer_types=["sliding_attention", "full_attention", "full_attention", "sliding_attention"],
+                    rms_norm_eps=3e-6, max_position_embeddings=512, tie_word_embeddings=False,
+                    eos_token_id=[7, 11]),
+        seed=9, std=0.06, gain_std=0.03, page_size=8),
 }
 
 STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}
