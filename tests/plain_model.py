@@ -137,7 +137,7 @@ def attention(q, k, v, positions, scale, window=0):
     q[n, nh, hd], k/v[n, nkv, hd]; token j sits at absolute position positions[j].
     kv_head = q_head // (nh // nkv); query at p sees keys t in
     [max(0, p-W+1), p] (W = 0: [0, p]); s_t = (q.k_t)*scale, scale applied after
-    the dot; o = sum softmax(s)_t v_t.  Masked keys are never scored.
+    the dot; o = sum softmax(s)_t v_t over the visible keys only.
     crates/kernels-hip/src/kernels/attention_prefill_f16.cu:50-51 (head map),
     :58-71 (limit and window start), :89-133 (scores, softmax, PV);
     window counts keys including the query's own: crates/ops/tests/swa_softcap_parity.rs:243;
@@ -150,18 +150,18 @@ def attention(q, k, v, positions, scale, window=0):
     n, nh, hd = q.shape
     nkv = k.shape[1]
     group = nh // nkv
+    # visible[i, t]: key t lies in [max(0, p_i - W + 1), p_i]
+    lo = np.maximum(0, positions - window + 1) if window > 0 else np.zeros_like(positions)
+    visible = (positions[None, :] >= lo[:, None]) & (positions[None, :] <= positions[:, None])
     out = np.zeros((n, nh, v.shape[2]), dtype=F64)
-    for i in range(n):
-        p = positions[i]
-        lo = max(0, p - window + 1) if window > 0 else 0
-        vis = np.nonzero((positions >= lo) & (positions <= p))[0]
-        for h in range(nh):
-            g = h // group
-            s = (k[vis, g, :] @ q[i, h, :]) * scale
-            s = s - s.max()
-            w = np.exp(s)
-            w = w / w.sum()
-            out[i, h, :] = w @ v[vis, g, :]
+    for h in range(nh):
+        g = h // group
+        s = (q[:, h, :] @ k[:, g, :].T) * scale
+        s = np.where(visible, s, -np.inf)              # keys outside the range take no part
+        s = s - s.max(axis=1, keepdims=True)
+        w = np.exp(s)
+        w = w / w.sum(axis=1, keepdims=True)
+        out[:, h, :] = w @ v[:, g, :]
     return out
 
 
@@ -227,8 +227,8 @@ def layer_window(c: dict, layer: int) -> int:
     return 0
 
 
-def forward(cfg: dict, w: dict, tokens, positions=None, keep_layers=None) -> np.ndarray:
-    """Logits [n, vocab] of one whole sequence.
+def forward(cfg: dict, w: dict, tokens, positions=None, keep_layers=None, rows=None) -> np.ndarray:
+    """Logits [n, vocab] of one whole sequence (``rows``: only at these places, [len(rows), vocab]).
 
     for l: x += Attn(Norm1(x)); x += MLP(Norm2(x)); logits = Head(NormF(x)).
     crates/forward/README.md:28-40; crates/models/qwen35-v2/src/model.rs:19-50;
@@ -249,6 +249,8 @@ def forward(cfg: dict, w: dict, tokens, positions=None, keep_layers=None) -> np.
         b = rmsnorm(x, w[p + "post_attention_layernorm.weight"], c["eps"])
         x = x + swiglu_mlp(b, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                            w[p + "mlp.down_proj.weight"])
+    if rows is not None:
+        x = x[np.asarray(rows, dtype=np.int64)]
     f = rmsnorm(x, w["model.norm.weight"], c["eps"])
     head = w["model.embed_tokens.weight"] if c["tied"] else w["lm_head.weight"]
     return linear(f, head)
