@@ -28,6 +28,7 @@ class EngineOptions:
     inflight_slots: int = 4
     prefill_chunk_tokens: int = 512
     max_batch_tokens: int | None = None     # tokens per step; default prefill_chunk_tokens + inflight_slots
+    row_granule: int | None = None          # steps of many rows hold a multiple of this many; default: the kernels' row tile
     paged_kv: int | None = None             # pages; default: enough for inflight_slots * ctx
     page_size: int = 16
     max_queue_depth: int = 0
@@ -52,7 +53,8 @@ class LLMEngine:
                                    prefill_chunk_tokens=opt.prefill_chunk_tokens,
                                    max_queue_depth=opt.max_queue_depth,
                                    eos_token_id=getattr(spec, "eos_token_ids", ()) or spec.eos_token_id,
-                                   default_seed=opt.seed)
+                                   default_seed=opt.seed,
+                                   row_granule=opt.row_granule or model.rt.row_granule)
         self.sampler = DeviceSampler(model.rt.device, max(opt.inflight_slots, 1))
         # tokens drawn on the device are fed to the next step on the device: the host enqueues
         # step i + 1 while step i runs and reads step i's tokens afterwards

@@ -29,6 +29,9 @@ class Runtime:
         # tuned kernels exist for bfloat16 only; the 32-bit path always runs the plain ones
         self.tuned = bool(tuned) and dtype == torch.bfloat16
         self.max_batch_tokens = int(max_batch_tokens)
+        # rows per tile of the matrix kernels that take prompt portions (a scheduler that knows it
+        # can fill whole tiles); the plain kernels have none
+        self.row_granule = 128 if self.tuned else 1
         self._buffers: dict = {}
         self._views: dict = {}
         self._scope = ""

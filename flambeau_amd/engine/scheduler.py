@@ -8,7 +8,9 @@ runs them, ``commit()`` takes the sampled tokens.  Rules:
   that one token (a decode row).  Decode rows are scheduled before prompt tokens.
 * What is left of ``max_batch_tokens`` is dealt to requests that still have prompt (or, after
   a pre-emption, earlier output) to run, in order of arrival, each getting at most
-  ``prefill_chunk_tokens`` per step; several portions may share a step.
+  ``prefill_chunk_tokens`` per step; several portions may share a step.  With a ``row_granule``
+  the portions' share is rounded down so that the step's rows are a multiple of it (the matrix
+  kernels work on tiles of rows; 8 decode rows beside a portion of 504 cost less than beside 512).
 * A waiting request is admitted when a slot is free and the free pages cover its first portion.
   Order of arrival is kept: nobody overtakes the head of the queue.
 * Pages are asked for before the batch is built, so the step itself never runs out.  If a decode
@@ -88,12 +90,16 @@ class Scheduled:
 
 class Scheduler:
     def __init__(self, manager: CacheManager, *, max_batch_tokens: int, prefill_chunk_tokens: int = 512,
-                 max_queue_depth: int = 0, eos_token_id=None, default_seed: int = 0):
+                 max_queue_depth: int = 0, eos_token_id=None, default_seed: int = 0, row_granule: int = 1):
         if max_batch_tokens < 1 or prefill_chunk_tokens < 1:
             raise ValueError("token budgets must be positive")
         self.manager = manager
         self.max_batch_tokens = max_batch_tokens
         self.prefill_chunk_tokens = prefill_chunk_tokens
+        # The kernels work on tiles of this many rows: a step of 520 rows costs what 640 cost.  Where a
+        # step holds more rows than one tile, the prompt portions are cut so that decode rows and
+        # portions together fill whole tiles.
+        self.row_granule = max(1, int(row_granule))
         self.max_queue_depth = max_queue_depth      # 0: no limit (routes.rs:481 "0 disables")
         # one id or several: any of them ends a request
         if eos_token_id is None:
@@ -216,7 +222,14 @@ class Scheduler:
             self._preempt(victim)
             # r itself may have been the victim; the loop looks at r again otherwise
 
-        # 2. portions of running requests, in order of admission
+        # 2. portions of running requests, in order of admission; their budget is rounded down so that
+        # the step's rows fill whole tiles (never below half the budget)
+        g = self.row_granule
+        if g > 1 and budget > 0:
+            used = self.max_batch_tokens - budget
+            whole = (used + budget) // g * g - used
+            if whole >= max(1, budget // 2):
+                budget = whole
         for r in list(self.running):
             if budget <= 0:
                 break

@@ -273,3 +273,23 @@ def test_token_access_without_joining_prompt_and_output():
     for a in range(6):
         for b in range(a, 6):
             assert r.token_slice(a, b) == r.tokens[a:b]
+
+
+def test_portions_are_cut_so_that_a_step_fills_whole_row_tiles():
+    """Budget 520 (a portion of 512 beside 8 decoding requests), tiles of 128 rows: with 3 decode
+    rows the portion is 509, so the step holds 512 rows; without a granule it is 512 + 3."""
+    for granule, want in ((128, 509), (1, 512)):
+        m = CacheManager([GroupSpec(1, 8, 0)], 400, 16, 9, 4096)
+        s = Scheduler(m, max_batch_tokens=520, prefill_chunk_tokens=512, row_granule=granule)
+        for rid in "abc":
+            s.add(rid, [1, 2, 3], SamplingParams(max_tokens=50))
+        run_step(m, s)
+        s.add("long", list(range(2000)), SamplingParams(max_tokens=2))
+        sched, _ = run_step(m, s)
+        assert [(e.request.request_id, len(e.tokens)) for e in sched] == [("a", 1), ("b", 1), ("c", 1), ("long", want)]
+    # a budget that holds less than a tile's worth of portions is left alone, and so is a short prompt
+    m = CacheManager([GroupSpec(1, 8, 0)], 400, 16, 9, 4096)
+    s = Scheduler(m, max_batch_tokens=100, prefill_chunk_tokens=64, row_granule=128)
+    s.add("x", list(range(90)), SamplingParams(max_tokens=2))
+    sched, _ = run_step(m, s)
+    assert [len(e.tokens) for e in sched] == [64]
