@@ -144,7 +144,9 @@ def run_prefill(model, dtype_name, reps=REPS, seed=1):
 def run_enqueue(model, dtype_name, rows=64, decoders=16, seed=2):
     """Host time to enqueue one mixed step of ``rows`` rows (a prompt portion beside ``decoders``
     decoding requests): the time ``ModelRunner.step`` takes to return, the device idle before and
-    not waited for after.  Median of 20 steps, in milliseconds."""
+    not waited for after.  Median of the last 30 of 80 steps, in milliseconds (the engine records a
+    step's launches and replays them from native code when its shape comes again; shapes that keep
+    coming back become graphs)."""
     import numpy as np
     import torch
     from flambeau_amd.engine import ModelRunner, StepEntry
@@ -158,7 +160,7 @@ def run_enqueue(model, dtype_name, rows=64, decoders=16, seed=2):
     runner.begin("p")
     runner.step([StepEntry(i, ids(60 + 5 * i), []) for i in range(decoders)])
     times = []
-    for k in range(24):
+    for k in range(80):
         entries = [StepEntry(i, ids(1), [0]) for i in range(decoders)] + [StepEntry("p", ids(rows - decoders), [rows - decoders - 1])]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -167,7 +169,7 @@ def run_enqueue(model, dtype_name, rows=64, decoders=16, seed=2):
         torch.cuda.synchronize()
     del runner
     torch.cuda.empty_cache()
-    return statistics.median(times[4:]) * 1e3
+    return statistics.median(times[-30:]) * 1e3
 
 
 def run_serving(model, cfg, dtype_name, prompts, n_new, slots, chunk, ctx):

@@ -122,6 +122,16 @@ int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int max_keys);
 int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 
+// ---- step programs (program.hip): launches recorded once, replayed with one call ----
+typedef union FlArg { void* p; long l; int i; float f; } FlArg;
+void* fl_program_new(void);
+void fl_program_free(void* program);
+int fl_program_size(const void* program);
+// name: one of the launch functions above (those that take a stream); args: its arguments in order,
+// the stream's value is ignored
+int fl_program_append(void* program, const char* name, const FlArg* args, int n_args);
+int fl_program_run(const void* program, hipStream_t stream, int* failed_at);
+
 #ifdef __cplusplus
 }
 #endif

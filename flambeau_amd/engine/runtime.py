@@ -35,6 +35,7 @@ class Runtime:
         self._buffers: dict = {}
         self._views: dict = {}
         self._scope = ""
+        self.generation = 0          # counts allocations of buffers: recorded launches name buffers by address
 
     # ------------------------------------------------------------ buffers
     def buffer(self, name: str, rows: int, cols: int, dtype=None, max_rows: int | None = None):
@@ -53,6 +54,7 @@ class Runtime:
             size = min(cap, max(16, 1 << max(rows - 1, 0).bit_length()))
             buf = torch.empty((size, cols), dtype=dtype, device=self.device)
             self._buffers[key] = buf
+            self.generation += 1
             for k in [k for k in self._views if k[0] == key]:
                 del self._views[k]
         view = self._views[(key, rows)] = buf[:rows]

@@ -14,6 +14,7 @@ block-table entries layer by layer (crates/forward/src/core/composites/standard_
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass, field
 
 import numpy as np
@@ -22,6 +23,7 @@ import torch
 from ..cache.manager import CacheError, CacheManager
 from ..cache.storage import CacheStorage
 from ..kernels import ops
+from ..kernels.library import Program
 from ..parts.base import HostBatch, StepState
 
 
@@ -42,7 +44,8 @@ class ModelRunner:
     """Owns the model, the cache and the step function."""
 
     def __init__(self, model, *, n_pages: int, page_size: int, max_slots: int, max_seq_len: int | None = None,
-                 max_logit_rows: int | None = None, decode_graphs: bool = True, max_graph_batch: int = 256):
+                 max_logit_rows: int | None = None, decode_graphs: bool = True, max_graph_batch: int = 256,
+                 step_programs: bool = True, max_programs: int = 96):
         self.model = model
         self.rt = model.rt
         spec = model.spec
@@ -65,6 +68,15 @@ class ModelRunner:
         # ``from_device`` read their token from it, so a step can be enqueued before the host has
         # seen the step before
         self.token_feedback = None
+        # Steps that no graph takes (anything with a prompt portion) are recorded while they run and
+        # replayed from native code when a step of the same shape and the same kernel choices comes
+        # again: ``{key: _RecordedStep}``, least recently used first.
+        self.step_programs = bool(step_programs) and model.replayable()
+        self.max_programs = max_programs
+        self.graph_after_hits = 3           # replays after which a recorded step is turned into a graph
+        self._programs: OrderedDict = OrderedDict()
+        self.n_replayed = 0
+        self.n_recorded = 0
 
     # ------------------------------------------------------------ requests
     def begin(self, request_id) -> bool:
@@ -165,8 +177,10 @@ class ModelRunner:
         if pad_to is not None:
             width = mgr.max_blocks
         else:
+            # the tables' width is a power of two: it is part of a step's shape (recorded steps are
+            # keyed by it) and should not change with every page a request gains
             need_blocks = max((-(-(st + q) // mgr.page_size) for st, q in zip(starts, q_lens)), default=1)
-            width = max(8, -(-need_blocks // 8) * 8)
+            width = max(8, 1 << (need_blocks - 1).bit_length())
         tables = []
         for g in range(len(mgr.groups)):
             t = np.full((S + n_pad, width), -1, dtype=np.int32)
@@ -257,11 +271,55 @@ class ModelRunner:
         else:
             batch, parts = self._assemble(entries)
             dev = self._upload(parts)
-            self._feed(dev, any(e.from_device is not None for e in entries))
-            step = self._state_from(batch, parts, dev)
-            logits = self.model.forward(step, self.storage.entries, self.max_logit_rows)
+            feed = any(e.from_device is not None for e in entries)
+            if self.step_programs:
+                logits = self._step_recorded(batch, parts, dev, feed)
+            else:
+                self._feed(dev, feed)
+                logits = self.model.forward(self._state_from(batch, parts, dev), self.storage.entries, self.max_logit_rows)
         for e in entries:
             self.manager.advance(e.request_id, len(e.tokens))
+        return logits
+
+    # ------------------------------------------------------------ recorded steps
+    def _program_key(self, batch, parts, feed: bool):
+        """Everything that decides which kernels a step launches and with which arguments: rows per
+        request, number and pattern of the wanted rows, shapes of all metadata (they fix where each
+        array lies on the device), whether tokens come from the device, and what the mixers decide
+        from the contexts' lengths."""
+        return (tuple(batch.q_lens), batch.n_logit_rows, batch.every_row, feed,
+                tuple(arr.shape for _, arr in parts), self.model.step_signature(batch))
+
+    def _step_recorded(self, batch, parts, dev, feed: bool):
+        key = self._program_key(batch, parts, feed)
+        hit = self._programs.get(key)
+        valid = (self.rt.generation, self._meta_dev.data_ptr())
+        if hit is not None and hit.valid == valid:
+            self._programs.move_to_end(key)
+            hit.hits += 1
+            if hit.graph is None and hit.hits >= self.graph_after_hits:
+                # a shape that keeps coming back: its launches become a graph (they are this
+                # library's kernels only, with fixed arguments), which costs one launch to replay
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    hit.program.run(torch.cuda.current_stream().cuda_stream)
+                hit.graph = graph
+            if hit.graph is not None:
+                hit.graph.replay()
+            else:
+                hit.program.run(torch.cuda.current_stream().cuda_stream)
+            self.n_replayed += 1
+            return hit.logits
+        program = Program()
+        with program.recording():
+            self._feed(dev, feed)
+            logits = self.model.forward(self._state_from(batch, parts, dev), self.storage.entries, self.max_logit_rows)
+        # (a buffer that grew during this very step moved before it was used: the generation is read afterwards)
+        self._programs[key] = _RecordedStep(program, logits, (self.rt.generation, self._meta_dev.data_ptr()))
+        self._programs.move_to_end(key)
+        while len(self._programs) > self.max_programs:
+            self._programs.popitem(last=False)
+        self.n_recorded += 1
         return logits
 
     # ------------------------------------------------------------ captured decode steps
@@ -305,6 +363,15 @@ class ModelRunner:
         if wanted == list(range(len(wanted))):
             return gs.logits[:len(wanted)]
         return gs.logits[torch.tensor(wanted, device=self.rt.device)]
+
+
+class _RecordedStep:
+    def __init__(self, program, logits, valid):
+        self.program = program
+        self.logits = logits
+        self.valid = valid          # (buffer generation, address of the metadata) the arguments belong to
+        self.hits = 0
+        self.graph = None
 
 
 class _GraphedStep:

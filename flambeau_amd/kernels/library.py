@@ -65,6 +65,7 @@ def register_signatures(extra: dict) -> None:
 
 
 _functions: dict = {}
+_recording = None        # the Program that launches are being appended to, or None
 
 
 def call(name: str, *args) -> None:
@@ -74,3 +75,81 @@ def call(name: str, *args) -> None:
     rc = fn(*args)
     if rc != 0:
         raise KernelError(f"{name}: {load().fl_last_error().decode(errors='replace')} (code {rc})")
+    if _recording is not None:
+        _recording.append(name, args)
+
+
+class FlArg(ctypes.Union):
+    _fields_ = [("p", c_void_p), ("l", c_long), ("i", c_int), ("f", c_float)]
+
+
+_FIELD = {P: "p", I: "i", F: "f", L: "l"}
+
+
+class Program:
+    """A list of launches recorded while they ran, replayed with one foreign call (csrc/program.hip).
+    ``with program.recording():`` appends every ``call`` made inside; ``run(stream)`` launches them
+    again with the arguments they had.  Whoever keeps a program answers for its arguments still
+    being valid: same buffers, same shapes."""
+
+    def __init__(self):
+        lib = load()
+        if not hasattr(lib, "_program_ready"):
+            lib.fl_program_new.restype = c_void_p
+            lib.fl_program_new.argtypes = []
+            lib.fl_program_free.restype = None
+            lib.fl_program_free.argtypes = [c_void_p]
+            lib.fl_program_size.restype = c_int
+            lib.fl_program_size.argtypes = [c_void_p]
+            lib.fl_program_append.restype = c_int
+            lib.fl_program_append.argtypes = [c_void_p, c_char_p, ctypes.POINTER(FlArg), c_int]
+            lib.fl_program_run.restype = c_int
+            lib.fl_program_run.argtypes = [c_void_p, c_void_p, ctypes.POINTER(c_int)]
+            lib._program_ready = True
+        self._lib = lib
+        self._handle = c_void_p(lib.fl_program_new())
+        self._failed = c_int(-1)
+        self._names: list = []
+
+    def __del__(self):
+        try:
+            if self._handle:
+                self._lib.fl_program_free(self._handle)
+                self._handle = None
+        except Exception:
+            pass
+
+    def __len__(self):
+        return len(self._names)
+
+    def append(self, name: str, args) -> None:
+        types = _SIGNATURES[name]
+        arr = (FlArg * len(types))()
+        for slot, t, v in zip(arr, types, args):
+            if v is not None:
+                setattr(slot, _FIELD[t], v)
+        if self._lib.fl_program_append(self._handle, name.encode(), arr, len(types)) != 0:
+            raise KernelError(f"recording {name}: {self._lib.fl_last_error().decode(errors='replace')}")
+        self._names.append(name)
+
+    def recording(self):
+        prog = self
+
+        class _Recording:
+            def __enter__(self_inner):
+                global _recording
+                if _recording is not None:
+                    raise KernelError("a program is already being recorded")
+                _recording = prog
+
+            def __exit__(self_inner, *exc):
+                global _recording
+                _recording = None
+        return _Recording()
+
+    def run(self, stream: int) -> None:
+        rc = self._lib.fl_program_run(self._handle, stream, ctypes.byref(self._failed))
+        if rc != 0:
+            at = self._failed.value
+            name = self._names[at] if 0 <= at < len(self._names) else "?"
+            raise KernelError(f"replay of {name} (call {at}): {self._lib.fl_last_error().decode(errors='replace')} (code {rc})")

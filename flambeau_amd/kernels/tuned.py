@@ -508,6 +508,24 @@ def prefill_supported(cache, table) -> bool:
     return decode_supported(cache) and ps >= 8 and ps & (ps - 1) == 0 and table.shape[1] <= PREFILL_MAX_PAGES
 
 
+def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int):
+    """``(parts of the keys for the tiled kernel, for the single-row kernel)`` for a batch: everything
+    that ``attention`` decides from the contexts' lengths (the rest follows from the batch's shape)."""
+    n_tiles = sum(-(-ql // PREFILL_TILE) for ql in batch.q_lens if ql > SHORT_PORTION)
+    n_items = sum(ql for ql in batch.q_lens if ql <= SHORT_PORTION)
+    p_split = n_split = 1
+    if n_tiles:
+        # few tiles before a long context: the keys are split too, so that the chip has blocks enough
+        longest = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + PREFILL_TILE)
+        p_split = attn_prefill_splits(n_tiles, n_heads, n_kv_heads, head_dim, longest)
+    if n_items:
+        max_ctx = batch.ctx_bound or batch.max_ctx_len
+        if window:
+            max_ctx = min(max_ctx, window + 32)
+        n_split = decode_splits(n_items, n_kv_heads, n_heads // n_kv_heads, max_ctx)
+    return p_split, n_split
+
+
 def attention(rt, q, out, cache, step, table, n_heads, scale, window):
     """Attention of one batch with the tuned kernels: rows of short portions through the split-K
     kernel, longer portions through the tiled kernel.  A cache shape one of them does not take
@@ -516,10 +534,12 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
     batch = step.host
     if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table)):
         return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
+    key = ("attention_splits", n_heads, cache.n_kv_heads, cache.head_dim, window)
+    splits = step.scratch.get(key)
+    if splits is None:
+        splits = step.scratch[key] = attention_splits(batch, n_heads, cache.n_kv_heads, cache.head_dim, window)
+    p_split, n_split = splits
     if tiles.shape[0]:
-        # few tiles before a long context: the keys are split too, so that the chip has blocks enough
-        longest = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + PREFILL_TILE)
-        p_split = attn_prefill_splits(tiles.shape[0], n_heads, cache.n_kv_heads, cache.head_dim, longest)
         p_o = p_ml = None
         if p_split > 1:
             n_rows = sum(ql for ql in batch.q_lens if ql > SHORT_PORTION)
@@ -528,11 +548,6 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
             p_ml = rt.buffer("attn_tile_part_ml", n_rows * n_heads * p_split, 2, torch.float32, max_rows=1 << 24)
         attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window, n_split=p_split, part_o=p_o, part_ml=p_ml)
     if rows.shape[0]:
-        group = n_heads // cache.n_kv_heads
-        max_ctx = batch.ctx_bound or batch.max_ctx_len
-        if window:
-            max_ctx = min(max_ctx, window + 32)
-        n_split = decode_splits(rows.shape[0], cache.n_kv_heads, group, max_ctx)
         part_o = part_ml = None
         if n_split > 1:
             hdp = -(-cache.head_dim // 32) * 32

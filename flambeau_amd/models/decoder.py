@@ -58,6 +58,7 @@ class DecoderModel:
         self.blocks = [BLOCKS.create(ls.block) for ls in spec.layers]
         self.final_norm = NORMS.create(spec.final_norm)
         self.head = OutputHead(spec.vocab_size, spec.hidden_size, tied=spec.tied_head)
+        self._signature_mixers = None
         for i, e in enumerate(spec.run_order):
             if not 0 <= e.layer < len(self.blocks):
                 raise ValueError(f"run-order entry {i} names layer {e.layer}, the model has {len(self.blocks)}")
@@ -104,6 +105,30 @@ class DecoderModel:
             specs.append(self.blocks[e.layer].cache_spec())
             shares.append(e.cache_of)
         return specs, shares
+
+    def all_parts(self) -> list:
+        """Every part of the model, the parts of parts included."""
+        out, todo = [], [self.embedding, self.final_norm, self.head, *self.blocks]
+        while todo:
+            p = todo.pop()
+            out.append(p)
+            todo += list(getattr(p, "subparts", lambda: [])())
+        return out
+
+    def replayable(self) -> bool:
+        """True if a step of this model can be recorded and replayed (``Part.replayable``)."""
+        return all(getattr(p, "replayable", False) for p in self.all_parts())
+
+    def step_signature(self, batch) -> tuple:
+        """What the mixers decide from the batch's numbers beyond its shape (``Mixer.step_signature``),
+        one entry per group of like mixers."""
+        if self._signature_mixers is None:
+            seen = {}
+            for b in self.blocks:
+                for m in getattr(b, "mixers", lambda: [])():
+                    seen.setdefault(m.signature_group(), m)
+            self._signature_mixers = list(seen.values())
+        return tuple(m.step_signature(batch) for m in self._signature_mixers)
 
     def mixer_classes(self):
         seen = []

@@ -24,6 +24,7 @@ from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, Prod
 class PagedGQAAttention(Mixer):
     graph_safe = True
     lazy_input = True
+    replayable = True
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, window: int = 0, scale: float | None = None):
@@ -39,6 +40,18 @@ class PagedGQAAttention(Mixer):
 
     def cache_spec(self):
         return PagedKVSpec(self.n_kv_heads, self.head_dim, self.window)
+
+    def subparts(self):
+        return [self.position]
+
+    def signature_group(self):
+        return ("paged_gqa_attention", self.n_heads, self.n_kv_heads, self.head_dim, self.window)
+
+    def step_signature(self, batch):
+        """Into how many parts the kernels split the keys: all that this mixer decides from the
+        contexts' lengths."""
+        from ..kernels import tuned
+        return tuned.attention_splits(batch, self.n_heads, self.n_kv_heads, self.head_dim, self.window)
 
     def tensors(self):
         H, qw, kvw = self.hidden_size, self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim

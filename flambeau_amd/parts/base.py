@@ -110,6 +110,18 @@ class Part:
     """Base of all parts.  Subclasses take their sizes and constants as keyword
     parameters, list their tensors, and receive them in ``bind``."""
 
+    # True if everything the part does on the device goes through the kernel library's launch
+    # functions, with arguments that are decided by the step's shape (rows per request, wanted rows,
+    # table widths, buffers) and, for a mixer, by what its ``step_signature`` returns.  A model
+    # of such parts can have its steps recorded and replayed from native code.  A part that calls
+    # torch operations, or looks at a step's values on the host, is not.
+    replayable = False
+
+    def subparts(self) -> list:
+        """The parts this part is made of (a block's mixer, norms and feed-forward; a mixer's
+        position encoding)."""
+        return []
+
     def tensors(self) -> dict:
         """``{local name: TensorSpec}``."""
         return {}
@@ -185,6 +197,17 @@ class Mixer(Part):
         """Integer arrays (numpy int32) this kind of mixer wants on the device for the batch,
         uploaded with the rest of the step's metadata and found in ``StepState.extra``."""
         return {}
+
+    def step_signature(self, batch: HostBatch):
+        """Whatever this mixer decides from the batch's numbers beyond its shape (how many ways it
+        splits the keys of a long context, ...), as a hashable value: two batches of the same shape
+        and the same signature must make the mixer launch the same kernels with the same arguments.
+        The default is exact and rarely repeats: where every request starts."""
+        return tuple(batch.start_pos)
+
+    def signature_group(self):
+        """Mixers with equal groups give equal signatures (one of them is asked per step)."""
+        return id(self)
 
     def forward(self, x, step: StepState, cache: LayerCache):
         """``x``: normed activations [n, hidden] in the compute dtype.  Returns the

@@ -55,6 +55,8 @@ class ResidualStream:
 
 @BLOCKS.register("prenorm")
 class PreNormBlock(Block):
+    replayable = True
+
     def __init__(self, mixer: PartSpec, feed_forward: PartSpec, norm: PartSpec):
         self.mixer_norm = NORMS.create(norm)
         self.mixer = MIXERS.create(mixer)
@@ -68,6 +70,9 @@ class PreNormBlock(Block):
 
     def mixers(self):
         return [self.mixer]
+
+    def subparts(self):
+        return list(self._parts.values())
 
     def tensors(self):
         return {f"{p}.{name}": spec for p, part in self._parts.items() for name, spec in part.tensors().items()}

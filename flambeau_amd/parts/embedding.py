@@ -13,6 +13,8 @@ from .base import Part, TensorSpec
 
 
 class TokenEmbedding(Part):
+    replayable = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
@@ -29,6 +31,8 @@ class TokenEmbedding(Part):
 
 
 class OutputHead(Part):
+    replayable = True
+
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size

@@ -10,6 +10,7 @@ from .base import FEED_FORWARDS, FeedForward, Product, TensorSpec
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    replayable = True
     lazy_input = True
 
     def __init__(self, hidden_size: int, intermediate_size: int):

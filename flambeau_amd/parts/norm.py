@@ -11,6 +11,8 @@ from .base import NORMS, Norm, TensorSpec
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
+    replayable = True
+
     def __init__(self, hidden_size: int, eps: float):
         self.hidden_size = hidden_size
         self.eps = eps

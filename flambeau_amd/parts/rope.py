@@ -15,6 +15,8 @@ from .base import POSITION_ENCODINGS, PositionEncoding
 
 @POSITION_ENCODINGS.register("rope_neox")
 class RotaryNeoX(PositionEncoding):
+    replayable = True
+
     def __init__(self, head_dim: int, theta: float, rotated_dims: int | None = None):
         self.head_dim = head_dim
         self.theta = float(theta)
@@ -41,6 +43,8 @@ class RotaryNeoX(PositionEncoding):
 
 @POSITION_ENCODINGS.register("none")
 class NoPositionEncoding(PositionEncoding):
+    replayable = True
+
     def __init__(self, **_):
         pass
 

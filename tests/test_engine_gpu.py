@@ -362,6 +362,50 @@ def test_captured_decode_steps_equal_eager_ones(model_dirs, dtype):
     rh.compare(graphed, reqs, rh.plain_logits(d, reqs), dtype, "captured steps")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_steps_equal_eager_ones(model_dirs, dtype):
+    """Steps that hold prompt portions are recorded while they run and replayed from native code when
+    a step of the same shape comes again.  Every replay, for other requests, contexts and pages than
+    the recording saw, gives bit for bit what the step gives when Python launches it."""
+    name = "D"                                        # two cache groups: two block tables in the metadata
+    d = model_dirs[(name, STORE[dtype])]
+    reqs = rh.make_requests(210, [70, 70, 70, 31, 31, 150], seed=27)
+    from flambeau_amd.engine import ModelRunner, load_model
+    model, _ = load_model(d, dtype=dtype, max_batch_tokens=256)
+    assert model.replayable()
+    portions = rh.trace_portions(reqs, sizes=(16, 9, 16, 2, 16, 9))          # the same sizes again and again
+    mixed = rh.trace_mixed(reqs, seed=4, max_portion=12)
+    results = []
+    for programs in (False, True):
+        runner = ModelRunner(model, n_pages=40, page_size=8, max_slots=4, max_logit_rows=256, step_programs=programs,
+                             decode_graphs=False)
+        runner.storage.fill(float("nan"))
+        got = rh.run_in_process(runner, portions)
+        got2 = rh.run_in_process(runner, mixed)
+        results.append((got, got2))
+        if programs:
+            assert runner.n_replayed > 20
+            # a longer step than any before makes buffers grow: programs recorded on the old ones are
+            # not replayed, and the steps after it are right
+            before = runner.n_recorded
+            big = {"big": rh.make_requests(210, [200], seed=5)["r0"]}
+            ref_big = rh.plain_logits(d, big)
+            rh.compare(rh.run_in_process(runner, rh.trace_whole(big)), big, ref_big, dtype, "after growth: whole")
+            again = rh.run_in_process(runner, portions)
+            assert runner.n_recorded > before + 3
+            for k in got:
+                assert np.array_equal(again[k], got[k]), k
+        else:
+            assert runner.n_replayed == 0 and runner.n_recorded == 0
+    (eager, eager2), (replayed, replayed2) = results
+    assert eager.keys() == replayed.keys() and eager2.keys() == replayed2.keys()
+    for k in eager:
+        assert np.array_equal(eager[k], replayed[k]), k
+    for k in eager2:
+        assert np.array_equal(eager2[k], replayed2[k]), k
+    rh.compare(replayed, reqs, rh.plain_logits(d, reqs), dtype, "recorded steps")
+
+
 @pytest.fixture(scope="module")
 def wide_model_dir(tmp_path_factory):
     """Two layers with the layer sizes of a 7B model (width 4096, 32 heads in 8 groups of 128,
