@@ -62,9 +62,10 @@ class PagePool:
 
 @dataclass(frozen=True)
 class GroupSpec:
-    """Shape of a cache group.  ``window`` = newest keys still needed, 0 = all."""
-    n_kv_heads: int
-    head_dim: int
+    """A cache group as the manager sees it: all it reads is ``window`` (newest rows still needed,
+    0 = all).  Any object with that attribute serves (``parts.base.PageGroup`` in the engine)."""
+    n_kv_heads: int = 1
+    head_dim: int = 1
     window: int = 0
 
 

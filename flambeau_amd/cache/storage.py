@@ -1,18 +1,19 @@
-"""Device memory of the caches: one pool per group of layers, one state table per stateful layer.
+"""Device memory of the caches: one pool per group of paged caches, one table of records per cache
+that keeps a state per slot.
 
-Layout of a group's pool: ``[entries_in_group, n_pages, 2 (K, V), n_kv_heads, page_size,
-head_dim]`` in the compute dtype, so that one (page, kv head) holds ``page_size`` rows of
-``head_dim`` values back to back: a decode kernel streams whole pages of one head.
-(The reference keeps ``[n_pages, page_size, kv_width]`` per layer,
+What a cache looks like is its spec's business (``parts.base.CacheSpec``): the storage asks a spec
+which group of pages it belongs to, lets the first spec of a group allocate the group's pool, and
+hands every entry its view of it.  For keys and values the pool is ``[entries_in_group, n_pages, 2
+(K, V), n_kv_heads, page_size, head_dim]`` in the compute dtype, so that one (page, kv head) holds
+``page_size`` rows of ``head_dim`` values back to back: a decode kernel streams whole pages of one
+head.  (The reference keeps ``[n_pages, page_size, kv_width]`` per layer,
 crates/forward/src/core/scratch.rs:453-586.)
 """
 from __future__ import annotations
 
 import torch
 
-from ..kernels.ops import PagedLayerCache
-from ..parts.base import LayerCache, PagedKVSpec, StateSpec
-from .manager import GroupSpec
+from ..parts.base import CacheSpec, LayerCache
 
 
 class CacheStorage:
@@ -22,23 +23,26 @@ class CacheStorage:
         having its own (or None)."""
         self.page_size = page_size
         self.n_pages = n_pages
-        self.group_specs: list[GroupSpec] = []
+        for i, spec in enumerate(entry_specs):
+            if spec is not None and not isinstance(spec, CacheSpec):
+                raise TypeError(f"run-order entry {i}: {spec!r} is no cache spec")
+        self.group_specs: list = []               # page groups (each has a ``window``), in order of first use
+        self._group_makers: list = []             # the spec that allocates each group's pool
         members: list[list[int]] = []
         owner_group: dict[int, int] = {}
         for i, (spec, share) in enumerate(zip(entry_specs, shares)):
-            if share is not None or not isinstance(spec, PagedKVSpec):
+            group = spec.page_group() if spec is not None and share is None else None
+            if group is None:
                 continue
-            gs = GroupSpec(spec.n_kv_heads, spec.head_dim, spec.window)
-            if gs not in self.group_specs:
-                self.group_specs.append(gs)
+            if group not in self.group_specs:
+                self.group_specs.append(group)
+                self._group_makers.append(spec)
                 members.append([])
-            g = self.group_specs.index(gs)
+            g = self.group_specs.index(group)
             members[g].append(i)
             owner_group[i] = g
-        self.pools = [
-            torch.zeros((len(m), n_pages, 2, gs.n_kv_heads, page_size, gs.head_dim), dtype=dtype, device=device)
-            for gs, m in zip(self.group_specs, members)
-        ]
+        self.pools = [maker.allocate_pool(len(m), n_pages, page_size, dtype, device)
+                      for maker, m in zip(self._group_makers, members)]
         self.states: dict[int, torch.Tensor] = {}
         self.entries: list[LayerCache] = []
         for i, (spec, share) in enumerate(zip(entry_specs, shares)):
@@ -49,17 +53,19 @@ class CacheStorage:
                 if entry_specs[share] != spec:
                     raise ValueError(f"run-order entry {i} reads the cache of entry {share}, whose shape differs")
             lc = LayerCache(writes=share is None)
-            if isinstance(spec, PagedKVSpec):
-                g = owner_group[src]
-                lc.group = g
-                lc.kv = PagedLayerCache(self.pools[g][members[g].index(src)])
-            elif isinstance(spec, StateSpec):
+            if spec is not None:
+                if spec.page_group() is not None:
+                    g = owner_group[src]
+                    lc.group = g
+                    lc.kv = spec.layer_view(self.pools[g], members[g].index(src))
                 if src not in self.states:
-                    self.states[src] = torch.zeros((max_slots, *spec.shape), dtype=spec.dtype, device=device)
-                lc.state = self.states[src]
-            elif spec is not None:
-                raise TypeError(f"run-order entry {i}: unknown cache spec {spec!r}")
+                    state = spec.allocate_state(max_slots, device)
+                    if state is not None:
+                        self.states[src] = state
+                lc.state = self.states.get(src)
             self.entries.append(lc)
+        self._bytes_per_token = sum(spec.bytes_per_token(torch.empty((), dtype=dtype).element_size())
+                                    for spec, share in zip(entry_specs, shares) if spec is not None and share is None)
 
     def zero_slots(self, slots) -> None:
         """Fixed-size state starts at zero for a newly claimed slot
@@ -77,7 +83,7 @@ class CacheStorage:
             p.fill_(value)
 
     def bytes_per_token(self) -> int:
-        return sum(p.shape[0] * 2 * p.shape[3] * p.shape[5] * p.element_size() for p in self.pools)
+        return self._bytes_per_token
 
     def nbytes(self) -> int:
         return sum(p.numel() * p.element_size() for p in self.pools) + sum(

@@ -164,8 +164,7 @@ def cmd_inspect(a) -> int:
             total += numel
     print(f"parameters: {total:,d}")
     specs, shares = model.cache_entries()
-    per_token = sum(2 * s.n_kv_heads * s.head_dim for s, sh in zip(specs, shares) if s is not None and sh is None
-                    and hasattr(s, "n_kv_heads"))
+    per_token = sum(s.bytes_per_token(1) for s, sh in zip(specs, shares) if s is not None and sh is None)
     print(f"cache per token: {per_token:,d} values ({2 * per_token:,d} B in bfloat16, {4 * per_token:,d} B in float32)")
     skipped = check_against_manifest(manifest, src, model.spec.ignored_tensors)
     print("tensors fit the model" + (f" ({len(skipped)} are not read: {', '.join(skipped)})" if skipped else ""))

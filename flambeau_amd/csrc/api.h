@@ -59,6 +59,11 @@ int fl_gemm_skinny_scale_parts(int N, int K, int in_parts);
 int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                 int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_mid_splits(int M, int N, int K);
+// for tests and measurements: waves per block (0, 4, 8) and K-splits (0 = chosen) from the caller
+int fl_gemm_mid_ex(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                   int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
+                   float eps, int waves, int forced_splits, hipStream_t stream);
+int fl_gemm_mid_splits_ex(int M, int N, int K, int waves, int forced);
 // The same fused with the norms around it, as fl_gemm_skinny_fused: a row scale from partial sums of
 // squares, and the product added to the residual stream with the next norm left in factors
 // (out_ssq[M, fl_gemm_mid_parts(N)]; the workspace holds splits * M * N floats, also for one split).
@@ -77,6 +82,15 @@ int fl_reduce_residual(const float* part, float* resid, const float* g, void* xg
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_tiled_splits(int M, int N, int K);
+// for tests and measurements: block shape (0 = chosen, 3 = 256 features x 128 tokens, 6 = 128 x 256) and
+// K-splits (0 = chosen) from the caller
+int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                     int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
+                     float eps, int variant, int forced_splits, hipStream_t stream);
+int fl_gemm_tiled_splits_ex(int M, int N, int K, int forced);
+int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, float* workspace, int M, int N, int K, float* resid,
+                              const float* g, void* xg, float* out_ssq, int variant, hipStream_t stream);
+int fl_gemm_tiled_parts_ex(int M, int N, int variant);
 // The joined q/k/v projection (rows of w in paired order) with rotation and the stores of q and the
 // cache rows in the product's kernel: at most 16 rows, and many rows (shapes whose K is not split).
 int fl_gemm_skinny_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,

@@ -407,9 +407,6 @@ static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, b
     kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from, part_o, part_ml);
 }
 
-static int g_pf_stages = 0;              // ring stages: 0 = two (two blocks fit a compute unit), 3 for experiments
-extern "C" int fl_attn_prefill_set_stages(int n) { g_pf_stages = n; return 0; }
-
 template <int HDP, int NS>
 static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                            const int* tiles, const int* positions, const int* block_table, int max_blocks, int nh,
@@ -501,22 +498,19 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, qt_hint);
     dim3 grid(n_tiles, nkv * (G / qt), n_split);
     const float sl = scale * 1.4426950408889634f;
-#define FL_PF(HDP_, NS_)                                                                                       \
-    if (NS_ == 3 && g_pf_stages == 3)                                                                          \
-        launch_prefill<HDP_, NS_>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                                  max_blocks, nh, sl, window, log2_ps, part_o, part_ml);                       \
-    else                                                                                                       \
-        launch_prefill<HDP_, 2>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                                max_blocks, nh, sl, window, log2_ps, part_o, part_ml)
+    // a ring of two stages: two blocks then fit a compute unit (three stages were no faster)
+#define FL_PF(HDP_)                                                                                            \
+    launch_prefill<HDP_, 2>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
+                            max_blocks, nh, sl, window, log2_ps, part_o, part_ml)
     switch (hdp) {
-        case 32: FL_PF(32, 3); break;
-        case 64: FL_PF(64, 3); break;
-        case 96: FL_PF(96, 3); break;
-        case 128: FL_PF(128, 3); break;
-        case 160: FL_PF(160, 2); break;
-        case 192: FL_PF(192, 2); break;
-        case 224: FL_PF(224, 2); break;
-        default: FL_PF(256, 2); break;
+        case 32: FL_PF(32); break;
+        case 64: FL_PF(64); break;
+        case 96: FL_PF(96); break;
+        case 128: FL_PF(128); break;
+        case 160: FL_PF(160); break;
+        case 192: FL_PF(192); break;
+        case 224: FL_PF(224); break;
+        default: FL_PF(256); break;
     }
 #undef FL_PF
     FL_LAUNCH_CHECK();

@@ -263,32 +263,30 @@ __global__ __launch_bounds__(1024) void gemm_mid_reduce_residual_kernel(const fl
     if (threadIdx.x == 0) out_ssq[(size_t)row * gridDim.x + blockIdx.x] = sq;
 }
 
-static int g_mid_splits = 0;             // 0: chosen from the sizes (a fixed number for experiments)
-static int g_mid_waves = 0;              // waves per block: 0 = chosen from the sizes, else 4 or 8
-extern "C" int fl_gemm_mid_set_splits(int s) { g_mid_splits = s; return 0; }
-extern "C" int fl_gemm_mid_set_waves(int w) { g_mid_waves = w; return 0; }
-
 #define GM_STEPS 4                       // k-steps per chunk
 
 // Waves per block: eight row groups share x where the matrix has row groups enough to fill the
 // chip with such blocks, four otherwise.
-static int mid_waves(int N) {
-    if (g_mid_waves == 4 || g_mid_waves == 8) return g_mid_waves;
+static int mid_waves(int N, int forced = 0) {
+    if (forced == 4 || forced == 8) return forced;
     return ceil_div(N, 16) >= 1024 ? 8 : 4;
 }
 
 // How many ways K is split.  These products are short (tens of microseconds) and run best with
 // about one block per compute unit (measured on the 7B shapes at 32 and 64 rows); a part is at
 // least 4 chunks long.
-extern "C" int fl_gemm_mid_splits(int M, int N, int K) {
+// (The entry points whose names end in _ex take waves per block and K-splits from the caller, for
+// tests and measurements: 0 = chosen here.)
+extern "C" int fl_gemm_mid_splits_ex(int M, int N, int K, int waves, int forced) {
     (void)M;
-    const int blocks = ceil_div(ceil_div(N, 16), mid_waves(N));
+    const int blocks = ceil_div(ceil_div(N, 16), mid_waves(N, waves));
     const int n_chunks = ceil_div(ceil_div(K, 32), GM_STEPS);
-    if (g_mid_splits > 0) return min(g_mid_splits, n_chunks);
+    if (forced > 0) return min(forced, n_chunks);
     int splits = 1;
     while (blocks * splits * 2 <= 320 && n_chunks / (splits * 2) >= 4 && splits < 32) splits *= 2;
     return splits;
 }
+extern "C" int fl_gemm_mid_splits(int M, int N, int K) { return fl_gemm_mid_splits_ex(M, N, K, 0, 0); }
 
 struct MidScale {              // the row scale of a product whose x is a norm in factors (or none)
     const float* in_ssq;
@@ -309,19 +307,19 @@ static void launch_mid_shape(const bf16_t* x, const bf16_t* wp, TOut* out, int M
 
 template <int MT, typename TOut, bool SWIGLU>
 static void launch_mid(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits, int out_cols,
-                       const MidScale& sc, hipStream_t stream) {
-    if (mid_waves(N) == 8) launch_mid_shape<MT, 8, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream);
+                       const MidScale& sc, hipStream_t stream, int waves) {
+    if (mid_waves(N, waves) == 8) launch_mid_shape<MT, 8, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream);
     else launch_mid_shape<MT, 4, GM_STEPS, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream);
 }
 
 template <typename TOut, bool SWIGLU>
 static void launch_mid_mt(int mt, const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int splits,
-                          int out_cols, const MidScale& sc, hipStream_t stream) {
+                          int out_cols, const MidScale& sc, hipStream_t stream, int waves = 0) {
     switch (mt) {
-        case 1: launch_mid<1, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
-        case 2: launch_mid<2, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
-        case 3: launch_mid<3, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
-        default: launch_mid<4, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream); break;
+        case 1: launch_mid<1, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream, waves); break;
+        case 2: launch_mid<2, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream, waves); break;
+        case 3: launch_mid<3, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream, waves); break;
+        default: launch_mid<4, TOut, SWIGLU>(x, wp, out, M, N, K, splits, out_cols, sc, stream, waves); break;
     }
 }
 
@@ -339,9 +337,10 @@ static int mid_checks(const void* x, const void* w_packed, int M, int N, int K) 
 // from the N interleaved gate/up rows of w; K is not split then.  in_ssq (or null): [M, in_parts]
 // partial sums of squares of the rows that x was made from; every token's results are multiplied
 // by rsqrt(sum / K + eps).
-extern "C" int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
-                                  int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
-                                  float eps, hipStream_t stream) {
+extern "C" int fl_gemm_mid_ex(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                              int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
+                              float eps, int waves, int forced_splits, hipStream_t stream) {
+    FL_CHECK(waves == 0 || waves == 4 || waves == 8, "gemm_mid: %d waves per block (0, 4 or 8)", waves);
     if (mid_checks(x, w_packed, M, N, K)) return -1;
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_mid: unknown output dtype %d", out_dtype);
     FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_mid: unknown epilogue %d", epilogue);
@@ -355,13 +354,13 @@ extern "C" int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
     const MidScale sc = {in_ssq, in_parts, eps};
-    const int splits = epilogue ? 1 : fl_gemm_mid_splits(M, N, K);
+    const int splits = epilogue ? 1 : fl_gemm_mid_splits_ex(M, N, K, waves, forced_splits);
     FL_CHECK(splits == 1 || workspace, "gemm_mid: this shape splits K %d ways and needs a workspace", splits);
     if (epilogue) {
-        if (out_dtype == FL_F32) launch_mid_mt<float, true>(mt, xb, wb, (float*)out, M, N, K, 1, out_cols, sc, stream);
-        else launch_mid_mt<bf16_t, true>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, out_cols, sc, stream);
+        if (out_dtype == FL_F32) launch_mid_mt<float, true>(mt, xb, wb, (float*)out, M, N, K, 1, out_cols, sc, stream, waves);
+        else launch_mid_mt<bf16_t, true>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, out_cols, sc, stream, waves);
     } else if (splits > 1) {
-        launch_mid_mt<float, false>(mt, xb, wb, workspace, M, N, K, splits, N, sc, stream);
+        launch_mid_mt<float, false>(mt, xb, wb, workspace, M, N, K, splits, N, sc, stream, waves);
         FL_LAUNCH_CHECK();
         const size_t total = (size_t)M * N;
         const unsigned rb = (unsigned)((total + 255) / 256);
@@ -370,12 +369,18 @@ extern "C" int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out
         else
             gemm_mid_reduce_kernel<bf16_t><<<rb, 256, 0, stream>>>(workspace, (bf16_t*)out, total, splits);
     } else if (out_dtype == FL_F32) {
-        launch_mid_mt<float, false>(mt, xb, wb, (float*)out, M, N, K, 1, N, sc, stream);
+        launch_mid_mt<float, false>(mt, xb, wb, (float*)out, M, N, K, 1, N, sc, stream, waves);
     } else {
-        launch_mid_mt<bf16_t, false>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, N, sc, stream);
+        launch_mid_mt<bf16_t, false>(mt, xb, wb, (bf16_t*)out, M, N, K, 1, N, sc, stream, waves);
     }
     FL_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
+                                  int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
+                                  float eps, hipStream_t stream) {
+    return fl_gemm_mid_ex(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, in_ssq, in_parts, eps, 0, 0, stream);
 }
 
 extern "C" int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,

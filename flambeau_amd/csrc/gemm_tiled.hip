@@ -399,10 +399,9 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 }
 
 // Shape of the block: 0 = chosen from the sizes, 3 = 256 features x 128 tokens (4 waves, ring of 3, two blocks
-// per compute unit), 6 = 128 x 256 (8 waves, ring of 4, one block per compute unit); set for tests and experiments.
-static int g_tiled_variant = 0;
-extern "C" int fl_gemm_tiled_set_variant(int v) { g_tiled_variant = v; return 0; }
-
+// per compute unit), 6 = 128 x 256 (8 waves, ring of 4, one block per compute unit).  The entry points
+// whose names end in _ex take the shape (and the number of K-splits) from the caller, for tests and
+// measurements; the others choose.
 static int tiled_variant(int variant, int splits, int M, int N) {
     // 256 x 128 where that fills the chip (and for few rows), else 128 x 256
     if (variant == 3 || variant == 6) return variant;
@@ -410,9 +409,10 @@ static int tiled_variant(int variant, int splits, int M, int N) {
 }
 
 // Parts in which the residual epilogue leaves a token's sum of squares: one per tile of features.
-extern "C" int fl_gemm_tiled_parts(int M, int N) {
-    return ceil_div(N, tiled_variant(g_tiled_variant, 1, M, N) == 6 ? 128 : 256);
+extern "C" int fl_gemm_tiled_parts_ex(int M, int N, int variant) {
+    return ceil_div(N, tiled_variant(variant, 1, M, N) == 6 ? 128 : 256);
 }
+extern "C" int fl_gemm_tiled_parts(int M, int N) { return fl_gemm_tiled_parts_ex(M, N, 0); }
 
 template <typename TOut, int EPI>
 static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out,
@@ -424,25 +424,25 @@ static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16
         launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu);
 }
 
-static int g_tiled_splits = 0;           // 0: chosen from the sizes (a fixed number for experiments)
-extern "C" int fl_gemm_tiled_set_splits(int s) { g_tiled_splits = s; return 0; }
-
-// How many ways K is split for a product of this shape: 1 if the grid fills the chip.
-extern "C" int fl_gemm_tiled_splits(int M, int N, int K) {
-    if (g_tiled_splits > 0) return max(1, min(g_tiled_splits, ceil_div(K, 32) / 8));
+// How many ways K is split for a product of this shape: 1 if the grid fills the chip (forced > 0: that
+// many, as far as K allows).
+extern "C" int fl_gemm_tiled_splits_ex(int M, int N, int K, int forced) {
+    if (forced > 0) return max(1, min(forced, ceil_div(K, 32) / 8));
     const int blocks = ceil_div(M, TG_BM) * ceil_div(N, TG_BN);
     const int steps = ceil_div(K, 32);
     int splits = 1;
     while (blocks * splits < 288 && splits < 16 && steps / (splits * 2) >= 8) splits *= 2;          // (288: measured on the 7B shapes, 65 to 1,536 rows)
     return splits;
 }
+extern "C" int fl_gemm_tiled_splits(int M, int N, int K) { return fl_gemm_tiled_splits_ex(M, N, K, 0); }
 
 // epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up from the
 // N interleaved gate/up rows of w (K is not split then).  in_ssq (or null): [M, in_parts] partial sums of
 // squares of the rows that x was made from; every token's results are multiplied by rsqrt(sum / K + eps).
-extern "C" int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* out, float* workspace,
-                                    int out_dtype, int M, int N, int K, int epilogue, int out_cols,
-                                    const float* in_ssq, int in_parts, float eps, hipStream_t stream) {
+extern "C" int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, float* workspace,
+                                int out_dtype, int M, int N, int K, int epilogue, int out_cols,
+                                const float* in_ssq, int in_parts, float eps, int variant, int forced_splits,
+                                hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_tiled: unknown output dtype %d", out_dtype);
@@ -454,12 +454,13 @@ extern "C" int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* o
     FL_CHECK(!in_ssq || in_parts > 0, "gemm_tiled: a row scale over %d parts", in_parts);
     if (M == 0) return 0;
     const int n_steps = ceil_div(K, 32);
-    const int splits = epilogue ? 1 : fl_gemm_tiled_splits(M, N, K);
+    FL_CHECK(variant == 0 || variant == 3 || variant == 6, "gemm_tiled: block shape %d (0, 3 or 6)", variant);
+    const int splits = epilogue ? 1 : fl_gemm_tiled_splits_ex(M, N, K, forced_splits);
     FL_CHECK(splits == 1 || workspace, "gemm_tiled: this shape splits K %d ways and needs a workspace", splits);
     const int per = ceil_div(n_steps, splits);
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
-    const int v = g_tiled_variant;
+    const int v = variant;
     const RopeStore none{};
     const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
     if (epilogue) {
@@ -485,10 +486,16 @@ extern "C" int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* o
     return 0;
 }
 
+extern "C" int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* out, float* workspace,
+                                    int out_dtype, int M, int N, int K, int epilogue, int out_cols,
+                                    const float* in_ssq, int in_parts, float eps, hipStream_t stream) {
+    return fl_gemm_tiled_ex(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, in_ssq, in_parts, eps, 0, 0, stream);
+}
+
 extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace,
                              int out_dtype, int M, int N, int K, int epilogue, int out_cols,
                              hipStream_t stream) {
-    return fl_gemm_tiled_scaled(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, stream);
+    return fl_gemm_tiled_ex(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, 0, 0, stream);
 }
 
 // resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_tiled_residual_parts(M, N, K)]
@@ -496,8 +503,10 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
 // product's epilogue does it (one part per tile of features); where it is, the partial sums go to
 // the workspace (fl_gemm_tiled_splits(M, N, K) * M * N floats) and the kernel that adds them does it
 // (one part per 4096 features, fl_reduce_residual).
-extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
-                                      float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream) {
+extern "C" int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                                         float* resid, const float* g, void* xg, float* out_ssq, int variant,
+                                         hipStream_t stream) {
+    FL_CHECK(variant == 0 || variant == 3 || variant == 6, "gemm_tiled_residual: block shape %d (0, 3 or 6)", variant);
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_residual: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled_residual: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(N % 4 == 0, "gemm_tiled_residual: N=%d is no multiple of 4 (16-byte accesses to the residual rows)", N);
@@ -509,16 +518,21 @@ extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, float
     const int splits = fl_gemm_tiled_splits(M, N, K);
     if (splits > 1) {
         FL_CHECK(workspace && (uintptr_t)workspace % 16 == 0, "gemm_tiled_residual: this shape splits K %d ways and needs a workspace", splits);
-        launch_tiled<float, TG_PLAIN>(g_tiled_variant, splits, stream, (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
+        launch_tiled<float, TG_PLAIN>(variant, splits, stream, (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
                                       n_steps, ceil_div(n_steps, splits), N, RopeStore{});
         FL_LAUNCH_CHECK();
         return fl_reduce_residual(workspace, resid, g, xg, out_ssq, M, N, splits, stream);
     }
     const TiledFusion fu = {nullptr, 0, 0.f, resid, g, (bf16_t*)xg, out_ssq};
-    launch_tiled<float, TG_RESIDUAL>(g_tiled_variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, resid, M, N, K,
+    launch_tiled<float, TG_RESIDUAL>(variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, resid, M, N, K,
                                      n_steps, n_steps, N, RopeStore{}, fu);
     FL_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                                      float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream) {
+    return fl_gemm_tiled_residual_ex(x, w_packed, workspace, M, N, K, resid, g, xg, out_ssq, 0, stream);
 }
 
 // Parts in which fl_gemm_tiled_residual leaves a token's sum of squares.
@@ -549,7 +563,7 @@ extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, in
                           PagedCache{cache_base, nkv, page_size, hd, n_pages}, nh, rot, write_cache};
     const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
     const int n_steps = ceil_div(K, 32);
-    launch_tiled<bf16_t, TG_ROPE>(g_tiled_variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)q_out,
+    launch_tiled<bf16_t, TG_ROPE>(0, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)q_out,
                                   M, N, K, n_steps, n_steps, N, rs, fu);
     FL_LAUNCH_CHECK();
     return 0;

@@ -30,6 +30,9 @@ register_signatures({
     "fl_gemm_mid_residual": [P, P, P, I, I, I, P, P, P, P, P],
     "fl_gemm_mid_parts": [I],
     "fl_gemm_mid_partials": [P, P, P, I, I, I, P, I, F, P],
+    "fl_gemm_mid_ex": [P, P, P, P, I, I, I, I, I, I, P, I, F, I, I, P],
+    "fl_gemm_tiled_ex": [P, P, P, P, I, I, I, I, I, I, P, I, F, I, I, P],
+    "fl_gemm_tiled_residual_ex": [P, P, P, I, I, I, P, P, P, P, I, P],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, P, I, P],
@@ -204,28 +207,34 @@ def gemm_tiled_rope(x, w_packed, n_features: int, store: RopeStore, row_scale: N
     return store.q_out
 
 
-def gemm_mid_splits(M: int, N: int, K: int) -> int:
+def gemm_mid_splits(M: int, N: int, K: int, waves: int = 0, splits: int = 0) -> int:
     from .library import load
-    return load().fl_gemm_mid_splits(M, N, K)
+    return load().fl_gemm_mid_splits_ex(M, N, K, waves, splits)
 
 
-def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None):
+def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None,
+             waves: int = 0, splits: int = 0):
     """``out = x @ w.T`` for 17 to 64 rows of x (fewer are allowed) and K a multiple of 32: the
     waves of a block share x through LDS.  A narrow matrix splits K and needs ``workspace``
     (float32, ``gemm_mid_splits(M, N, K) * M * N`` values).  ``swiglu_rows`` and ``row_scale`` as in
-    ``gemm_skinny``."""
+    ``gemm_skinny``.  ``waves`` (4 or 8 per block) and ``splits`` fix what the kernel would choose
+    (for tests and measurements)."""
     M, K = x.shape
     N = swiglu_rows or out.shape[1]
     if w_packed.numel() != _packed_size(N, K):
         raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
-    splits = 1 if swiglu_rows else gemm_mid_splits(M, N, K)
-    if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
-        raise KernelError(f"gemm_mid: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
+    n_splits = 1 if swiglu_rows else gemm_mid_splits(M, N, K, waves, splits)
+    if n_splits > 1 and (workspace is None or workspace.numel() < n_splits * M * N):
+        raise KernelError(f"gemm_mid: [{M}, {N}, {K}] splits K {n_splits} ways and needs a workspace of {n_splits * M * N} floats")
     ssq, parts, eps = _row_scale_args(row_scale, M, K)
-    call("fl_gemm_mid_scaled", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         _check(out, "gemm.out", None, (M, None)),
-         _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps, stream_handle())
+    args = (_check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+            _check(out, "gemm.out", None, (M, None)),
+            _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
+            dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps)
+    if waves or splits:
+        call("fl_gemm_mid_ex", *args, int(waves), int(splits), stream_handle())
+    else:
+        call("fl_gemm_mid_scaled", *args, stream_handle())
     return out
 
 
@@ -267,37 +276,46 @@ def gemm_mid_residual(x, w_packed, resid, g, xg, ssq, eps: float, workspace) -> 
     return NormedRows(xg, ssq, float(eps), resid, g)
 
 
-def gemm_tiled_splits(M: int, N: int, K: int) -> int:
+def gemm_tiled_splits(M: int, N: int, K: int, splits: int = 0) -> int:
     from .library import load
-    return load().fl_gemm_tiled_splits(M, N, K)
+    return load().fl_gemm_tiled_splits_ex(M, N, K, splits)
 
 
-def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None):
+def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None,
+               variant: int = 0, splits: int = 0):
     """``out = x @ w.T`` for many rows of x.  A shape whose grid would not fill the chip splits K
     and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values).  With
-    ``swiglu_rows`` and ``row_scale`` see ``gemm_skinny``."""
+    ``swiglu_rows`` and ``row_scale`` see ``gemm_skinny``.  ``variant`` (block shape: 3 = 256 features x
+    128 tokens, 6 = 128 x 256) and ``splits`` fix what the kernel would choose (for tests and
+    measurements)."""
     M, K = x.shape
     N = swiglu_rows or out.shape[1]
     if w_packed.numel() != _packed_size(N, K):
         raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
-    splits = 1 if swiglu_rows else gemm_tiled_splits(M, N, K)
-    if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
-        raise KernelError(f"gemm_tiled: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
+    n_splits = 1 if swiglu_rows else gemm_tiled_splits(M, N, K, splits)
+    if n_splits > 1 and (workspace is None or workspace.numel() < n_splits * M * N):
+        raise KernelError(f"gemm_tiled: [{M}, {N}, {K}] splits K {n_splits} ways and needs a workspace of {n_splits * M * N} floats")
     ssq, parts, eps = _row_scale_args(row_scale, M, K)
-    call("fl_gemm_tiled_scaled", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         _check(out, "gemm.out", None, (M, None)),
-         _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-         dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps, stream_handle())
+    args = (_check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+            _check(out, "gemm.out", None, (M, None)),
+            _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
+            dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps)
+    if variant or splits:
+        call("fl_gemm_tiled_ex", *args, int(variant), int(splits), stream_handle())
+    else:
+        call("fl_gemm_tiled_scaled", *args, stream_handle())
     return out
 
 
-def tiled_parts(M: int, n_features: int, K: int) -> int:
+def tiled_parts(M: int, n_features: int, K: int, variant: int = 0) -> int:
     """Parts in which ``gemm_tiled_residual`` leaves the sums of squares of its N features."""
     from .library import load
+    if variant and gemm_tiled_splits(M, n_features, K) == 1:
+        return load().fl_gemm_tiled_parts_ex(M, n_features, variant)
     return load().fl_gemm_tiled_residual_parts(M, n_features, K)
 
 
-def gemm_tiled_residual(x, w_packed, resid, g, xg, ssq, eps: float, workspace=None) -> NormedRows:
+def gemm_tiled_residual(x, w_packed, resid, g, xg, ssq, eps: float, workspace=None, variant: int = 0) -> NormedRows:
     """``gemm_skinny_residual`` for many rows: ``ssq[m, p]`` = sums over the tiles of features where K
     is not split, else over 4096 features each (the kernel that adds the K-splits does it then and
     needs ``workspace``: float32, ``gemm_tiled_splits(M, N, K) * M * N`` values)."""
@@ -308,11 +326,15 @@ def gemm_tiled_residual(x, w_packed, resid, g, xg, ssq, eps: float, workspace=No
     splits = gemm_tiled_splits(M, N, K)
     if splits > 1 and (workspace is None or workspace.numel() < splits * M * N):
         raise KernelError(f"gemm_tiled_residual: [{M}, {N}, {K}] splits K {splits} ways and needs a workspace of {splits * M * N} floats")
-    call("fl_gemm_tiled_residual", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-         M, N, K, _check(resid, "gemm.resid", torch.float32, (M, N)), _check(g, "gemm.g", torch.float32, (N,)),
-         _check(xg, "gemm.xg", torch.bfloat16, (M, N)), _check(ssq, "gemm.ssq", torch.float32, (M, tiled_parts(M, N, K))),
-         stream_handle())
+    args = (_check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+            _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
+            M, N, K, _check(resid, "gemm.resid", torch.float32, (M, N)), _check(g, "gemm.g", torch.float32, (N,)),
+            _check(xg, "gemm.xg", torch.bfloat16, (M, N)),
+            _check(ssq, "gemm.ssq", torch.float32, (M, tiled_parts(M, N, K, variant))))
+    if variant:
+        call("fl_gemm_tiled_residual_ex", *args, int(variant), stream_handle())
+    else:
+        call("fl_gemm_tiled_residual", *args, stream_handle())
     return NormedRows(xg, ssq, float(eps), resid, g)
 
 

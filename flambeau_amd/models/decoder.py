@@ -15,7 +15,7 @@ from dataclasses import dataclass, field
 import torch
 
 from ..kernels import ops
-from ..parts import BLOCKS, NORMS, OutputHead, PartSpec, ResidualStream, TokenEmbedding
+from ..parts import BLOCKS, EMBEDDINGS, HEADS, NORMS, PartSpec, ResidualStream
 
 
 @dataclass
@@ -43,6 +43,8 @@ class ModelSpec:
     tied_head: bool = False
     eos_token_id: int | None = None
     bos_token_id: int | None = None
+    embedding: PartSpec | None = None  # None: the plain table look-up ("token_embedding")
+    head: PartSpec | None = None       # None: the plain matrix product ("linear_head"), tied or not
     eos_token_ids: tuple = ()         # every id that ends a sequence (eos_token_id is the first)
     ignored_tensors: tuple = ()       # name patterns (fnmatch) of tensors a file may hold and the model does not read
 
@@ -54,10 +56,11 @@ class DecoderModel:
     def __init__(self, spec: ModelSpec, rt):
         self.spec = spec
         self.rt = rt
-        self.embedding = TokenEmbedding(spec.vocab_size, spec.hidden_size)
+        sizes = dict(vocab_size=spec.vocab_size, hidden_size=spec.hidden_size)
+        self.embedding = EMBEDDINGS.create(spec.embedding or PartSpec("token_embedding", sizes))
         self.blocks = [BLOCKS.create(ls.block) for ls in spec.layers]
         self.final_norm = NORMS.create(spec.final_norm)
-        self.head = OutputHead(spec.vocab_size, spec.hidden_size, tied=spec.tied_head)
+        self.head = HEADS.create(spec.head or PartSpec("linear_head", dict(sizes, tied=spec.tied_head)))
         self._signature_mixers = None
         for i, e in enumerate(spec.run_order):
             if not 0 <= e.layer < len(self.blocks):

@@ -38,20 +38,78 @@ class TensorSpec:
     role: str = "matrix"
 
 
+class CacheSpec:
+    """What one run-order entry keeps per request, and how that is laid out on the device.  The cache
+    storage and the manager know nothing of keys, values or states: they ask the spec.
+
+    A spec is either *paged* (per-token rows that grow with the request: ``page_group()`` names the
+    group of layers it shares pages and block tables with, ``allocate_pool`` makes the group's
+    memory, ``layer_view`` hands one entry its part of it) or *per slot* (a record of fixed size per
+    live request: ``allocate_state``).  Another kind of cache (latent rows, keys and values of
+    different widths) is another subclass; nothing in ``cache/`` changes."""
+
+    def page_group(self):
+        """A hashable key with a ``window`` attribute (newest rows still needed, 0: all): entries with
+        equal keys share one page pool, one free list and one block table per request.  ``None``:
+        this cache is not paged."""
+        return None
+
+    def allocate_pool(self, n_entries: int, n_pages: int, page_size: int, dtype, device):
+        """The memory of a group of ``n_entries`` paged caches; its first axis indexes the entries."""
+        raise NotImplementedError
+
+    def layer_view(self, pool, index: int):
+        """What entry ``index`` of the group sees of the pool (given to its mixer as ``LayerCache.kv``)."""
+        raise NotImplementedError
+
+    def allocate_state(self, max_slots: int, device):
+        """``[max_slots, ...]``: one record per slot, or ``None`` if this cache keeps none."""
+        return None
+
+    def bytes_per_token(self, element_size: int) -> int:
+        """Bytes one token adds to one entry's cache (for reports)."""
+        return 0
+
+
 @dataclass(frozen=True)
-class PagedKVSpec:
-    """Per-token rows that grow with the request: keys and values in pages.
-    ``window`` = number of newest keys still needed (0: all)."""
+class PageGroup:
+    """Key of a group of paged caches.  ``window`` = newest rows still needed, 0 = all."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
 
 
 @dataclass(frozen=True)
-class StateSpec:
+class PagedKVSpec(CacheSpec):
+    """Per-token rows that grow with the request: keys and values in pages.
+    ``window`` = number of newest keys still needed (0: all).  One (page, kv head) holds
+    ``page_size`` rows of ``head_dim`` values back to back, keys row by row and values transposed."""
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+    def page_group(self):
+        return PageGroup(self.n_kv_heads, self.head_dim, self.window)
+
+    def allocate_pool(self, n_entries, n_pages, page_size, dtype, device):
+        return torch.zeros((n_entries, n_pages, 2, self.n_kv_heads, page_size, self.head_dim), dtype=dtype, device=device)
+
+    def layer_view(self, pool, index):
+        from ..kernels.ops import PagedLayerCache
+        return PagedLayerCache(pool[index])
+
+    def bytes_per_token(self, element_size):
+        return 2 * self.n_kv_heads * self.head_dim * element_size
+
+
+@dataclass(frozen=True)
+class StateSpec(CacheSpec):
     """Per-request state of fixed size, one record per slot, zeroed when a slot is claimed."""
     shape: tuple
     dtype: torch.dtype = torch.float32
+
+    def allocate_state(self, max_slots, device):
+        return torch.zeros((max_slots, *self.shape), dtype=self.dtype, device=device)
 
 
 @dataclass
@@ -260,6 +318,8 @@ class PartRegistry:
         return sorted(self._makers)
 
 
+EMBEDDINGS = PartRegistry("embedding")
+HEADS = PartRegistry("output head")
 MIXERS = PartRegistry("mixer")
 FEED_FORWARDS = PartRegistry("feed-forward")
 NORMS = PartRegistry("norm")

@@ -1,4 +1,8 @@
-"""Token embedding and output head.
+"""Token embedding and output head.  Both are parts like the others: a model's description names
+them by registry key (``EMBEDDINGS``, ``HEADS``), so a scaled embedding or a head with a soft cap is
+another registered class, not a change to the model's code.  An embedding must offer ``weight``
+(the table, for a tied head) and ``forward(tokens, out)``; a head ``bind(weights, rt,
+embedding_table=...)`` and ``forward(x, max_rows) -> float32 logits``.
 
 h0[i,:] = E[token[i],:], no scaling (crates/forward/src/core/composites/embed.rs:26-62);
 logits = norm_f(x) Wlm^T in 32-bit, a tied head being the embedding table again
@@ -9,9 +13,10 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import Part, TensorSpec
+from .base import EMBEDDINGS, HEADS, Part, TensorSpec
 
 
+@EMBEDDINGS.register("token_embedding")
 class TokenEmbedding(Part):
     replayable = True
 
@@ -30,6 +35,7 @@ class TokenEmbedding(Part):
         return ops.embed(self.weight, tokens, out)
 
 
+@HEADS.register("linear_head")
 class OutputHead(Part):
     replayable = True
 

@@ -55,4 +55,5 @@ def config_from_dir(model_dir):
 
 
 def _load_builtin():
-    from .models import mistral  # noqa: F401  (registers itself)
+    from . import models
+    models.discover()           # every module under models/ registers its architecture

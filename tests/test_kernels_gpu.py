@@ -483,34 +483,35 @@ def test_gemm_tiled_block_shapes(variant, M, N, K):
     x, w = rnd(M, K, dtype=torch.bfloat16, seed=23), rnd(N, K, dtype=torch.bfloat16, seed=24, scale=0.05)
     g = 1 + rnd(N, seed=25, scale=0.1)
     resid0 = rnd(M, N, seed=26)
-    load().fl_gemm_tiled_set_variant(variant)
-    try:
-        splits = tuned().gemm_tiled_splits(M, N, K)
-        ws = torch.empty(splits * M * N, dtype=torch.float32, device=DEV) if splits > 1 else None
-        got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
-        tuned().gemm_tiled(x, pack_weight(w), got, ws)
-        ref = x.double() @ w.double().T
-        assert (got.double() - ref).abs().max() < 1e-5 * ref.abs().max()
-        if splits == 1:
-            resid = resid0.clone()
-            xg = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
-            ssq = torch.full((M, tuned().tiled_parts(M, N, K)), float("nan"), dtype=torch.float32, device=DEV)
-            rows = tuned().gemm_tiled_residual(x, pack_weight(w), resid, g, xg, ssq, 1e-5)
-            want = resid0.double() + ref
-            assert (resid.double() - want).abs().max() < 1e-5 * want.abs().max()
-            assert (xg.double() - want * g.double()).abs().max() < 5e-3 * (want * g.double()).abs().max()
-            assert (ssq.double().sum(dim=1) - (want * want).sum(dim=1)).abs().max() < 1e-4 * (want * want).sum(dim=1).max()
-            # the rows in factors feed a product that scales by the norm itself
-            w2 = rnd(200, N, dtype=torch.bfloat16, seed=27, scale=0.05)
-            out2 = torch.full((M, 200), float("nan"), dtype=torch.float32, device=DEV)
-            sp2 = tuned().gemm_tiled_splits(M, 200, N)
-            ws2 = torch.empty(sp2 * M * 200, dtype=torch.float32, device=DEV) if sp2 > 1 else None
-            tuned().gemm_tiled(rows.xg, pack_weight(w2), out2, ws2, row_scale=rows)
-            normed = want * g.double() * torch.rsqrt((want * want).mean(dim=1, keepdim=True) + 1e-5)
-            ref2 = normed @ w2.double().T
-            assert (out2.double() - ref2).abs().max() < 1e-2 * ref2.abs().max()
-    finally:
-        load().fl_gemm_tiled_set_variant(0)
+    splits = tuned().gemm_tiled_splits(M, N, K)
+    ws = torch.empty(splits * M * N, dtype=torch.float32, device=DEV) if splits > 1 else None
+    got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    tuned().gemm_tiled(x, pack_weight(w), got, ws, variant=variant)
+    ref = x.double() @ w.double().T
+    assert (got.double() - ref).abs().max() < 1e-5 * ref.abs().max()
+    # a number of K-splits that the sizes would not choose
+    ws3 = torch.empty(3 * M * N, dtype=torch.float32, device=DEV)
+    got3 = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    tuned().gemm_tiled(x, pack_weight(w), got3, ws3, variant=variant, splits=3)
+    assert (got3.double() - ref).abs().max() < 1e-5 * ref.abs().max()
+    if splits == 1:
+        resid = resid0.clone()
+        xg = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ssq = torch.full((M, tuned().tiled_parts(M, N, K, variant)), float("nan"), dtype=torch.float32, device=DEV)
+        rows = tuned().gemm_tiled_residual(x, pack_weight(w), resid, g, xg, ssq, 1e-5, variant=variant)
+        want = resid0.double() + ref
+        assert (resid.double() - want).abs().max() < 1e-5 * want.abs().max()
+        assert (xg.double() - want * g.double()).abs().max() < 5e-3 * (want * g.double()).abs().max()
+        assert (ssq.double().sum(dim=1) - (want * want).sum(dim=1)).abs().max() < 1e-4 * (want * want).sum(dim=1).max()
+        # the rows in factors feed a product that scales by the norm itself
+        w2 = rnd(200, N, dtype=torch.bfloat16, seed=27, scale=0.05)
+        out2 = torch.full((M, 200), float("nan"), dtype=torch.float32, device=DEV)
+        sp2 = tuned().gemm_tiled_splits(M, 200, N)
+        ws2 = torch.empty(sp2 * M * 200, dtype=torch.float32, device=DEV) if sp2 > 1 else None
+        tuned().gemm_tiled(rows.xg, pack_weight(w2), out2, ws2, row_scale=rows, variant=variant)
+        normed = want * g.double() * torch.rsqrt((want * want).mean(dim=1, keepdim=True) + 1e-5)
+        ref2 = normed @ w2.double().T
+        assert (out2.double() - ref2).abs().max() < 1e-2 * ref2.abs().max()
 
 
 def test_gemm_tiled_splits_k_for_small_grids():
@@ -535,18 +536,12 @@ def test_gemm_mid_against_plain(out_dtype, waves, M, N, K):
     packed = pack_weight(w)
     ref = x.double() @ w.double().T
     tol = 1e-5 if out_dtype == torch.float32 else 5e-3
-    load().fl_gemm_mid_set_waves(waves)
-    try:
-        for splits in (0, 1, 3):
-            load().fl_gemm_mid_set_splits(splits)
-            n = tuned().gemm_mid_splits(M, N, K)
-            ws = torch.full((n * M * N,), float("nan"), dtype=torch.float32, device=DEV) if n > 1 else None
-            got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-            tuned().gemm_mid(x, packed, got, ws)
-            assert (got.double() - ref).abs().max() < tol * ref.abs().max(), (splits, n)
-    finally:
-        load().fl_gemm_mid_set_splits(0)
-        load().fl_gemm_mid_set_waves(0)
+    for splits in (0, 1, 3):
+        n = tuned().gemm_mid_splits(M, N, K, waves, splits)
+        ws = torch.full((n * M * N,), float("nan"), dtype=torch.float32, device=DEV) if n > 1 else None
+        got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+        tuned().gemm_mid(x, packed, got, ws, waves=waves, splits=splits)
+        assert (got.double() - ref).abs().max() < tol * ref.abs().max(), (splits, n)
 
 
 def test_gemm_mid_refuses_what_it_cannot_do():

@@ -201,8 +201,8 @@ def _register_toys():
     from flambeau_amd.config.base import KeyReader
     from flambeau_amd.kernels import ops
     from flambeau_amd.models.decoder import LayerSpec, ModelSpec, RunEntry
-    from flambeau_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward, Mixer, Norm, PartSpec,
-                                    PositionEncoding, StateSpec, TensorSpec)
+    from flambeau_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheSpec, FeedForward, Mixer, Norm,
+                                    PageGroup, PartSpec, PositionEncoding, StateSpec, TensorSpec)
     from flambeau_amd.registry import register_architecture
 
     if "toy_decay_sum" in MIXERS.known():
@@ -234,6 +234,56 @@ def _register_toys():
                 cache.state[slot] = s
             delta = self.rt.buffer("delta", n, H, torch.float32)
             self.rt.gemm(sums.to(x.dtype), self.w, delta)
+            return delta
+
+    @dataclass(frozen=True)
+    class LatentRows(CacheSpec):
+        """A paged cache that is not keys and values: one float32 row of ``width`` per token, in a
+        pool laid out ``[entries, pages, page_size, width]``; the newest ``window`` rows are needed."""
+        width: int
+        window: int
+
+        def page_group(self):
+            return PageGroup(0, self.width, self.window)
+
+        def allocate_pool(self, n_entries, n_pages, page_size, dtype, device):
+            return torch.full((n_entries, n_pages, page_size, self.width), float("nan"), dtype=torch.float32, device=device)
+
+        def layer_view(self, pool, index):
+            return pool[index]
+
+        def bytes_per_token(self, element_size):
+            return 4 * self.width
+
+    @MIXERS.register("toy_window_mean")
+    class WindowMean(Mixer):
+        """z_t = x_t is kept in pages of its own kind; delta_t = mean(z over the last ``window`` tokens) W^T."""
+        def __init__(self, hidden_size, window):
+            self.hidden_size, self.window = hidden_size, window
+
+        def cache_spec(self):
+            return LatentRows(self.hidden_size, self.window)
+
+        def tensors(self):
+            return {"w.weight": TensorSpec((self.hidden_size, self.hidden_size))}
+
+        def bind(self, weights, rt):
+            self.rt, self.w = rt, rt.prepare_weight(weights["w.weight"])
+
+        def forward(self, x, step, cache):
+            n, H = x.shape
+            pool, table = cache.kv, step.block_tables[cache.group]
+            ps = pool.shape[1]
+            pos, seq = step.positions.long(), step.tok_seq.long()
+            pool[table[seq, pos // ps].long(), pos % ps] = x.float()          # this step's rows first, then every query reads the pages
+            means = torch.empty(n, H, dtype=torch.float32, device=x.device)
+            for s, (q0, ql, p0) in enumerate(zip(step.host.q_starts, step.host.q_lens, step.host.start_pos)):
+                for i in range(ql):
+                    p = p0 + i
+                    t = torch.arange(max(0, p - self.window + 1), p + 1, device=x.device)
+                    means[q0 + i] = pool[table[s, t // ps].long(), t % ps].mean(dim=0)
+            delta = self.rt.buffer("delta", n, H, torch.float32)
+            self.rt.gemm(means.to(x.dtype), self.w, delta)
             return delta
 
     @POSITION_ENCODINGS.register("toy_position_scale")
@@ -329,6 +379,7 @@ def _register_toys():
         ffns = {"swiglu": PartSpec("swiglu", dict(hidden_size=H, intermediate_size=2 * H)),
                 "routed": PartSpec("toy_routed", dict(hidden_size=H, inner_size=24, n_experts=3))}
         mixers = {
+            "mean": PartSpec("toy_window_mean", dict(hidden_size=H, window=10)),
             "decay": PartSpec("toy_decay_sum", dict(hidden_size=H, decay=cfg.decay)),
             "attn": PartSpec("paged_gqa_attention", dict(hidden_size=H, n_heads=2, n_kv_heads=1, head_dim=16,
                                                          position=PartSpec("toy_position_scale", dict(rate=cfg.rate)))),
@@ -339,7 +390,7 @@ def _register_toys():
             # a routed layer norms with the centered norm, the others with the built-in one
             block = PartSpec("prenorm", dict(mixer=mixers[kind], feed_forward=ffns[cfg.ffn_kinds[l]],
                                              norm=centered if routed else norm))
-            local = ["w"] if kind == "decay" else ["q", "k", "v", "o"]
+            local = ["w"] if kind in ("decay", "mean") else ["q", "k", "v", "o"]
             names = {f"mixer.{t}.weight": f"toy.{l}.mix.{t}" for t in local}
             names.update({"mixer_norm.weight": f"toy.{l}.n1", "ffn_norm.weight": f"toy.{l}.n2"})
             if routed:
@@ -381,6 +432,8 @@ def _toy_plain(cfg, w, toks):
                 s = cfg["decay"] * s + a[t]
                 sums.append(s)
             d = np.stack(sums) @ w[f"toy.{l}.mix.w"].T
+        elif cfg["layer_kinds"][l] == "mean":
+            d = np.stack([a[max(0, t - 9):t + 1].mean(axis=0) for t in range(n)]) @ w[f"toy.{l}.mix.w"].T
         else:
             f = (1.0 + cfg["rate"] * np.cos(np.arange(n)))[:, None, None]
             q = (a @ w[f"toy.{l}.mix.q"].T).reshape(n, 2, 16) * f
@@ -409,32 +462,48 @@ def _toy_plain(cfg, w, toks):
     return pm.rmsnorm(x, w["toy.norm"], 1e-5) @ w["toy.head"].T
 
 
-def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
+    """Parts that only this test knows (a mixer with a state per request, a mixer whose pages hold
+    something else than keys and values, a routed feed-forward, another norm, another position
+    encoding), an architecture made of them and of built-in parts, a layer that runs twice: registered,
+    built from a config.json and stepped in every cutting, without a change to the framework's files.
+    In bfloat16 the routed feed-forward stays out: an expert chosen by an argmax over rounded numbers
+    may differ from the plain choice, which says nothing about the framework."""
     import replay_helpers as rh
     from flambeau_amd.engine import ModelRunner, load_model
     from flambeau_amd.weights import write_random_model
     _register_toys()
-    cfg = dict(architectures=["ToyStateLM"], hidden_size=32, vocab_size=90, layer_kinds=["decay", "attn", "decay"],
-               ffn_kinds=["routed", "swiglu", "routed"], decay=0.8, rate=0.3, max_position_embeddings=128)
+    routed = dtype == "float32"
+    cfg = dict(architectures=["ToyStateLM"], hidden_size=32, vocab_size=90, layer_kinds=["decay", "attn", "mean", "decay"],
+               ffn_kinds=["routed" if routed else "swiglu", "swiglu", "swiglu", "routed" if routed else "swiglu"],
+               decay=0.8, rate=0.3, max_position_embeddings=128)
     d = write_random_model(cfg, tmp_path / "toy", seed=4, std=0.15, gain_std=0.05, store_dtype=torch.float32)
-    model, _ = load_model(d, dtype="float32", max_batch_tokens=128)
-    assert [type(b.mixer).__name__ for b in model.blocks] == ["DecaySum", "PagedGQAAttention", "DecaySum"]
-    assert [type(b.ffn).__name__ for b in model.blocks] == ["Routed", "SwiGLU", "Routed"]
-    assert [type(b.ffn_norm).__name__ for b in model.blocks] == ["CenteredNorm", "RMSNorm", "CenteredNorm"]
+    model, _ = load_model(d, dtype=dtype, max_batch_tokens=128)
+    assert [type(b.mixer).__name__ for b in model.blocks] == ["DecaySum", "PagedGQAAttention", "WindowMean", "DecaySum"]
+    if routed:
+        assert [type(b.ffn).__name__ for b in model.blocks] == ["Routed", "SwiGLU", "SwiGLU", "Routed"]
+        assert [type(b.ffn_norm).__name__ for b in model.blocks] == ["CenteredNorm", "RMSNorm", "RMSNorm", "CenteredNorm"]
     runner = ModelRunner(model, n_pages=16, page_size=8, max_slots=3, max_logit_rows=128)
-    assert not runner.decode_graphs                                    # a mixer with state of its own never replays
-    assert len(runner.storage.states) == 2 and len(runner.storage.pools) == 1
+    # a mixer with state of its own never replays a padded graph, and parts that call torch are not recorded
+    assert not runner.decode_graphs and not runner.step_programs
+    # two states; two page pools of different kinds (keys and values; latent rows), each with a table of its own
+    assert len(runner.storage.states) == 2 and len(runner.storage.pools) == 2
     assert runner.storage.pools[0].shape[0] == 1                       # the repeated layer reads, it owns no cache
+    assert runner.storage.pools[1].shape == (1, 16, 8, 32) and [g.window for g in runner.manager.groups] == [0, 10]
     w = {k: v for k, v in pm.read_safetensors(d / "model.safetensors").items()}
+    if dtype == "bfloat16":
+        w = {k: pm.round_bf16(v) if v.ndim == 2 else v for k, v in w.items()}
     reqs = rh.make_requests(90, [30, 17, 41, 9, 25], seed=2)
     ref = {rid: _toy_plain(cfg, w, toks) for rid, toks in reqs.items()}
     for mode, steps in [("whole", rh.trace_whole(reqs)), ("tail", rh.trace_tail(reqs, tail=8)),
                         ("portions", rh.trace_portions(reqs, sizes=(2, 7, 3, 11))),
                         ("mixed", rh.trace_mixed(reqs, seed=1, max_live=3, max_portion=9, decode_tail=4))]:
         got = rh.run_in_process(runner, steps)
-        rh.compare(got, reqs, ref, "float32", f"toy {mode}")
+        rh.compare(got, reqs, ref, dtype, f"toy {mode}")
+    assert not runner.manager.live and runner.manager.free_pages() == [16, 16]
     # slots are zeroed when they are claimed again: a second pass over the same requests agrees
-    rh.compare(rh.run_in_process(runner, rh.trace_mixed(reqs, seed=3, max_live=3)), reqs, ref, "float32", "toy again")
+    rh.compare(rh.run_in_process(runner, rh.trace_mixed(reqs, seed=3, max_live=3)), reqs, ref, dtype, "toy again")
 
 
 def test_unknown_part_names_the_known_ones():
