@@ -459,15 +459,51 @@ extern "C" int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split
     return 0;
 }
 
+// Merge of the parts of the keys (at most 16): out[d] = sum_s part_o[s][d] e^(m_s - m) / sum_s l_s e^(m_s - m),
+// m = max m_s, the sums in rising s.  A thread owns four head dims of one (row, head); a tile's 64 rows
+// x heads x dims are dealt to its blocks in that order, so a wave reads whole rows of the partial
+// outputs side by side.
 __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_o,
                                                                  const float* __restrict__ part_ml,
                                                                  bf16_t* __restrict__ out, const int* __restrict__ tiles,
-                                                                 int nh, int hd, int hdp, int n_split) {
-    const int tile = blockIdx.x / PF_TOKENS, qtok = blockIdx.x % PF_TOKENS, head = blockIdx.y;
+                                                                 int nh, int hd, int hdp, int n_split, int blocks_per_tile) {
+    const int tile = blockIdx.x / blocks_per_tile;
     const int row0 = tiles[4 * tile + 1], cnt = tiles[4 * tile + 2], item0 = tiles[4 * tile + 3];
-    if (qtok >= cnt) return;                                       // (the whole block leaves)
-    attn_merge_splits(part_o, part_ml, out + ((size_t)(row0 + qtok) * nh + head) * hd,
-                      ((size_t)(item0 + qtok) * nh + head) * n_split, hd, hdp, n_split);
+    const int quads = hdp >> 2;
+    const int idx = (blockIdx.x % blocks_per_tile) * 256 + threadIdx.x;       // (row of the tile, head, quad of dims)
+    const int q4 = idx % quads, head = (idx / quads) % nh, qtok = idx / (quads * nh);
+    if (qtok >= cnt) return;
+    const size_t base = ((size_t)(item0 + qtok) * nh + head) * n_split;
+    float ms[16], ls[16];
+    float mm = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        if (s < n_split) {
+            const float2 ml = *(const float2*)(part_ml + (base + s) * 2);
+            ms[s] = ml.x;
+            ls[s] = ml.y;
+            mm = fmaxf(mm, ml.x);
+        }
+    }
+    float ll = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        if (s < n_split) {
+            const float f = ms[s] == -INFINITY ? 0.f : expf(ms[s] - mm);
+            ll += ls[s] * f;
+            acc += *(const f32x4*)(part_o + (base + s) * hdp + 4 * q4) * f;
+        }
+    }
+    const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+    const int d = 4 * q4;
+    bf16_t* orow = out + ((size_t)(row0 + qtok) * nh + head) * hd;
+    if (d + 4 <= hd) {
+        const bf16x4 ov = {(bf16_t)(acc[0] * inv), (bf16_t)(acc[1] * inv), (bf16_t)(acc[2] * inv), (bf16_t)(acc[3] * inv)};
+        *(bf16x4*)(orow + d) = ov;
+    } else {
+        for (int r = 0; r < 4 && d + r < hd; ++r) orow[d + r] = (bf16_t)(acc[r] * inv);
+    }
 }
 
 // tiles[n_tiles][4] = (row of the request in the block table, first row, rows (at most 64), index of
@@ -486,9 +522,10 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     FL_CHECK(max_blocks <= PF_MAX_PAGES, "attn_prefill: %d pages per request, at most %d", max_blocks, PF_MAX_PAGES);
     FL_CHECK(window >= 0, "attn_prefill: negative window");
     FL_CHECK(scale > 0.f, "attn_prefill: the score scale must be positive");
-    FL_CHECK(n_split >= 1 && n_split <= 256, "attn_prefill: %d splits", n_split);
+    FL_CHECK(n_split >= 1 && n_split <= 16, "attn_prefill: %d splits (at most 16)", n_split);
     FL_CHECK(n_split == 1 || (part_o && part_ml && (uintptr_t)part_o % 16 == 0), "attn_prefill: splits need a 16-byte aligned workspace");
-    FL_CHECK(n_tiles <= 65535 / PF_TOKENS || n_split == 1, "attn_prefill: %d tiles are too many to split", n_tiles);
+    FL_CHECK(n_split == 1 || (long long)n_tiles * PF_TOKENS * nh * (ceil_div(hd, 32) * 8) / 256 < (1ll << 31),
+             "attn_prefill: %d tiles are too many to split", n_tiles);
     if (n_tiles == 0) return 0;
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
     const int G = nh / nkv;
@@ -515,8 +552,9 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
 #undef FL_PF
     FL_LAUNCH_CHECK();
     if (n_split > 1) {
-        dim3 mg(n_tiles * PF_TOKENS, nh);
-        attn_prefill_merge_kernel<<<mg, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, tiles, nh, hd, hdp, n_split);
+        const int blocks_per_tile = ceil_div(PF_TOKENS * nh * (hdp / 4), 256);
+        attn_prefill_merge_kernel<<<n_tiles * blocks_per_tile, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, tiles, nh, hd,
+                                                                                 hdp, n_split, blocks_per_tile);
         FL_LAUNCH_CHECK();
     }
     return 0;

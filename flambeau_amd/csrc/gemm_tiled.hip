@@ -542,8 +542,9 @@ extern "C" int fl_gemm_tiled_residual_parts(int M, int N, int K) {
 
 // The joined q/k/v projection of many rows with its rows in paired order: q is rotated and written to
 // q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens' positions; cs[M,
-// rot / 2, 2] are the step's cosines and sines.  Only for shapes whose K is not split
-// (fl_gemm_tiled_splits == 1).  in_ssq as in fl_gemm_tiled_scaled.
+// rot / 2, 2] are the step's cosines and sines.  K is never split here (for shapes whose K the plain
+// product would split, that product followed by the rotation kernel is the faster way).  in_ssq as in
+// fl_gemm_tiled_scaled.
 extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
                                   int in_parts, float eps, const int* positions, const int* tok_seq,
                                   const int* block_table, int max_blocks, const float* cs, void* q_out,
@@ -555,7 +556,6 @@ extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, in
              "gemm_tiled_rope: needs positions, requests, block table, angles, q and the cache");
     FL_CHECK(hd % 16 == 0 && rot % 16 == 0 && rot <= hd && N == (nh + 2 * nkv) * hd,
              "gemm_tiled_rope: %d features with heads of %d (%d rotated), %d + 2 x %d heads", N, hd, rot, nh, nkv);
-    FL_CHECK(fl_gemm_tiled_splits(M, N, K) == 1, "gemm_tiled_rope: this shape splits K");
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0), "gemm_tiled_rope: operands must be 16-byte aligned");
     FL_CHECK(!in_ssq || in_parts > 0, "gemm_tiled_rope: a row scale over %d parts", in_parts);
     if (M == 0) return 0;
