@@ -141,6 +141,39 @@ def run_prefill(model, dtype_name, reps=REPS, seed=1):
     return statistics.median(times)
 
 
+def run_portion(model, dtype_name, portion, ctx_before, reps=REPS, seed=3):
+    """Time of one prompt portion of ``portion`` tokens behind ``ctx_before`` cached ones (the context
+    is filled in portions of 2,048 first); median of ``reps`` portions that follow one another."""
+    import numpy as np
+    import torch
+    from flambeau_amd.engine import ModelRunner, StepEntry
+    rng = np.random.default_rng(seed)
+    V = model.spec.vocab_size
+    total = ctx_before + (reps + 1) * portion
+    runner = ModelRunner(model, n_pages=-(-total // PAGE) + 1, page_size=PAGE, max_slots=1, max_seq_len=total,
+                         max_logit_rows=1)
+    runner.begin("p")
+    ids = lambda n: [int(t) for t in rng.integers(0, V, n)]
+    at = 0
+    while at < ctx_before:
+        k = min(2048, ctx_before - at)
+        runner.step([StepEntry("p", ids(k), [])])
+        at += k
+    times = []
+    for rep in range(reps + 1):
+        toks = ids(portion)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry("p", toks, [portion - 1])])
+        torch.cuda.synchronize()
+        if rep:
+            times.append(time.perf_counter() - t0)
+    runner.end("p")
+    del runner
+    torch.cuda.empty_cache()
+    return statistics.median(times)
+
+
 def run_enqueue(model, dtype_name, rows=64, decoders=16, seed=2):
     """Host time to enqueue one mixed step of ``rows`` rows (a prompt portion beside ``decoders``
     decoding requests): the time ``ModelRunner.step`` takes to return, the device idle before and
@@ -281,7 +314,7 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="run only the first layers (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
-    ap.add_argument("--only", choices=["decode", "prefill", "enqueue"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "enqueue", "portion"], default=None,
                     help="run one part only and print its numbers (for profiling)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -307,6 +340,10 @@ def main():
         return 0
     if a.only == "enqueue":
         print(json.dumps({"enqueue_ms_mixed64": round(run_enqueue(model, dtype_name), 3)}))
+        return 0
+    if a.only == "portion":
+        t = run_portion(model, dtype_name, 512, 7680)
+        print(json.dumps({"portion_ms": round(t * 1e3, 3), "tokens": 512, "context": 7680, "tok_s": round(512 / t, 1)}))
         return 0
     if a.only == "decode":
         a.no_points = True
@@ -346,6 +383,13 @@ def main():
             points[f"decode_b{b}_ms"] = round(dtb / k * 1e3, 4)
             points[f"decode_b{b}_frac"] = round(decode_bytes(sz, b, ctxb, el) / (dtb / k) / PEAK_HBM, 4)
         points["enqueue_ms_mixed64"] = round(run_enqueue(model, dtype_name), 3)
+        # a portion of 512 tokens behind 8k and 32k of context: tokens/s and the fraction of the matrix peak
+        for label, ctx in (("8k", 8192 - 512 * (a.reps + 1)), ("32k", 32768 - 512 * (a.reps + 1))):
+            t = run_portion(model, dtype_name, 512, ctx, reps=a.reps)
+            mid = ctx + 512 * (a.reps + 1) // 2
+            key = f"prefill512_ctx{label}"
+            points[key] = round(512 / t, 1)
+            points[key + "_frac"] = round(prefill_flops(sz, 512, mid) / t / PEAK_FLOPS[a.dtype], 4)
         out["points"] = points
     print(json.dumps(out), flush=True)
     return 0
