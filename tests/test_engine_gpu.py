@@ -430,7 +430,8 @@ def test_cutting_at_real_layer_sizes(wide_model_dir, dtype):
     runner = ModelRunner(model, n_pages=24, page_size=16, max_slots=4, max_logit_rows=512)
     runner.storage.fill(float("nan"))
     ref = rh.plain_logits(wide_model_dir, reqs)
-    for what, steps in (("portions", rh.trace_portions(reqs, sizes=(2, 70, 3, 17, 2, 130, 31, 4))),
+    for what, steps in (("whole", rh.trace_whole(reqs)), ("tail", rh.trace_tail(reqs, tail=12)),
+                        ("portions", rh.trace_portions(reqs, sizes=(2, 70, 3, 17, 2, 130, 31, 4))),
                         ("mixed", rh.trace_mixed(reqs, seed=3, max_portion=90))):
         got = rh.run_in_process(runner, steps)
         assert not runner.manager.live
@@ -459,3 +460,41 @@ def test_short_portions_behind_a_long_context(tmp_path_factory, dtype):
     steps = rh.trace_portions(reqs, sizes=(700, 500, 100, 64, 9, 70, 30, 27))
     got = rh.run_in_process(runner, steps)
     rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, "long context")
+
+
+def test_serving_loop_under_random_pressure(model_dirs):
+    """Random mixes of requests, slots, pages, portion sizes, sampling and stop ids through the serving
+    loop (which runs a step ahead of the host and pre-empts when pages run out): every request's
+    tokens are those it gets alone, whatever happens around it, and no page or slot is lost."""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    from flambeau_amd.engine import load_model
+    n_pre = n_stopped = 0
+    for name, ps in (("A", 8), ("D", 8), ("B", 16)):
+        d = model_dirs[(name, "float32")]
+        vocab = TINY[name]["config"]["vocab_size"]
+        ctx = min(TINY[name]["config"]["max_position_embeddings"], 256)
+        model, _ = load_model(d, dtype="float32", max_batch_tokens=ctx + 8)
+        alone = LLMEngine(model, EngineOptions(dtype="float32", inflight_slots=1, prefill_chunk_tokens=ctx, page_size=ps, ctx_cap=ctx))
+        for case in range(40):
+            rng = np.random.default_rng(1000 * ps + case)
+            n_req = int(rng.integers(3, 8))
+            new = int(rng.integers(4, 30))
+            prompts = [[int(t) for t in rng.integers(0, vocab, int(rng.integers(1, ctx - new - 1)))] for _ in range(n_req)]
+            temp = float(rng.choice([0.0, 0.0, 0.8]))
+            stops = tuple(int(t) for t in rng.integers(0, vocab, int(rng.integers(0, 12))))
+            params = [SamplingParams(max_tokens=new, temperature=temp, seed=100 + i, stop_token_ids=stops) for i in range(n_req)]
+            want = [alone.generate([p], sp)[0] for p, sp in zip(prompts, params)]
+            longest = -(-(max(len(p) for p in prompts) + new) // ps)
+            slots = int(rng.integers(2, 6))
+            pages = longest + int(rng.integers(1, 2 * longest))
+            chunk = int(rng.choice([16, 64, ctx]))
+            eng = LLMEngine(model, EngineOptions(dtype="float32", inflight_slots=slots, prefill_chunk_tokens=chunk, page_size=ps,
+                                                 paged_kv=pages, ctx_cap=ctx, max_batch_tokens=ctx + 8))
+            got = eng.generate(prompts, params)
+            what = f"{name} case {case}: slots {slots}, pages {pages}, portions {chunk}, temperature {temp}, {len(stops)} stop ids"
+            assert got == want, what
+            assert not eng.runner.manager.live and all(f == pages for f in eng.runner.manager.free_pages()), what
+            eng.runner.manager.check_invariants()
+            n_pre += eng.scheduler.n_preemptions
+            n_stopped += sum(len(g) < new for g in got)
+    assert n_pre > 0 and n_stopped > 0          # the cases did pre-empt, and did stop requests early
