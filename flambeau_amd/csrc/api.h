@@ -82,15 +82,21 @@ int fl_reduce_residual(const float* part, float* resid, const float* g, void* xg
 int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_tiled_splits(int M, int N, int K);
-// for tests and measurements: block shape (0 = chosen, 3 = 256 features x 128 tokens, 6 = 128 x 256) and
-// K-splits (0 = chosen) from the caller
+// for tests and measurements: block shape (0 = chosen, 3 = 256 features x 128 tokens, 7 = 192 x 128,
+// 8 = 128 x 128, 6 = 128 x 256 with eight waves) and K-splits (0 = chosen) from the caller
 int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                      int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
                      float eps, int variant, int forced_splits, hipStream_t stream);
 int fl_gemm_tiled_splits_ex(int M, int N, int K, int forced);
+int fl_gemm_tiled_shape(int M, int N, int K, int may_split);
 int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, float* workspace, int M, int N, int K, float* resid,
                               const float* g, void* xg, float* out_ssq, int variant, hipStream_t stream);
-int fl_gemm_tiled_parts_ex(int M, int N, int variant);
+int fl_gemm_tiled_parts_ex(int M, int N, int K, int variant);
+int fl_gemm_tiled_rope_ex(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
+                          int in_parts, float eps, const int* positions, const int* tok_seq,
+                          const int* block_table, int max_blocks, const float* cs, void* q_out, void* cache_base,
+                          int nh, int nkv, int hd, int page_size, int n_pages, int rot, int write_cache, int variant,
+                          hipStream_t stream);
 // The joined q/k/v projection (rows of w in paired order) with rotation and the stores of q and the
 // cache rows in the product's kernel: at most 16 rows, and many rows (shapes whose K is not split).
 int fl_gemm_skinny_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
@@ -110,7 +116,7 @@ int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* out, float* 
                          float eps, hipStream_t stream);
 int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K, float* resid,
                            const float* g, void* xg, float* out_ssq, hipStream_t stream);
-int fl_gemm_tiled_parts(int M, int N);
+int fl_gemm_tiled_parts(int M, int N, int K);
 int fl_gemm_tiled_residual_parts(int M, int N, int K);
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                    const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,

@@ -34,8 +34,6 @@
 #include "api.h"
 #include "rope_store.h"
 
-#define TG_BM 128                        // block tile the split-K rule counts with
-#define TG_BN 128
 #define TG_PLAIN 0                       // epilogues
 #define TG_SWIGLU 1
 #define TG_ROPE 2
@@ -398,43 +396,94 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     out[i] = from_f32<TOut>(s);
 }
 
-// Shape of the block: 0 = chosen from the sizes, 3 = 256 features x 128 tokens (4 waves, ring of 3, two blocks
-// per compute unit), 6 = 128 x 256 (8 waves, ring of 4, one block per compute unit).  The entry points
-// whose names end in _ex take the shape (and the number of K-splits) from the caller, for tests and
-// measurements; the others choose.
-static int tiled_variant(int variant, int splits, int M, int N) {
-    // 256 x 128 where that fills the chip (and for few rows), else 128 x 256
-    if (variant == 3 || variant == 6) return variant;
-    return (ceil_div(N, 256) * ceil_div(M, 128) * splits >= 320 || M < 192) ? 3 : 6;
+// Shape of the block: 3 = 256 features x 128 tokens (4 waves, ring of 3, two blocks per compute unit),
+// 7 = 192 x 128 and 8 = 128 x 128 (the same with fewer features), 6 = 128 x 256 (8 waves, ring of 4, one
+// block per compute unit); 0 = chosen here, together with the number of K-splits.  The entry points
+// whose names end in _ex take either from the caller, for tests and measurements.
+//
+// What a shape costs follows from what bounds the kernel, the copies into LDS: a compute unit takes
+// about 0.1 us per k-step and round of resident blocks plus 17.5 ns per KB that its blocks copy
+// (57 GB/s per unit, whatever the shape and however many blocks share the unit).  So the time of a
+// product is that of the units' load, taken half from the mean and half from the unit with the
+// most blocks; splitting K adds the parts' way to memory and back and the kernel that sums them.
+// Fitted on the 7B and 24B shapes at 128 to 2,048 rows with cold weights, it picks within 1 % of
+// the best measured shape and split on average (14 % off at worst, a long K at 1,024 rows).
+struct TileShape { int variant, features, tokens, per_unit; };
+static const TileShape g_shapes[] = {{3, 256, 128, 2}, {7, 192, 128, 2}, {8, 128, 128, 2}, {6, 128, 256, 1}};
+static const TileShape& tile_shape(int variant) {
+    for (const TileShape& t : g_shapes)
+        if (t.variant == variant) return t;
+    return g_shapes[0];
+}
+static bool tiled_known(int variant) { return variant == 0 || tile_shape(variant).variant == variant; }
+
+static float tiled_cost(const TileShape& t, int splits, int M, int N, int K) {
+    const int units = 256;
+    const int steps = ceil_div(ceil_div(K, 32), splits);
+    const long blocks = (long)ceil_div(N, t.features) * ceil_div(M, t.tokens) * splits;
+    const long most = (blocks + units - 1) / units;                    // blocks of the unit with the most
+    const long rounds = (most + t.per_unit - 1) / t.per_unit;
+    const float mean = blocks > units ? (float)blocks / units : 1.f;
+    const float kb = (t.features + t.tokens) * 64 / 1024.f;            // copied per block and k-step
+    float us = steps * (0.10f * rounds + 0.0175f * kb * 0.5f * (mean + most)) + 3.f;
+    if (splits > 1) us += 3.f + (float)M * N * 4.f * (2 * splits + 1) / 4.5e6f;
+    return us;
+}
+
+struct TilePlan { int variant, splits; };
+// forced_variant / forced_splits: 0 = free; may_split: the epilogue allows parts of K.  The number of
+// splits never depends on a forced shape (a caller sizes the workspace from the sizes alone).
+static TilePlan tiled_plan(int M, int N, int K, bool may_split, int forced_variant, int forced_splits) {
+    const int steps = ceil_div(K, 32);
+    int splits = 1;
+    if (forced_splits > 0) {
+        splits = max(1, min(forced_splits, steps / 8));
+    } else if (may_split) {
+        float best_us = 0.f;
+        for (const TileShape& t : g_shapes) {
+            if (t.variant == 6) continue;                              // (the 8-wave shape only on request)
+            for (int s = 1; s <= 16 && (s == 1 || steps / s >= 8); s *= 2) {
+                const float us = tiled_cost(t, s, M, N, K);
+                if (best_us == 0.f || us < best_us * 0.999f) { best_us = us; splits = s; }
+            }
+        }
+    }
+    if (forced_variant) return {forced_variant, splits};
+    TilePlan best = {3, splits};
+    float best_us = 0.f;
+    for (const TileShape& t : g_shapes) {
+        if (t.variant == 6) continue;
+        const float us = tiled_cost(t, splits, M, N, K);
+        if (best_us == 0.f || us < best_us * 0.999f) { best_us = us; best.variant = t.variant; }
+    }
+    return best;
 }
 
 // Parts in which the residual epilogue leaves a token's sum of squares: one per tile of features.
-extern "C" int fl_gemm_tiled_parts_ex(int M, int N, int variant) {
-    return ceil_div(N, tiled_variant(variant, 1, M, N) == 6 ? 128 : 256);
+extern "C" int fl_gemm_tiled_parts_ex(int M, int N, int K, int variant) {
+    return ceil_div(N, tile_shape(tiled_plan(M, N, K, false, variant, 0).variant).features);
 }
-extern "C" int fl_gemm_tiled_parts(int M, int N) { return fl_gemm_tiled_parts_ex(M, N, 0); }
+extern "C" int fl_gemm_tiled_parts(int M, int N, int K) { return fl_gemm_tiled_parts_ex(M, N, K, 0); }
 
 template <typename TOut, int EPI>
 static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16_t* x, const bf16_t* wp, TOut* out,
                          int M, int N, int K, int n_steps, int per, int out_cols, const RopeStore& rs,
                          const TiledFusion& fu = TiledFusion{}) {
-    if (tiled_variant(variant, splits, M, N) == 6)
-        launch_async<4, 4, 4, 4, 1, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu);
-    else
-        launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu);
+    switch (variant) {                                 // (decided by tiled_plan)
+        case 6: launch_async<4, 4, 4, 4, 1, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
+        case 7: launch_async<6, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
+        case 8: launch_async<4, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
+        default: launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
+    }
 }
 
-// How many ways K is split for a product of this shape: 1 if the grid fills the chip (forced > 0: that
-// many, as far as K allows).
+// How many ways K is split for a product of this shape (forced > 0: that many, as far as K allows).
 extern "C" int fl_gemm_tiled_splits_ex(int M, int N, int K, int forced) {
-    if (forced > 0) return max(1, min(forced, ceil_div(K, 32) / 8));
-    const int blocks = ceil_div(M, TG_BM) * ceil_div(N, TG_BN);
-    const int steps = ceil_div(K, 32);
-    int splits = 1;
-    while (blocks * splits < 288 && splits < 16 && steps / (splits * 2) >= 8) splits *= 2;          // (288: measured on the 7B shapes, 65 to 1,536 rows)
-    return splits;
+    return tiled_plan(M, N, K, true, 0, forced).splits;
 }
 extern "C" int fl_gemm_tiled_splits(int M, int N, int K) { return fl_gemm_tiled_splits_ex(M, N, K, 0); }
+// The block shape chosen for a product of this shape (may_split = 0: an epilogue that takes whole sums only).
+extern "C" int fl_gemm_tiled_shape(int M, int N, int K, int may_split) { return tiled_plan(M, N, K, may_split != 0, 0, 0).variant; }
 
 // epilogue 0: out[M, N] = x w^T.  epilogue 1 (SwiGLU): out[M, out_cols] = silu(gate) * up from the
 // N interleaved gate/up rows of w (K is not split then).  in_ssq (or null): [M, in_parts] partial sums of
@@ -454,13 +503,13 @@ extern "C" int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, 
     FL_CHECK(!in_ssq || in_parts > 0, "gemm_tiled: a row scale over %d parts", in_parts);
     if (M == 0) return 0;
     const int n_steps = ceil_div(K, 32);
-    FL_CHECK(variant == 0 || variant == 3 || variant == 6, "gemm_tiled: block shape %d (0, 3 or 6)", variant);
-    const int splits = epilogue ? 1 : fl_gemm_tiled_splits_ex(M, N, K, forced_splits);
+    FL_CHECK(tiled_known(variant), "gemm_tiled: block shape %d (0, 3, 6, 7 or 8)", variant);
+    const TilePlan plan = tiled_plan(M, N, K, !epilogue, variant, epilogue ? 1 : forced_splits);
+    const int splits = plan.splits, v = plan.variant;
     FL_CHECK(splits == 1 || workspace, "gemm_tiled: this shape splits K %d ways and needs a workspace", splits);
     const int per = ceil_div(n_steps, splits);
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
-    const int v = variant;
     const RopeStore none{};
     const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
     if (epilogue) {
@@ -506,7 +555,7 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
 extern "C" int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
                                          float* resid, const float* g, void* xg, float* out_ssq, int variant,
                                          hipStream_t stream) {
-    FL_CHECK(variant == 0 || variant == 3 || variant == 6, "gemm_tiled_residual: block shape %d (0, 3 or 6)", variant);
+    FL_CHECK(tiled_known(variant), "gemm_tiled_residual: block shape %d (0, 3, 6, 7 or 8)", variant);
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_residual: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled_residual: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(N % 4 == 0, "gemm_tiled_residual: N=%d is no multiple of 4 (16-byte accesses to the residual rows)", N);
@@ -515,16 +564,17 @@ extern "C" int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, fl
              ((uintptr_t)g % 16 == 0) && ((uintptr_t)xg % 8 == 0), "gemm_tiled_residual: operands must be aligned (16 bytes, xg 8)");
     if (M == 0) return 0;
     const int n_steps = ceil_div(K, 32);
-    const int splits = fl_gemm_tiled_splits(M, N, K);
+    const TilePlan plan = tiled_plan(M, N, K, true, variant, 0);
+    const int splits = plan.splits;
     if (splits > 1) {
         FL_CHECK(workspace && (uintptr_t)workspace % 16 == 0, "gemm_tiled_residual: this shape splits K %d ways and needs a workspace", splits);
-        launch_tiled<float, TG_PLAIN>(variant, splits, stream, (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
+        launch_tiled<float, TG_PLAIN>(plan.variant, splits, stream, (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
                                       n_steps, ceil_div(n_steps, splits), N, RopeStore{});
         FL_LAUNCH_CHECK();
         return fl_reduce_residual(workspace, resid, g, xg, out_ssq, M, N, splits, stream);
     }
     const TiledFusion fu = {nullptr, 0, 0.f, resid, g, (bf16_t*)xg, out_ssq};
-    launch_tiled<float, TG_RESIDUAL>(variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, resid, M, N, K,
+    launch_tiled<float, TG_RESIDUAL>(plan.variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, resid, M, N, K,
                                      n_steps, n_steps, N, RopeStore{}, fu);
     FL_LAUNCH_CHECK();
     return 0;
@@ -537,7 +587,7 @@ extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, float
 
 // Parts in which fl_gemm_tiled_residual leaves a token's sum of squares.
 extern "C" int fl_gemm_tiled_residual_parts(int M, int N, int K) {
-    return fl_gemm_tiled_splits(M, N, K) > 1 ? fl_gemm_mid_parts(N) : fl_gemm_tiled_parts(M, N);
+    return fl_gemm_tiled_splits(M, N, K) > 1 ? fl_gemm_mid_parts(N) : fl_gemm_tiled_parts(M, N, K);
 }
 
 // The joined q/k/v projection of many rows with its rows in paired order: q is rotated and written to
@@ -545,11 +595,12 @@ extern "C" int fl_gemm_tiled_residual_parts(int M, int N, int K) {
 // rot / 2, 2] are the step's cosines and sines.  K is never split here (for shapes whose K the plain
 // product would split, that product followed by the rotation kernel is the faster way).  in_ssq as in
 // fl_gemm_tiled_scaled.
-extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
-                                  int in_parts, float eps, const int* positions, const int* tok_seq,
-                                  const int* block_table, int max_blocks, const float* cs, void* q_out,
-                                  void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages, int rot,
-                                  int write_cache, hipStream_t stream) {
+extern "C" int fl_gemm_tiled_rope_ex(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
+                                     int in_parts, float eps, const int* positions, const int* tok_seq,
+                                     const int* block_table, int max_blocks, const float* cs, void* q_out,
+                                     void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages, int rot,
+                                     int write_cache, int variant, hipStream_t stream) {
+    FL_CHECK(tiled_known(variant), "gemm_tiled_rope: block shape %d (0, 3, 6, 7 or 8)", variant);
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_rope: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled_rope: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(positions && tok_seq && block_table && cs && q_out && cache_base,
@@ -563,8 +614,17 @@ extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, in
                           PagedCache{cache_base, nkv, page_size, hd, n_pages}, nh, rot, write_cache};
     const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
     const int n_steps = ceil_div(K, 32);
-    launch_tiled<bf16_t, TG_ROPE>(0, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)q_out,
+    launch_tiled<bf16_t, TG_ROPE>(tiled_plan(M, N, K, false, variant, 0).variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, (bf16_t*)q_out,
                                   M, N, K, n_steps, n_steps, N, rs, fu);
     FL_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
+                                  int in_parts, float eps, const int* positions, const int* tok_seq,
+                                  const int* block_table, int max_blocks, const float* cs, void* q_out,
+                                  void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages, int rot,
+                                  int write_cache, hipStream_t stream) {
+    return fl_gemm_tiled_rope_ex(x, w_packed, M, N, K, in_ssq, in_parts, eps, positions, tok_seq, block_table, max_blocks, cs,
+                                 q_out, cache_base, nh, nkv, hd, page_size, n_pages, rot, write_cache, 0, stream);
 }

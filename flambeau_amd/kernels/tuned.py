@@ -20,9 +20,10 @@ register_signatures({
     "fl_gemm_skinny_scale_parts": [I, I, I],
     "fl_gemm_skinny_rope": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
     "fl_gemm_tiled_rope": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
+    "fl_gemm_tiled_rope_ex": [P, P, I, I, I, P, I, F, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, P],
     "fl_gemm_tiled_scaled": [P, P, P, P, I, I, I, I, I, I, P, I, F, P],
     "fl_gemm_tiled_residual": [P, P, P, I, I, I, P, P, P, P, P],
-    "fl_gemm_tiled_parts": [I, I],
+    "fl_gemm_tiled_parts": [I, I, I],
     "fl_gemm_tiled_residual_parts": [I, I, I],
     "fl_gemm_mid": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_mid_splits": [I, I, I],
@@ -35,6 +36,7 @@ register_signatures({
     "fl_gemm_tiled_residual_ex": [P, P, P, I, I, I, P, P, P, P, I, P],
     "fl_gemm_tiled": [P, P, P, P, I, I, I, I, I, I, P],
     "fl_gemm_tiled_splits": [I, I, I],
+    "fl_gemm_tiled_shape": [I, I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, P, I, P],
     "fl_attn_prefill_splits": [I, I, I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
@@ -199,14 +201,18 @@ def gemm_rope_store(x, w: Weight, store: RopeStore, rt=None) -> bool:
     return False
 
 
-def gemm_tiled_rope(x, w_packed, n_features: int, store: RopeStore, row_scale: NormedRows | None = None):
-    """``gemm_skinny_rope`` for many rows (shapes whose K is not split)."""
+def gemm_tiled_rope(x, w_packed, n_features: int, store: RopeStore, row_scale: NormedRows | None = None, variant: int = 0):
+    """``gemm_skinny_rope`` for many rows (shapes whose K is not split); ``variant`` as in ``gemm_tiled``."""
     M, K = x.shape
     if w_packed.numel() != _packed_size(n_features, K):
         raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{n_features}, {K}] matrix packs to {_packed_size(n_features, K)}")
     ssq, parts, eps = _row_scale_args(row_scale, M, K)
-    call("fl_gemm_tiled_rope", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         M, n_features, K, ssq, parts, eps, *_rope_args(store, M, n_features), stream_handle())
+    args = (_check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+            M, n_features, K, ssq, parts, eps, *_rope_args(store, M, n_features))
+    if variant:
+        call("fl_gemm_tiled_rope_ex", *args, int(variant), stream_handle())
+    else:
+        call("fl_gemm_tiled_rope", *args, stream_handle())
     return store.q_out
 
 
@@ -289,8 +295,8 @@ def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale
     """``out = x @ w.T`` for many rows of x.  A shape whose grid would not fill the chip splits K
     and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values).  With
     ``swiglu_rows`` and ``row_scale`` see ``gemm_skinny``.  ``variant`` (block shape: 3 = 256 features x
-    128 tokens, 6 = 128 x 256) and ``splits`` fix what the kernel would choose (for tests and
-    measurements)."""
+    128 tokens, 7 = 192 x 128, 8 = 128 x 128, 6 = 128 x 256) and ``splits`` fix what the kernel would
+    choose (for tests and measurements)."""
     M, K = x.shape
     N = swiglu_rows or out.shape[1]
     if w_packed.numel() != _packed_size(N, K):
@@ -314,7 +320,7 @@ def tiled_parts(M: int, n_features: int, K: int, variant: int = 0) -> int:
     """Parts in which ``gemm_tiled_residual`` leaves the sums of squares of its N features."""
     from .library import load
     if variant and gemm_tiled_splits(M, n_features, K) == 1:
-        return load().fl_gemm_tiled_parts_ex(M, n_features, variant)
+        return load().fl_gemm_tiled_parts_ex(M, n_features, K, variant)
     return load().fl_gemm_tiled_residual_parts(M, n_features, K)
 
 

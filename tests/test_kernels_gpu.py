@@ -473,11 +473,12 @@ def test_gemm_tiled_against_plain(out_dtype, M, N, K):
     assert (got.double() - ref).abs().max() < tol * scale
 
 
-@pytest.mark.parametrize("variant", [3, 6])
+@pytest.mark.parametrize("variant", [3, 6, 7, 8])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 72), (129, 264, 96), (1100, 640, 256)])
 def test_gemm_tiled_block_shapes(variant, M, N, K):
-    """Both block shapes of the tiled product (256 x 128 and 128 x 256), whichever the sizes would
-    choose, through the plain epilogue, the row scale and the add-to-the-stream epilogue."""
+    """Every block shape of the tiled product (256 x 128, 192 x 128, 128 x 128 and 128 x 256 features x
+    tokens), whichever the sizes would choose, through the plain epilogue, SwiGLU, the row scale and
+    the add-to-the-stream epilogue."""
     from flambeau_amd.kernels.library import load
     from flambeau_amd.kernels.packing import pack_weight
     x, w = rnd(M, K, dtype=torch.bfloat16, seed=23), rnd(N, K, dtype=torch.bfloat16, seed=24, scale=0.05)
@@ -494,6 +495,13 @@ def test_gemm_tiled_block_shapes(variant, M, N, K):
     got3 = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
     tuned().gemm_tiled(x, pack_weight(w), got3, ws3, variant=variant, splits=3)
     assert (got3.double() - ref).abs().max() < 1e-5 * ref.abs().max()
+    # gate and up rows interleaved in fours, activation in the epilogue
+    inter = N // 2
+    Wgu = tuned().prepare_gate_up(w[:inter].contiguous(), w[inter:2 * inter].contiguous())
+    act = torch.full((M, inter), float("nan"), dtype=torch.float32, device=DEV)
+    tuned().gemm_tiled(x, Wgu.packed, act, swiglu_rows=Wgu.packed_rows, variant=variant)
+    want_act = torch.nn.functional.silu(ref[:, :inter]) * ref[:, inter:2 * inter]
+    assert (act.double() - want_act).abs().max() < 2e-5 * want_act.abs().max()
     if splits == 1:
         resid = resid0.clone()
         xg = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
@@ -618,6 +626,14 @@ def test_gemm_with_rotation_and_stores_in_its_kernel(M, nh, nkv, hd, rot, ps, H)
     assert (q_a.float() - q_b.float()).abs().max() <= 2e-2 * top
     assert (cache_a.pool.float() - cache_b.pool.float()).abs().max() <= 2e-2 * cache_a.pool.float().abs().max()
     assert ((cache_a.pool != 0) == (cache_b.pool != 0)).all()          # the same places were written
+    if M > 64:
+        # every block shape of the tiled product writes the same
+        for variant in (3, 6, 7, 8):
+            cache_v = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
+            q_v = torch.full((M, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+            store_v = tuned().RopeStore(pos_d, seq_d, table, angles, q_v, cache_v, nh, rot, True)
+            tuned().gemm_tiled_rope(x, W.packed, N, store_v, variant=variant)
+            assert torch.equal(q_v, q_b) and torch.equal(cache_v.pool, cache_b.pool), variant
     # float64 reference of q
     ref = (x.double() @ w.double().T)[:, :nh * hd].reshape(M, nh, hd)
     ref = rope_ref(ref, pos_d, theta, rot)
