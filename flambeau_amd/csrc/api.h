@@ -83,7 +83,7 @@ int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspa
                   int M, int N, int K, int epilogue, int out_cols, hipStream_t stream);
 int fl_gemm_tiled_splits(int M, int N, int K);
 // for tests and measurements: block shape (0 = chosen, 3 = 256 features x 128 tokens, 7 = 192 x 128,
-// 8 = 128 x 128, 6 = 128 x 256 with eight waves) and K-splits (0 = chosen) from the caller
+// 8 = 128 x 128; with eight waves 10 = 256 x 256, 6 = 128 x 256) and K-splits (0 = chosen) from the caller
 int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                      int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
                      float eps, int variant, int forced_splits, hipStream_t stream);

@@ -161,9 +161,9 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
     };
 
     // One block per CU has nothing that runs beside its epilogue, so the residual epilogue's reads
-    // are issued here, ahead of all other loads, and wait in registers (there is room: half the
-    // registers of the CU belong to each wave).
-    constexpr bool PREFETCH = EPI == TG_RESIDUAL && OCC == 1;
+    // are issued here, ahead of all other loads, and wait in registers (where there is room: with 4 x 4
+    // tiles per wave, not with 8 x 4).
+    constexpr bool PREFETCH = EPI == TG_RESIDUAL && OCC == 1 && FT * TT <= 16;
     const int j = lane & 15, g = lane >> 4;
     f32x4 pre[PREFETCH ? FT : 1][PREFETCH ? TT : 1];
     if (PREFETCH) {
@@ -397,19 +397,24 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 }
 
 // Shape of the block: 3 = 256 features x 128 tokens (4 waves, ring of 3, two blocks per compute unit),
-// 7 = 192 x 128 and 8 = 128 x 128 (the same with fewer features), 6 = 128 x 256 (8 waves, ring of 4, one
-// block per compute unit); 0 = chosen here, together with the number of K-splits.  The entry points
-// whose names end in _ex take either from the caller, for tests and measurements.
+// 7 = 192 x 128 and 8 = 128 x 128 (the same with fewer features), 10 = 256 x 256 (8 waves, ring of 4, one
+// block per compute unit), 6 = 128 x 256 (the same with fewer features); 0 = chosen here, together
+// with the number of K-splits.  The entry points whose names end in _ex take either from the caller, for
+// tests and measurements.
 //
 // What a shape costs follows from what bounds the kernel, the copies into LDS: a compute unit takes
 // about 0.1 us per k-step and round of resident blocks plus 17.5 ns per KB that its blocks copy
 // (57 GB/s per unit, whatever the shape and however many blocks share the unit).  So the time of a
 // product is that of the units' load, taken half from the mean and half from the unit with the
 // most blocks; splitting K adds the parts' way to memory and back and the kernel that sums them.
-// Fitted on the 7B and 24B shapes at 128 to 2,048 rows with cold weights, it picks within 1 % of
-// the best measured shape and split on average (14 % off at worst, a long K at 1,024 rows).
+// A 256 x 256 block copies a third less per product and is bound by the matrix cores as much as by
+// the copies: 0.80 us per k-step, and 8 us per block that nothing overlaps.  It wins where its few
+// blocks still load the units evenly (large products: 10 to 20 % at the 24B feed-forward, 12 to 15 %
+// at 7B o/down and 4,096 rows, and the 7B down product at 2,048 rows with K in two parts).
+// Fitted on the 7B and 24B shapes at 128 to 4,096 rows with cold weights, the formula picks within
+// 1 % of the best measured shape and split on average (14 % off at worst, a long K at 1,024 rows).
 struct TileShape { int variant, features, tokens, per_unit; };
-static const TileShape g_shapes[] = {{3, 256, 128, 2}, {7, 192, 128, 2}, {8, 128, 128, 2}, {6, 128, 256, 1}};
+static const TileShape g_shapes[] = {{3, 256, 128, 2}, {7, 192, 128, 2}, {8, 128, 128, 2}, {10, 256, 256, 1}, {6, 128, 256, 1}};
 static const TileShape& tile_shape(int variant) {
     for (const TileShape& t : g_shapes)
         if (t.variant == variant) return t;
@@ -425,7 +430,9 @@ static float tiled_cost(const TileShape& t, int splits, int M, int N, int K) {
     const long rounds = (most + t.per_unit - 1) / t.per_unit;
     const float mean = blocks > units ? (float)blocks / units : 1.f;
     const float kb = (t.features + t.tokens) * 64 / 1024.f;            // copied per block and k-step
-    float us = steps * (0.10f * rounds + 0.0175f * kb * 0.5f * (mean + most)) + 3.f;
+    float us;
+    if (t.variant == 10) us = most * (steps * 0.80f + 8.f) + 3.f;               // eight waves, a unit to itself: one block after the other
+    else us = steps * (0.10f * rounds + 0.0175f * kb * 0.5f * (mean + most)) + 3.f;
     if (splits > 1) us += 3.f + (float)M * N * 4.f * (2 * splits + 1) / 4.5e6f;
     return us;
 }
@@ -441,7 +448,7 @@ static TilePlan tiled_plan(int M, int N, int K, bool may_split, int forced_varia
     } else if (may_split) {
         float best_us = 0.f;
         for (const TileShape& t : g_shapes) {
-            if (t.variant == 6) continue;                              // (the 8-wave shape only on request)
+            if (t.variant == 6) continue;                              // (128 x 256 only on request)
             for (int s = 1; s <= 16 && (s == 1 || steps / s >= 8); s *= 2) {
                 const float us = tiled_cost(t, s, M, N, K);
                 if (best_us == 0.f || us < best_us * 0.999f) { best_us = us; splits = s; }
@@ -473,6 +480,7 @@ static void launch_tiled(int variant, int splits, hipStream_t stream, const bf16
         case 6: launch_async<4, 4, 4, 4, 1, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
         case 7: launch_async<6, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
         case 8: launch_async<4, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
+        case 10: launch_async<8, 4, 4, 4, 1, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
         default: launch_async<8, 4, 2, 3, 2, TOut, EPI>(splits, stream, x, wp, out, M, N, K, n_steps, per, out_cols, rs, fu); break;
     }
 }
@@ -503,7 +511,7 @@ extern "C" int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, 
     FL_CHECK(!in_ssq || in_parts > 0, "gemm_tiled: a row scale over %d parts", in_parts);
     if (M == 0) return 0;
     const int n_steps = ceil_div(K, 32);
-    FL_CHECK(tiled_known(variant), "gemm_tiled: block shape %d (0, 3, 6, 7 or 8)", variant);
+    FL_CHECK(tiled_known(variant), "gemm_tiled: block shape %d (0, 3, 6, 7, 8 or 10)", variant);
     const TilePlan plan = tiled_plan(M, N, K, !epilogue, variant, epilogue ? 1 : forced_splits);
     const int splits = plan.splits, v = plan.variant;
     FL_CHECK(splits == 1 || workspace, "gemm_tiled: this shape splits K %d ways and needs a workspace", splits);
@@ -555,7 +563,7 @@ extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, flo
 extern "C" int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
                                          float* resid, const float* g, void* xg, float* out_ssq, int variant,
                                          hipStream_t stream) {
-    FL_CHECK(tiled_known(variant), "gemm_tiled_residual: block shape %d (0, 3, 6, 7 or 8)", variant);
+    FL_CHECK(tiled_known(variant), "gemm_tiled_residual: block shape %d (0, 3, 6, 7, 8 or 10)", variant);
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_residual: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled_residual: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(N % 4 == 0, "gemm_tiled_residual: N=%d is no multiple of 4 (16-byte accesses to the residual rows)", N);
@@ -600,7 +608,7 @@ extern "C" int fl_gemm_tiled_rope_ex(const void* x, const void* w_packed, int M,
                                      const int* block_table, int max_blocks, const float* cs, void* q_out,
                                      void* cache_base, int nh, int nkv, int hd, int page_size, int n_pages, int rot,
                                      int write_cache, int variant, hipStream_t stream) {
-    FL_CHECK(tiled_known(variant), "gemm_tiled_rope: block shape %d (0, 3, 6, 7 or 8)", variant);
+    FL_CHECK(tiled_known(variant), "gemm_tiled_rope: block shape %d (0, 3, 6, 7, 8 or 10)", variant);
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_rope: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled_rope: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(positions && tok_seq && block_table && cs && q_out && cache_base,

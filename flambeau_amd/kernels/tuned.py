@@ -295,7 +295,7 @@ def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale
     """``out = x @ w.T`` for many rows of x.  A shape whose grid would not fill the chip splits K
     and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values).  With
     ``swiglu_rows`` and ``row_scale`` see ``gemm_skinny``.  ``variant`` (block shape: 3 = 256 features x
-    128 tokens, 7 = 192 x 128, 8 = 128 x 128, 6 = 128 x 256) and ``splits`` fix what the kernel would
+    128 tokens, 7 = 192 x 128, 8 = 128 x 128, 10 = 256 x 256, 6 = 128 x 256) and ``splits`` fix what the kernel would
     choose (for tests and measurements)."""
     M, K = x.shape
     N = swiglu_rows or out.shape[1]

@@ -473,11 +473,11 @@ def test_gemm_tiled_against_plain(out_dtype, M, N, K):
     assert (got.double() - ref).abs().max() < tol * scale
 
 
-@pytest.mark.parametrize("variant", [3, 6, 7, 8])
+@pytest.mark.parametrize("variant", [3, 6, 7, 8, 10])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 72), (129, 264, 96), (1100, 640, 256)])
 def test_gemm_tiled_block_shapes(variant, M, N, K):
-    """Every block shape of the tiled product (256 x 128, 192 x 128, 128 x 128 and 128 x 256 features x
-    tokens), whichever the sizes would choose, through the plain epilogue, SwiGLU, the row scale and
+    """Every block shape of the tiled product (256 x 128, 192 x 128, 128 x 128, 256 x 256 and 128 x 256
+    features x tokens), whichever the sizes would choose, through the plain epilogue, SwiGLU, the row scale and
     the add-to-the-stream epilogue."""
     from flambeau_amd.kernels.library import load
     from flambeau_amd.kernels.packing import pack_weight
@@ -628,7 +628,7 @@ def test_gemm_with_rotation_and_stores_in_its_kernel(M, nh, nkv, hd, rot, ps, H)
     assert ((cache_a.pool != 0) == (cache_b.pool != 0)).all()          # the same places were written
     if M > 64:
         # every block shape of the tiled product writes the same
-        for variant in (3, 6, 7, 8):
+        for variant in (3, 6, 7, 8, 10):
             cache_v = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
             q_v = torch.full((M, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
             store_v = tuned().RopeStore(pos_d, seq_d, table, angles, q_v, cache_v, nh, rot, True)
