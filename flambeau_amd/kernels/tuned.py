@@ -216,6 +216,34 @@ def gemm_tiled_rope(x, w_packed, n_features: int, store: RopeStore, row_scale: N
     return store.q_out
 
 
+def gemm_add_norm(rt, x, w: Weight, resid, norm_weight, eps: float):
+    """``resid += x @ w.T`` with the norm that follows left in factors (``NormedRows``: ``resid * g`` in
+    the compute dtype and the sums of squares in parts), by the product's own kernel or the kernel that
+    adds its K-splits; ``None`` where no kernel takes the shape (the caller then runs product, addition
+    and norm apart).  All shape rules of these kernels live here."""
+    n, H = resid.shape
+    if (w.packed is None or w.swiglu_cols or isinstance(x, NormedRows) or x.dtype != torch.bfloat16
+            or x.shape[1] % 8 or H % 8):
+        return None
+    K = x.shape[1]
+    xg = rt.buffer("normed_xg", n, H)
+    if n <= FUSED_NORM_MAX_ROWS:
+        ssq = rt.buffer("normed_ssq", n, skinny_parts(H), torch.float32)
+        return gemm_skinny_residual(x, w.packed, resid, norm_weight, xg, ssq, eps)
+    if n <= SKINNY_MAX_ROWS and K % 32 == 0 and H % 32 == 0:
+        # 17 to 64 rows: the kernel that adds the K-splits of the product does it
+        ssq = rt.buffer("normed_ssq_mid", n, mid_parts(H), torch.float32)
+        workspace = _split_workspace(rt, gemm_mid_splits(n, H, K) * n * H, x.device)
+        return gemm_mid_residual(x, w.packed, resid, norm_weight, xg, ssq, eps, workspace)
+    if n > SKINNY_MAX_ROWS and H % 4 == 0:
+        # many rows (a prompt portion): the tiled product's epilogue does it, or the kernel that adds its K-splits
+        ssq = rt.buffer("normed_ssq_tiled", n, tiled_parts(n, H, K), torch.float32)
+        splits = gemm_tiled_splits(n, H, K)
+        workspace = _split_workspace(rt, splits * n * H, x.device) if splits > 1 else None
+        return gemm_tiled_residual(x, w.packed, resid, norm_weight, xg, ssq, eps, workspace)
+    return None
+
+
 def gemm_mid_splits(M: int, N: int, K: int, waves: int = 0, splits: int = 0) -> int:
     from .library import load
     return load().fl_gemm_mid_splits_ex(M, N, K, waves, splits)

@@ -50,8 +50,7 @@ class PagedGQAAttention(Mixer):
     def step_signature(self, batch):
         """Into how many parts the kernels split the keys: all that this mixer decides from the
         contexts' lengths."""
-        from ..kernels import tuned
-        return tuned.attention_splits(batch, self.n_heads, self.n_kv_heads, self.head_dim, self.window)
+        return self.rt.attention_splits(batch, self.n_heads, self.n_kv_heads, self.head_dim, self.window)
 
     def tensors(self):
         H, qw, kvw = self.hidden_size, self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
@@ -66,14 +65,11 @@ class PagedGQAAttention(Mixer):
     def bind(self, weights, rt):
         self.rt = rt
         w_qkv = torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0)
-        # With the tuned kernels the rows of a rotated projection are put in an order in which the
+        # Where the runtime's kernels want it, the rows of a rotated projection are put in an order in which the
         # product's own kernel can rotate (8 dims, their 8 partners, ...); the rotation kernel reads
         # that order too.
         rotary = self.position.rotary_parameters()
-        order = None
-        if rt.tuned and rotary is not None and rotary[0]:
-            from ..kernels.packing import rotary_paired_rows
-            order = rotary_paired_rows(self.n_heads, self.n_kv_heads, self.head_dim, rotary[0])
+        order = rt.rotary_row_order(self.n_heads, self.n_kv_heads, self.head_dim, rotary[0]) if rotary is not None else None
         self.paired = order is not None
         if self.paired:
             w_qkv = w_qkv[order.to(w_qkv.device)]
@@ -90,9 +86,7 @@ class PagedGQAAttention(Mixer):
         q = rt.buffer("attn_q", n, nh * hd)
         fused = False
         if self.paired and angles is not None:
-            from ..kernels.tuned import RopeStore
-            fused = rt.gemm_rope_store(x, self.w_qkv, RopeStore(step.positions, step.tok_seq, table, angles, q, cache.kv,
-                                                                nh, rotary[0], cache.writes))
+            fused = rt.gemm_rope_store(x, self.w_qkv, step, table, angles, q, cache.kv, nh, rotary[0], cache.writes)
         if not fused:
             qkv = rt.buffer("attn_qkv", n, (nh + 2 * nkv) * hd, torch.float32)
             rt.gemm(x, self.w_qkv, qkv)
@@ -102,9 +96,5 @@ class PagedGQAAttention(Mixer):
             ops.rope_kv_write(qkv, step.positions, step.tok_seq, table, q, cache.kv, nh, rotary[0], rotary[1],
                               write_cache=cache.writes, table=angles, paired=self.paired)
         out = rt.buffer("attn_out", n, nh * hd)
-        if rt.tuned:
-            from ..kernels import tuned
-            tuned.attention(rt, q, out, cache.kv, step, table, nh, self.scale, self.window)
-        else:
-            ops.attn_plain(q, out, cache.kv, step.positions, step.tok_seq, table, nh, self.scale, self.window)
+        rt.attention(q, out, cache.kv, step, table, nh, self.scale, self.window)
         return Product(out, self.w_o)

@@ -3,8 +3,6 @@
 pending delta to the residual stream follows rmsnorm_f16_add_residual.cu."""
 from __future__ import annotations
 
-import torch
-
 from ..kernels import ops
 from .base import NORMS, Norm, TensorSpec
 
@@ -31,28 +29,4 @@ class RMSNorm(Norm):
         """Where a kernel for the shape exists the product's kernel adds its result to the stream and
         leaves the norm in factors: x * w in the compute dtype and the sums of squares in parts.
         The product that follows multiplies by rsqrt(mean + eps) itself: no norm kernel runs."""
-        if not rt.tuned:
-            return None
-        from ..kernels import tuned
-        n, H = resid.shape
-        w, x = product.weight, product.x
-        if (w.packed is None or w.swiglu_cols or isinstance(x, tuned.NormedRows) or x.dtype != torch.bfloat16
-                or x.shape[1] % 8 or H % 8):
-            return None
-        K = x.shape[1]
-        xg = rt.buffer("normed_xg", n, H)
-        if n <= tuned.FUSED_NORM_MAX_ROWS:
-            ssq = rt.buffer("normed_ssq", n, tuned.skinny_parts(H), torch.float32)
-            return tuned.gemm_skinny_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps)
-        if n <= tuned.SKINNY_MAX_ROWS and K % 32 == 0 and H % 32 == 0:
-            # 17 to 64 rows: the kernel that adds the K-splits of the product does it
-            ssq = rt.buffer("normed_ssq_mid", n, tuned.mid_parts(H), torch.float32)
-            workspace = tuned._split_workspace(rt, tuned.gemm_mid_splits(n, H, K) * n * H, x.device)
-            return tuned.gemm_mid_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps, workspace)
-        if n > tuned.SKINNY_MAX_ROWS and H % 4 == 0:
-            # many rows (a prompt portion): the tiled product's epilogue does it, or the kernel that adds its K-splits
-            ssq = rt.buffer("normed_ssq_tiled", n, tuned.tiled_parts(n, H, K), torch.float32)
-            splits = tuned.gemm_tiled_splits(n, H, K)
-            workspace = tuned._split_workspace(rt, splits * n * H, x.device) if splits > 1 else None
-            return tuned.gemm_tiled_residual(x, w.packed, resid, self.weight, xg, ssq, self.eps, workspace)
-        return None
+        return rt.gemm_add_norm(product.x, product.weight, resid, self.weight, self.eps)
