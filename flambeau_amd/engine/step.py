@@ -294,28 +294,42 @@ class ModelRunner:
         key = self._program_key(batch, parts, feed)
         hit = self._programs.get(key)
         valid = (self.rt.generation, self._meta_dev.data_ptr())
+        stream = torch.cuda.current_stream().cuda_stream
         if hit is not None and hit.valid == valid:
             self._programs.move_to_end(key)
             hit.hits += 1
-            if hit.graph is None and hit.hits >= self.graph_after_hits:
+            whole = len(hit.stretches) == 1 and isinstance(hit.stretches[0], Program)
+            if whole and hit.graph is None and hit.hits >= self.graph_after_hits:
                 # a shape that keeps coming back: its launches become a graph (they are this
                 # library's kernels only, with fixed arguments), which costs one launch to replay
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
-                    hit.program.run(torch.cuda.current_stream().cuda_stream)
+                    hit.stretches[0].run(torch.cuda.current_stream().cuda_stream)
                 hit.graph = graph
             if hit.graph is not None:
                 hit.graph.replay()
+            elif whole:
+                hit.stretches[0].run(stream)
             else:
-                hit.program.run(torch.cuda.current_stream().cuda_stream)
+                # recorded stretches, and between them the blocks that cannot be replayed, run as they are
+                now = self._state_from(batch, parts, dev)
+                with ops.pinned_stream():
+                    for s in hit.stretches:
+                        if isinstance(s, Program):
+                            s.run(stream)
+                        else:
+                            s(now)
             self.n_replayed += 1
             return hit.logits
-        program = Program()
-        with program.recording():
+        recorder = _StepRecorder()
+        state = self._state_from(batch, parts, dev)
+        state.recorder = recorder
+        with recorder:
             self._feed(dev, feed)
-            logits = self.model.forward(self._state_from(batch, parts, dev), self.storage.entries, self.max_logit_rows)
+            logits = self.model.forward(state, self.storage.entries, self.max_logit_rows)
+        state.recorder = None
         # (a buffer that grew during this very step moved before it was used: the generation is read afterwards)
-        self._programs[key] = _RecordedStep(program, logits, (self.rt.generation, self._meta_dev.data_ptr()))
+        self._programs[key] = _RecordedStep(recorder.stretches, logits, (self.rt.generation, self._meta_dev.data_ptr()))
         self._programs.move_to_end(key)
         while len(self._programs) > self.max_programs:
             self._programs.popitem(last=False)
@@ -365,9 +379,44 @@ class ModelRunner:
         return gs.logits[torch.tensor(wanted, device=self.rt.device)]
 
 
+class _StepRecorder:
+    """Records a step as stretches of launches (``Program``) with, between them, whatever a model
+    says cannot be recorded (``cut``): callables that take the step's state and run again at every
+    replay."""
+
+    def __init__(self):
+        self.stretches: list = []
+        self._open = None
+
+    def _begin(self):
+        self._open = Program()
+        self._ctx = self._open.recording()
+        self._ctx.__enter__()
+
+    def _end(self):
+        self._ctx.__exit__(None, None, None)
+        if len(self._open):
+            self.stretches.append(self._open)
+        self._open = None
+
+    def __enter__(self):
+        self._begin()
+        return self
+
+    def __exit__(self, *exc):
+        self._end()
+
+    def cut(self, run_again) -> None:
+        """End the stretch that is being recorded, note ``run_again(step_state)`` for the replays,
+        begin the next stretch.  The caller runs the thing itself now, with recording suspended."""
+        self._end()
+        self.stretches.append(run_again)
+        self._begin()
+
+
 class _RecordedStep:
-    def __init__(self, program, logits, valid):
-        self.program = program
+    def __init__(self, stretches, logits, valid):
+        self.stretches = stretches  # Programs, and callables for what cannot be recorded
         self.logits = logits
         self.valid = valid          # (buffer generation, address of the metadata) the arguments belong to
         self.hits = 0

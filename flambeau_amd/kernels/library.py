@@ -86,6 +86,20 @@ class FlArg(ctypes.Union):
 _FIELD = {P: "p", I: "i", F: "f", L: "l"}
 
 
+class suspended:
+    """``with suspended():`` launches made inside run, but are not appended to the program that is
+    being recorded (a part that cannot be replayed runs between two recorded stretches)."""
+
+    def __enter__(self):
+        global _recording
+        self._was = _recording
+        _recording = None
+
+    def __exit__(self, *exc):
+        global _recording
+        _recording = self._was
+
+
 class Program:
     """A list of launches recorded while they ran, replayed with one foreign call (csrc/program.hip).
     ``with program.recording():`` appends every ``call`` made inside; ``run(stream)`` launches them

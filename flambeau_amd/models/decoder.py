@@ -15,6 +15,7 @@ from dataclasses import dataclass, field
 import torch
 
 from ..kernels import ops
+from ..kernels.library import suspended
 from ..parts import BLOCKS, EMBEDDINGS, HEADS, NORMS, PartSpec, ResidualStream
 
 
@@ -62,6 +63,7 @@ class DecoderModel:
         self.final_norm = NORMS.create(spec.final_norm)
         self.head = HEADS.create(spec.head or PartSpec("linear_head", dict(sizes, tied=spec.tied_head)))
         self._signature_mixers = None
+        self._recorded_blocks = None        # per block: can its launches be recorded?
         for i, e in enumerate(spec.run_order):
             if not 0 <= e.layer < len(self.blocks):
                 raise ValueError(f"run-order entry {i} names layer {e.layer}, the model has {len(self.blocks)}")
@@ -119,15 +121,29 @@ class DecoderModel:
         return out
 
     def replayable(self) -> bool:
-        """True if a step of this model can be recorded and replayed (``Part.replayable``)."""
-        return all(getattr(p, "replayable", False) for p in self.all_parts())
+        """True if steps of this model can be recorded and replayed (``Part.replayable``): embedding,
+        final norm and head must be; a block that is not runs as it is between the recorded stretches."""
+        return all(self._part_replayable(p) for p in (self.embedding, self.final_norm, self.head))
+
+    @staticmethod
+    def _part_replayable(part) -> bool:
+        todo = [part]
+        while todo:
+            p = todo.pop()
+            if not getattr(p, "replayable", False):
+                return False
+            todo += list(getattr(p, "subparts", lambda: [])())
+        return True
 
     def step_signature(self, batch) -> tuple:
         """What the mixers decide from the batch's numbers beyond its shape (``Mixer.step_signature``),
-        one entry per group of like mixers."""
+        one entry per group of like mixers.  Mixers of blocks that are never recorded decide anew in
+        every step and have no say here."""
         if self._signature_mixers is None:
             seen = {}
             for b in self.blocks:
+                if not self._part_replayable(b):
+                    continue
                 for m in getattr(b, "mixers", lambda: [])():
                     seen.setdefault(m.signature_group(), m)
             self._signature_mixers = list(seen.values())
@@ -154,8 +170,26 @@ class DecoderModel:
         resid = rt.buffer("residual", step.n_tokens, self.spec.hidden_size, torch.float32)
         self.embedding.forward(step.tokens, resid)
         stream = ResidualStream(resid, rt)
+        if self._recorded_blocks is None:
+            self._recorded_blocks = [self._part_replayable(b) for b in self.blocks]
         for i, e in enumerate(self.spec.run_order):
-            self.blocks[e.layer].forward(stream, step, caches[i])
+            block = self.blocks[e.layer]
+            if step.recorder is not None and not self._recorded_blocks[e.layer]:
+                # A block that cannot be replayed ends the recorded stretch: when the step is replayed it
+                # runs again with that step's metadata.  Whatever it allocates lies elsewhere then, so
+                # all that passes between it and the recorded stretches is the residual stream itself:
+                # pending sums are added before it starts and before it ends.
+                stream.flush()
+
+                def run_block(now, block=block, cache=caches[i], resid=resid, rt=rt):
+                    own = ResidualStream(resid, rt)
+                    block.forward(own, now, cache)
+                    own.flush()
+                step.recorder.cut(run_block)
+                with suspended():
+                    run_block(step)
+            else:
+                block.forward(stream, step, caches[i])
         if step.logit_rows.shape[0] == 0:
             stream.flush()
             return None

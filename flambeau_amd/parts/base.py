@@ -139,6 +139,7 @@ class StepState:
     host: "HostBatch"              # the same numbers on the host, for choosing kernels
     extra: dict = field(default_factory=dict)   # metadata parts asked for (step_metadata)
     scratch: dict = field(default_factory=dict)  # what parts compute once per forward pass and share between layers; emptied when a pass begins
+    recorder: object = None        # set while the step is being recorded (engine/step.py): ``cut(fn)`` ends a recorded stretch
 
 
 @dataclass

@@ -406,6 +406,54 @@ def test_recorded_steps_equal_eager_ones(model_dirs, dtype):
     rh.compare(replayed, reqs, rh.plain_logits(d, reqs), dtype, "recorded steps")
 
 
+def test_a_block_that_cannot_be_recorded_runs_between_recorded_stretches(model_dirs, tmp_path):
+    """One block of the model says that its launches cannot be recorded (as a block with a part that
+    calls torch would): steps are still recorded, in stretches, and the block runs again between them at
+    every replay, with that step's requests and pages.  Logits agree with the plain implementation
+    and, but for the add and the norm around the block that are not fused then, with the unrecorded
+    engine."""
+    import json, shutil
+    from flambeau_amd.config.mistral import MistralConfig
+    from flambeau_amd.engine import ModelRunner, load_model
+    from flambeau_amd.kernels.library import Program
+    from flambeau_amd.models.decoder import LayerSpec
+    from flambeau_amd.models.mistral import mistral_spec
+    from flambeau_amd.parts import BLOCKS, PartSpec
+    from flambeau_amd.parts.block import PreNormBlock
+    from flambeau_amd.registry import register_architecture
+    if "prenorm_unrecorded" not in BLOCKS.known():
+        @BLOCKS.register("prenorm_unrecorded")
+        class Unrecorded(PreNormBlock):
+            replayable = False
+
+        def spec(cfg):
+            m = mistral_spec(cfg)
+            m.layers[1] = LayerSpec(PartSpec("prenorm_unrecorded", m.layers[1].block.params), m.layers[1].names)
+            return m
+        register_architecture("MistralOneBlockUnrecorded", MistralConfig, spec)
+    dtype = "bfloat16"
+    src = model_dirs[("D", STORE[dtype])]
+    d = tmp_path / "model"
+    shutil.copytree(src, d)
+    raw = json.loads((d / "config.json").read_text())
+    raw["architectures"] = ["MistralOneBlockUnrecorded"]
+    (d / "config.json").write_text(json.dumps(raw))
+    reqs = rh.make_requests(210, [70, 70, 31, 31, 150], seed=29)
+    ref = rh.plain_logits(src, reqs)
+    model, _ = load_model(d, dtype=dtype, max_batch_tokens=256)
+    assert model.replayable() and not model._part_replayable(model.blocks[1])
+    runner = ModelRunner(model, n_pages=40, page_size=8, max_slots=4, max_logit_rows=256, decode_graphs=False)
+    runner.storage.fill(float("nan"))
+    portions = rh.trace_portions(reqs, sizes=(16, 9, 16, 2, 16, 9))
+    got = rh.run_in_process(runner, portions)
+    got2 = rh.run_in_process(runner, rh.trace_mixed(reqs, seed=6, max_portion=12))
+    assert runner.n_replayed > 20
+    kinds = [[isinstance(s, Program) for s in r.stretches] for r in runner._programs.values()]
+    assert kinds and all(k == [True, False, True] for k in kinds)          # launches, the block, launches
+    rh.compare(got, reqs, ref, dtype, "one unrecorded block: portions")
+    rh.compare(got2, reqs, ref, dtype, "one unrecorded block: mixed")
+
+
 @pytest.fixture(scope="module")
 def wide_model_dir(tmp_path_factory):
     """Two layers with the layer sizes of a 7B model (width 4096, 32 heads in 8 groups of 128,

@@ -485,8 +485,9 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
         assert [type(b.ffn).__name__ for b in model.blocks] == ["Routed", "SwiGLU", "SwiGLU", "Routed"]
         assert [type(b.ffn_norm).__name__ for b in model.blocks] == ["CenteredNorm", "RMSNorm", "RMSNorm", "CenteredNorm"]
     runner = ModelRunner(model, n_pages=16, page_size=8, max_slots=3, max_logit_rows=128)
-    # a mixer with state of its own never replays a padded graph, and parts that call torch are not recorded
-    assert not runner.decode_graphs and not runner.step_programs
+    # a mixer with state of its own never replays a padded graph; blocks with parts that call torch are not
+    # recorded: they run again, between the recorded stretches, whenever a step of a known shape is replayed
+    assert not runner.decode_graphs and runner.step_programs
     # two states; two page pools of different kinds (keys and values; latent rows), each with a table of its own
     assert len(runner.storage.states) == 2 and len(runner.storage.pools) == 2
     assert runner.storage.pools[0].shape[0] == 1                       # the repeated layer reads, it owns no cache
@@ -502,6 +503,7 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
         got = rh.run_in_process(runner, steps)
         rh.compare(got, reqs, ref, dtype, f"toy {mode}")
     assert not runner.manager.live and runner.manager.free_pages() == [16, 16]
+    assert runner.n_replayed > 20 and runner.n_recorded > 3
     # slots are zeroed when they are claimed again: a second pass over the same requests agrees
     rh.compare(rh.run_in_process(runner, rh.trace_mixed(reqs, seed=3, max_live=3)), reqs, ref, dtype, "toy again")
 
