@@ -28,7 +28,7 @@
 
 #define PF_TOKENS 64          // query tokens per block
 #define PF_STAGE 64           // keys per LDS stage
-#define PF_MAX_PAGES 4096     // block-table entries a block keeps in LDS
+#define PF_MAX_PAGES 16384    // block-table entries a block keeps in LDS (64 KB; beyond 4,096 one block per compute unit)
 
 // Which key sits in row i of the two 16-key score tiles of a 32-key chunk: tile a holds keys
 // 8 (i / 4) + i % 4, tile b the same + 4.  A lane (query, g) of the score accumulators then owns

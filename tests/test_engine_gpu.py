@@ -510,6 +510,43 @@ def test_short_portions_behind_a_long_context(tmp_path_factory, dtype):
     rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, "long context")
 
 
+def test_context_beyond_65536_tokens(tmp_path):
+    """70,000 tokens of context (4,375 pages of 16: a block table 8,192 wide): the prompt in portions of
+    4,096, the last tokens one by one; the bfloat16 kernels against the 32-bit path of the same engine on
+    the same (bfloat16-valued) weights.  The plain implementation cannot hold a score matrix this large."""
+    import torch
+    from flambeau_amd.engine import ModelRunner, load_model
+    from flambeau_amd.weights import write_random_model
+    config = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "hidden_act": "silu",
+              "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2,
+              "intermediate_size": 96, "vocab_size": 150, "rope_theta": 1e6, "sliding_window": None,
+              "rms_norm_eps": 1e-5, "max_position_embeddings": 131072, "tie_word_embeddings": False}
+    d = write_random_model(config, tmp_path / "model", seed=14, std=0.08, gain_std=0.02, store_dtype=torch.bfloat16)
+    n, tail = 70000, 6
+    toks = rh.make_requests(150, [n], seed=10)["r0"]
+    steps, at = [], 0
+    while at < n - tail:
+        cnt = min(4096, n - tail - at)
+        steps.append(dict(step=len(steps), entries=[dict(id="r0", tokens=toks[at:at + cnt], want=[cnt - 1] if at + cnt == n - tail else [])], end=[]))
+        at += cnt
+    for i in range(n - tail, n):
+        steps.append(dict(step=len(steps), entries=[dict(id="r0", tokens=toks[i:i + 1], want=[0])], end=["r0"] if i == n - 1 else []))
+    results = {}
+    for dtype in ("float32", "bfloat16"):
+        model, _ = load_model(d, dtype=dtype, max_batch_tokens=4096)
+        runner = ModelRunner(model, n_pages=4400, page_size=16, max_slots=2, max_logit_rows=8)
+        runner.storage.fill(float("nan"))
+        results[dtype] = rh.run_in_process(runner, steps)
+        assert not runner.manager.live and runner.manager.free_pages() == [4400]
+        del runner, model
+        torch.cuda.empty_cache()
+    want, got = results["float32"], results["bfloat16"]
+    assert sorted(want) == sorted(got) and len(want) == tail + 1
+    scale = max(float(np.abs(v).max()) for v in want.values())
+    for k in want:
+        assert np.isfinite(got[k]).all() and np.abs(got[k] - want[k]).max() <= 2e-2 * scale, k
+
+
 def test_serving_loop_under_random_pressure(model_dirs):
     """Random mixes of requests, slots, pages, portion sizes, sampling and stop ids through the serving
     loop (which runs a step ahead of the host and pre-empts when pages run out): every request's
