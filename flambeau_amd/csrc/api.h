@@ -38,6 +38,12 @@ int fl_feed_tokens(int* tokens, const int* ids, const int* src, int n, hipStream
 int fl_argmax(const float* logits, int* out, int rows, int V, hipStream_t stream);
 int fl_sample(const float* logits, const float* inv_temp, const float* uniform, int* out,
               int rows, int V, hipStream_t stream);
+// The same draw through top-k, top-p and min-p for the rows that ask for them (top_k[r] >= 1 as a float,
+// 0 < top_p[r] < 1, min_p[r] > 0); other rows are left to fl_sample.  At most fl_sample_filtered_max_k()
+// candidates are kept.
+int fl_sample_filtered(const float* logits, const float* inv_temp, const float* uniform, const float* top_k,
+                       const float* top_p, const float* min_p, int* out, int rows, int V, hipStream_t stream);
+int fl_sample_filtered_max_k(void);
 
 // ---- tuned bf16 kernels ----
 // nw_hint: waves per block that split K (0: chosen from the sizes)

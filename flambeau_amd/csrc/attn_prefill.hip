@@ -29,6 +29,7 @@
 #define PF_TOKENS 64          // query tokens per block
 #define PF_STAGE 64           // keys per LDS stage
 #define PF_MAX_PAGES 16384    // block-table entries a block keeps in LDS (64 KB; beyond 4,096 one block per compute unit)
+#define PF_LDS_BYTES (160 * 1024)     // LDS of a compute unit: the ring of key/value stages and the table share it
 
 // Which key sits in row i of the two 16-key score tiles of a 32-key chunk: tile a holds keys
 // 8 (i / 4) + i % 4, tile b the same + 4.  A lane (query, g) of the score accumulators then owns
@@ -401,7 +402,7 @@ static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, b
     auto kern = attn_prefill_kernel<HDP, QT, NS>;
     if (!configured) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  RING + PF_MAX_PAGES * (int)sizeof(int));
+                                  min(RING + PF_MAX_PAGES * (int)sizeof(int), PF_LDS_BYTES));
         configured = true;
     }
     kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from, part_o, part_ml);
@@ -519,7 +520,11 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     FL_CHECK(page_size >= 8 && (page_size & (page_size - 1)) == 0,
              "attn_prefill: page size %d must be a power of two, at least 8", page_size);
     FL_CHECK((long long)2 * nkv * page_size * hd < (1ll << 31), "attn_prefill: a page of %d heads x %d keys x %d is too large (2^31 values)", nkv, page_size, hd);
-    FL_CHECK(max_blocks <= PF_MAX_PAGES, "attn_prefill: %d pages per request, at most %d", max_blocks, PF_MAX_PAGES);
+    {
+        // (the ring of two stages of 64 keys and values: 256 bytes per padded head dim and stage)
+        const int hdp = (hd + 31) / 32 * 32, most = min(PF_MAX_PAGES, (PF_LDS_BYTES - 2 * hdp * 256) / (int)sizeof(int));
+        FL_CHECK(max_blocks <= most, "attn_prefill: %d pages per request, at most %d with heads of %d", max_blocks, most, hd);
+    }
     FL_CHECK(window >= 0, "attn_prefill: negative window");
     FL_CHECK(scale > 0.f, "attn_prefill: the score scale must be positive");
     FL_CHECK(n_split >= 1 && n_split <= 16, "attn_prefill: %d splits (at most 16)", n_split);

@@ -126,14 +126,14 @@ class LLMEngine:
             inv_t = [0.0 if s.request.params.is_greedy else 1.0 / s.request.params.temperature for s in rows]
             us = [0.0 if s.request.params.is_greedy else s.request.rng.next_f32() for s in rows]
             if rows:
-                handle = self.sampler.sample_async(logits, inv_t, us)
+                handle = self.sampler.sample_async(logits, inv_t, us, [s.request.params.device_filters for s in rows])
             else:
                 handle = (0, 0)
             self.scheduler.advance(sched)
             finished += self.flush()                  # the step before; this one is running meanwhile
             self._in_flight = (sched, handle) if rows else None
             return finished
-        # Some request wants penalties, a bias or filters: its logits go to the host sampler and nothing
+        # Some request wants penalties or a bias: its logits go to the host sampler and nothing
         # stays in flight.  Rows that the device can draw are still drawn there (by the same kernel,
         # from the same numbers of their own generators), so a request's tokens do not depend on
         # what its neighbours ask for.
@@ -146,7 +146,7 @@ class LLMEngine:
             inv_t = [0.0 if p.is_greedy else 1.0 / p.temperature for p in params]
             us = [0.0 if p.is_greedy else rows[i].request.rng.next_f32() for i, p in zip(on_dev, params)]
             picked = logits if on_dev == list(range(logits.shape[0])) else self._pick_rows(logits, on_dev)
-            for i, t in zip(on_dev, self.sampler.sample(picked, inv_t, us)):
+            for i, t in zip(on_dev, self.sampler.sample(picked, inv_t, us, [p.device_filters for p in params])):
                 sampled[rows[i].request.request_id] = t
         on_host = [i for i in live if i not in on_dev]
         if on_host:

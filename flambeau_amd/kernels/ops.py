@@ -206,6 +206,17 @@ def argmax(logits, out):
     return out
 
 
+def sample_filtered(logits, inv_temp, uniform, top_k, top_p, min_p, out):
+    """The temperature draw through top-k, top-p and min-p for the rows that ask for them (``top_k``
+    >= 1 as a float, 0 < ``top_p`` < 1, ``min_p`` > 0); other rows of ``out`` are not touched."""
+    R, V = logits.shape
+    f = lambda t, name: _check(t, "sample_filtered." + name, torch.float32, (R,))
+    call("fl_sample_filtered", _check(logits, "sample_filtered.logits", torch.float32), f(inv_temp, "inv_temp"),
+         f(uniform, "uniform"), f(top_k, "top_k"), f(top_p, "top_p"), f(min_p, "min_p"),
+         _check(out, "sample_filtered.out", torch.int32, (R,)), R, V, stream_handle())
+    return out
+
+
 def sample(logits, inv_temp, uniform, out):
     R, V = logits.shape
     call("fl_sample", _check(logits, "sample.logits", torch.float32),

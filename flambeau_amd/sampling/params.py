@@ -4,6 +4,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+DEVICE_TOP_K_MAX = 2048       # candidates the device sampler keeps (fl_sample_filtered_max_k)
+
 
 @dataclass
 class SamplingParams:
@@ -43,6 +45,16 @@ class SamplingParams:
 
     @property
     def device_ok(self) -> bool:
-        """Greedy and plain temperature sampling run on the device; penalties, bias and
-        filters need the logits on the host."""
-        return not (self.has_penalties or self.has_filters or self.logit_bias)
+        """Greedy sampling, the temperature draw and the filters (top-k up to 2048, top-p, min-p) run
+        on the device; penalties and a bias need the request's history and the logits on the host."""
+        return not (self.has_penalties or self.logit_bias or (self.top_k is not None and self.top_k > DEVICE_TOP_K_MAX))
+
+    @property
+    def device_filters(self) -> tuple:
+        """``(top_k, top_p, min_p)`` as the device sampler takes them: 0 for what is not asked for."""
+        top_p = self.top_p if self.top_p is not None and 0.0 < self.top_p < 1.0 else 0.0
+        min_p = self.min_p if self.min_p is not None and self.min_p > 0.0 else 0.0
+        top_k = int(self.top_k) if self.top_k is not None else (DEVICE_TOP_K_MAX if (top_p or min_p) else 0)
+        if self.has_filters and not (top_k or top_p or min_p):
+            top_k = DEVICE_TOP_K_MAX          # filters that cut nothing (top_p = 1) still draw among the 2048 most probable
+        return (top_k, top_p, min_p)

@@ -413,6 +413,61 @@ def test_sample_is_the_inverse_cdf_in_index_order(V):
     assert bad <= 2
 
 
+@pytest.mark.parametrize("V", [97, 1000, 32768, 131072])
+def test_filtered_sample_is_the_host_sampler_s(V):
+    """Top-k, top-p and min-p on the device against the host sampler (itself checked against the plain
+    one) with the same uniform numbers: rows of every combination of filters, logits with ties, rows
+    without a filter and greedy rows among them (those keep what the plain kernel drew)."""
+    from flambeau_amd.sampling.host import sample_host
+    from flambeau_amd.sampling.params import SamplingParams
+    rng = np.random.default_rng(V)
+    combos = []
+    for top_k in (None, 1, 5, 40, 700, 2048):
+        for top_p in (None, 0.15, 0.9, 0.999, 1.0):
+            for min_p in (None, 0.02, 0.6):
+                combos.append((top_k, top_p, min_p))
+    R = len(combos) + 2
+    logits = rnd(R, V, seed=16, scale=2.5)
+    logits[3] = torch.round(logits[3] * 2) / 2            # many equal logits: ties go by index
+    logits[7, :] = 0.25                                    # all equal
+    logits[9] = torch.round(logits[9])
+    temps = rng.choice([0.6, 0.8, 1.0, 1.7], R).tolist()
+    us = rng.random(R).astype(np.float32)
+    us[4], us[5] = 0.0, np.float32(0.9999999)
+    params = [SamplingParams(temperature=t, top_k=c[0], top_p=c[1], min_p=c[2]) for t, c in zip(temps, combos)]
+    params += [SamplingParams(temperature=0.9), SamplingParams(temperature=0.0, top_k=5)]       # no filter; greedy
+    assert all(p.device_ok for p in params)
+    f32 = lambda v: torch.tensor(np.asarray(v, dtype=np.float32), device=DEV)
+    inv_t = f32([0.0 if p.is_greedy else 1.0 / p.temperature for p in params])
+    filt = [p.device_filters for p in params]
+    out = torch.full((R,), -1, dtype=torch.int32, device=DEV)
+    plain_draw = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops().sample(logits, inv_t, f32(us), plain_draw)
+    out.copy_(plain_draw)
+    ops().sample_filtered(logits, inv_t, f32(us), f32([f[0] for f in filt]), f32([f[1] for f in filt]), f32([f[2] for f in filt]), out)
+    assert out[R - 2] == plain_draw[R - 2] and out[R - 1] == plain_draw[R - 1] == int(torch.argmax(logits[R - 1]))
+
+    class OneNumber:
+        def __init__(self, u): self.u = u
+        def next_f32(self): return self.u
+    l = logits.cpu().numpy()
+    differ = 0
+    for r in range(R - 2):
+        want = sample_host(l[r], params[r], [], OneNumber(us[r]))
+        got = int(out[r])
+        if got != want:
+            # sums in another order: a draw on a boundary may fall to the neighbour in the order of probability
+            p = np.exp((l[r].astype(np.float64) - l[r].max()) / temps[r]); p /= p.sum()
+            order = np.argsort(-p, kind="stable").tolist()
+            assert abs(order.index(got) - order.index(want)) == 1, (r, combos[r], got, want)
+            differ += 1
+    assert differ <= 2
+    # a filter that leaves one candidate is the argmax, whatever the number drawn
+    for r, c in enumerate(combos):
+        if c[0] == 1:
+            assert int(out[r]) == int(np.argmax(l[r]))
+
+
 # ---------------------------------------------------------------- tuned attention for single rows
 def decode_rows(case, picked):
     """(row, position, request, 0) of the picked rows, as the decode kernel wants them."""
