@@ -274,6 +274,29 @@ def test_a_request_s_tokens_do_not_depend_on_what_its_neighbours_ask_for(model_d
     assert host.generate(prompts[:2], greedy) == eng.generate(prompts[:2], greedy)
 
 
+def test_filtered_requests_stay_on_the_device(model_dirs, monkeypatch):
+    """Top-k, top-p and min-p are drawn by the device sampler: no logits go to the host sampler (it
+    raises here if called), the engine keeps a step in flight, and the tokens are the plain sampler's."""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    import flambeau_amd.engine.llm as llm
+
+    def no_host(*a, **k):
+        raise AssertionError("the host sampler was called")
+    monkeypatch.setattr(llm, "sample_host", no_host)
+    d = model_dirs[("B", "float32")]
+    prompts = list(rh.make_requests(384, [5, 23, 40, 12], seed=31).values())
+    opts = [dict(temperature=0.9, top_k=12, seed=601), dict(temperature=0.7, top_p=0.8, seed=602),
+            dict(temperature=1.2, top_k=50, top_p=0.95, min_p=0.05, seed=603), dict(temperature=1.0, min_p=0.2, seed=604)]
+    eng = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", page_size=16, inflight_slots=4, prefill_chunk_tokens=32))
+    seen_in_flight = []
+    step = eng.step
+    monkeypatch.setattr(eng, "step", lambda: (step(), seen_in_flight.append(eng._in_flight is not None))[0])
+    outs = eng.generate(prompts, [SamplingParams(max_tokens=16, **o) for o in opts])
+    assert any(seen_in_flight)
+    for prompt, out, o in zip(prompts, outs, opts):
+        assert out == _plain_generate(d, prompt, 16, **o)[0]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_stop_tokens_end_requests_while_the_next_step_is_in_flight(model_dirs, dtype):
     """The engine runs one step ahead of the host: when a stop id (or one of several end-of-sequence
