@@ -40,9 +40,10 @@ int fl_sample(const float* logits, const float* inv_temp, const float* uniform, 
               int rows, int V, hipStream_t stream);
 // The same draw through top-k, top-p and min-p for the rows that ask for them (top_k[r] >= 1 as a float,
 // 0 < top_p[r] < 1, min_p[r] > 0); other rows are left to fl_sample.  At most fl_sample_filtered_max_k()
-// candidates are kept.
+// candidates are kept.  stash: rows * V values of scratch for vocabularies beyond 32,768, or null.
 int fl_sample_filtered(const float* logits, const float* inv_temp, const float* uniform, const float* top_k,
-                       const float* top_p, const float* min_p, int* out, int rows, int V, hipStream_t stream);
+                       const float* top_p, const float* min_p, int* out, int rows, int V, unsigned* stash,
+                       hipStream_t stream);
 int fl_sample_filtered_max_k(void);
 
 // ---- tuned bf16 kernels ----

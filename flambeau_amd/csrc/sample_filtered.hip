@@ -14,7 +14,7 @@
 // One block of 1,024 threads per row:
 //   1. maximum and sum of the exponentials (coalesced);
 //   2. the k-th largest probability by a radix selection over the bits of p (p >= 0, so the bits
-//      order like the values): eight passes of 4 bits, counted with ballots (vocabularies up to
+//      order like the values): eight passes of 4 bits, counted in registers (vocabularies up to
 //      32,768 keep their probabilities in registers between the passes);
 //   3. the candidates above it, and of those equal to it the first by index, go to LDS as 64-bit
 //      keys (bits of p, then the complement of the index) and are sorted by a bitonic network;
@@ -35,7 +35,8 @@ __device__ __forceinline__ float sf_prob(float logit, float inv_t, float scaled_
 }
 
 // KEEP: every thread holds the bits of its probabilities in registers (element tid + e * SF_THREADS in
-// place e); otherwise they are formed again in every pass.
+// place e); otherwise they are written to the row's part of `stash` once and read back by every pass
+// (or, without a stash, formed again in every pass).
 template <bool KEEP>
 __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float* __restrict__ logits,
                                                                     const float* __restrict__ inv_temp,
@@ -43,7 +44,8 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
                                                                     const float* __restrict__ top_k,
                                                                     const float* __restrict__ top_p,
                                                                     const float* __restrict__ min_p,
-                                                                    int* __restrict__ out, int V) {
+                                                                    int* __restrict__ out, int V,
+                                                                    unsigned* __restrict__ stash) {
     __shared__ unsigned long long cand[SF_MAX_K];
     __shared__ unsigned bins[SF_WAVES][16];
     __shared__ int per_thread[SF_THREADS];
@@ -83,43 +85,67 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
             part += p;
         }
     } else {
-        for (int i = tid; i < V; i += SF_THREADS) part += sf_prob(row[i], it, smax);
+        unsigned* mine = stash ? stash + (size_t)r * V : nullptr;
+        for (int i = tid; i < V; i += SF_THREADS) {
+            const float p = sf_prob(row[i], it, smax);
+            if (mine) mine[i] = __float_as_uint(p);
+            part += p;
+        }
     }
-    const float total = block_sum<SF_WAVES>(part, red);
+    const float total = block_sum<SF_WAVES>(part, red);               // (its barriers also order the stash's writes before the reads below: every thread reads what it wrote)
+    const unsigned* stashed = (!KEEP && stash) ? stash + (size_t)r * V : nullptr;
     auto bits_at = [&](int e, int i) -> unsigned {
-        return KEEP ? kept_bits[KEEP ? e : 0] : __float_as_uint(sf_prob(row[i], it, smax));
+        if (KEEP) return kept_bits[KEEP ? e : 0];
+        return stashed ? stashed[i] : __float_as_uint(sf_prob(row[i], it, smax));
     };
 
-    // ---- 2. the bits of the k-th largest probability: eight passes of four bits.  A wave counts the
-    // elements of each of sixteen values with a ballot (most probabilities share their leading bits:
-    // a histogram in LDS would serialise on a few bins); the waves' counts are added by one thread.
+    // ---- 2. the bits of the k-th largest probability: eight passes of four bits.  Every lane counts its
+    // elements of each of sixteen values in registers (most probabilities share their leading bits: a
+    // histogram in LDS would serialise on a few bins); the counts are added over the wave, then over
+    // the waves by one thread.
     if (tid == 0) { s_prefix = 0u; s_remaining = (unsigned)k; }
     __syncthreads();
     unsigned known = 0u;                                                   // mask of the bits fixed so far
     const int n_elems = (V + SF_THREADS - 1) / SF_THREADS;
     for (int shift = 28; shift >= 0; shift -= 4) {
         const unsigned prefix = s_prefix;
-        unsigned cnt[16];
-#pragma unroll
-        for (int b = 0; b < 16; ++b) cnt[b] = 0u;
+        // sixteen counters of eight bits in two 64-bit words per lane (a lane sees at most 255 elements
+        // in a pass), unpacked and added over the wave at the end of the pass
+        unsigned long long c_lo = 0ull, c_hi = 0ull;
         auto count = [&](unsigned bits, bool valid) {
-            const unsigned d = (valid && (bits & known) == prefix) ? (bits >> shift) & 15u : 16u;
-#pragma unroll
-            for (int b = 0; b < 16; ++b) cnt[b] += (unsigned)__popcll(__ballot(d == (unsigned)b));
+            const bool hit = valid && (bits & known) == prefix;
+            const unsigned d = (bits >> shift) & 15u;
+            const unsigned long long inc = 1ull << ((d & 7u) * 8u);
+            c_lo += (hit && d < 8u) ? inc : 0ull;
+            c_hi += (hit && d >= 8u) ? inc : 0ull;
         };
         if (KEEP) {
 #pragma unroll
             for (int e = 0; e < SF_KEEP; ++e)
                 if (e < n_elems) count(kept_bits[KEEP ? e : 0], tid + e * SF_THREADS < V);
         } else {
-            for (int e = 0; e < n_elems; ++e) {
+            int e = 0;
+            for (; e + 4 <= n_elems; e += 4) {                              // four loads in flight
+                unsigned v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int i = tid + (e + u) * SF_THREADS;
+                    v[u] = i < V ? bits_at(e + u, i) : 0u;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) count(v[u], tid + (e + u) * SF_THREADS < V);
+            }
+            for (; e < n_elems; ++e) {
                 const int i = tid + e * SF_THREADS;
                 count(i < V ? bits_at(e, i) : 0u, i < V);
             }
         }
-        if (lane == 0) {
 #pragma unroll
-            for (int b = 0; b < 16; ++b) bins[wave][b] = cnt[b];
+        for (int b = 0; b < 16; ++b) {
+            unsigned c = (unsigned)(((b < 8 ? c_lo : c_hi) >> ((b & 7) * 8)) & 255ull);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+            if (lane == 0) bins[wave][b] = c;
         }
         __syncthreads();
         if (tid == 0) {
@@ -145,15 +171,30 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
     // the k-th are taken in index order: element i = tid + e * SF_THREADS, so place e by place e the
     // threads' counts are scanned (few elements are equal: the scan runs over the places that have any).
     if (tid == 0) s_count = 0u;
+    int n_mine = 0;                                                        // my elements equal to the k-th
+    for (int e = 0; e < n_elems; ++e) {
+        const int i = tid + e * SF_THREADS;
+        n_mine += i < V && (KEEP ? kept_bits[KEEP ? min(e, SF_KEEP - 1) : 0] : bits_at(e, i)) == kth;
+    }
+    per_thread[tid] = n_mine;
+    __syncthreads();
+    // (usually all elements equal to the k-th are wanted: then their order does not matter)
+    int all_equal = 0;
+    for (int t = lane; t < SF_THREADS; t += 64) all_equal += per_thread[t];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) all_equal += __shfl_xor(all_equal, o, 64);
+    const bool take_all = all_equal == n_equal;
     __syncthreads();
     int base_rank = 0;
     for (int e = 0; e < n_elems; ++e) {
         const int i = tid + e * SF_THREADS;
         const unsigned bits = i < V ? (KEEP ? kept_bits[KEEP ? min(e, SF_KEEP - 1) : 0] : bits_at(e, i)) : 0u;
-        if (i < V && bits > kth) {
+        if (i < V && (bits > kth || (take_all && bits == kth))) {
             const unsigned at = atomicAdd(&s_count, 1u);
             if (at < SF_MAX_K) cand[at] = ((unsigned long long)bits << 32) | (unsigned long long)(0xFFFFFFFFu - (unsigned)i);
         }
+        if (take_all) continue;
+        // more elements equal the k-th than are wanted: the first by index, place by place
         const bool eq = i < V && bits == kth;
         if (__syncthreads_or(eq) && base_rank < n_equal) {
             // ranks of this place's equal elements, in the order of the threads (which is index order)
@@ -255,17 +296,20 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
 
 // Rows with a filter (top_k[r] >= 1, 0 < top_p[r] < 1 or min_p[r] > 0) and inv_temp[r] > 0 are drawn
 // here; the others are not touched (fl_sample draws them).  top_k travels as a float (exact below 2^24);
-// more than 2048 candidates are not kept: the caller sends such rows to the host sampler.
+// more than 2048 candidates are not kept: the caller sends such rows to the host sampler.  A vocabulary
+// beyond 32,768 is read ten times: with `stash` (rows * V values, or null) the probabilities are formed
+// once and kept there.
 extern "C" int fl_sample_filtered(const float* logits, const float* inv_temp, const float* uniform,
                                   const float* top_k, const float* top_p, const float* min_p, int* out,
-                                  int rows, int V, hipStream_t stream) {
+                                  int rows, int V, unsigned* stash, hipStream_t stream) {
     FL_CHECK(rows >= 0 && V > 0, "sample_filtered: bad sizes");
+    FL_CHECK(V <= 255 * SF_THREADS, "sample_filtered: a vocabulary of %d, at most %d", V, 255 * SF_THREADS);
     FL_CHECK(logits && inv_temp && uniform && top_k && top_p && min_p && out, "sample_filtered: needs all its arrays");
     if (rows == 0) return 0;
     if (V <= SF_KEEP * SF_THREADS)
-        sample_filtered_kernel<true><<<rows, SF_THREADS, 0, stream>>>(logits, inv_temp, uniform, top_k, top_p, min_p, out, V);
+        sample_filtered_kernel<true><<<rows, SF_THREADS, 0, stream>>>(logits, inv_temp, uniform, top_k, top_p, min_p, out, V, nullptr);
     else
-        sample_filtered_kernel<false><<<rows, SF_THREADS, 0, stream>>>(logits, inv_temp, uniform, top_k, top_p, min_p, out, V);
+        sample_filtered_kernel<false><<<rows, SF_THREADS, 0, stream>>>(logits, inv_temp, uniform, top_k, top_p, min_p, out, V, stash);
     FL_LAUNCH_CHECK();
     return 0;
 }

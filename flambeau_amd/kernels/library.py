@@ -27,7 +27,7 @@ _SIGNATURES = {
     "fl_feed_tokens": [P, P, P, I, P],
     "fl_argmax": [P, P, I, I, P],
     "fl_sample": [P, P, P, P, I, I, P],
-    "fl_sample_filtered": [P, P, P, P, P, P, P, I, I, P],
+    "fl_sample_filtered": [P, P, P, P, P, P, P, I, I, P, P],
 }
 
 

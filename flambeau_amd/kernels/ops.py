@@ -206,14 +206,19 @@ def argmax(logits, out):
     return out
 
 
-def sample_filtered(logits, inv_temp, uniform, top_k, top_p, min_p, out):
+def sample_filtered(logits, inv_temp, uniform, top_k, top_p, min_p, out, stash=None):
     """The temperature draw through top-k, top-p and min-p for the rows that ask for them (``top_k``
-    >= 1 as a float, 0 < ``top_p`` < 1, ``min_p`` > 0); other rows of ``out`` are not touched."""
+    >= 1 as a float, 0 < ``top_p`` < 1, ``min_p`` > 0); other rows of ``out`` are not touched.
+    ``stash`` (int32 or float32, at least R * V values): scratch that spares a vocabulary beyond 32,768
+    the forming of its probabilities in every pass."""
     R, V = logits.shape
+    if stash is not None and (stash.numel() < R * V or stash.element_size() != 4 or not stash.is_contiguous()):
+        raise KernelError(f"sample_filtered.stash: {stash.numel()} values of {stash.element_size()} bytes, {R * V} of 4 wanted")
     f = lambda t, name: _check(t, "sample_filtered." + name, torch.float32, (R,))
     call("fl_sample_filtered", _check(logits, "sample_filtered.logits", torch.float32), f(inv_temp, "inv_temp"),
          f(uniform, "uniform"), f(top_k, "top_k"), f(top_p, "top_p"), f(min_p, "min_p"),
-         _check(out, "sample_filtered.out", torch.int32, (R,)), R, V, stream_handle())
+         _check(out, "sample_filtered.out", torch.int32, (R,)), R, V,
+         stash.data_ptr() if stash is not None else None, stream_handle())
     return out
 
 

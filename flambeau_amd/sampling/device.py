@@ -24,6 +24,7 @@ class DeviceSampler:
         self._ids_host = torch.empty((2, max_rows), dtype=torch.int32, pin_memory=True)
         self._events = [torch.cuda.Event(), torch.cuda.Event()]
         self._turn = 0
+        self._stash = None           # scratch of the filtered draw for vocabularies beyond 32,768
 
     def sample_async(self, logits, inv_temps, uniforms, filters=None):
         """Enqueue the draw for ``logits`` float32 [R, V] (per row ``inv_temp``, <= 0: argmax, and a
@@ -56,8 +57,11 @@ class DeviceSampler:
                 ops.sample(logits, self._dev[0, :R], self._dev[1, :R], ids)
                 if filtered:
                     # rows with a filter are drawn again, through it; the others keep their draw
+                    V = logits.shape[1]
+                    if V > 32768 and (self._stash is None or self._stash.numel() < self.max_rows * V):
+                        self._stash = torch.empty(self.max_rows * V, dtype=torch.int32, device=self.device)
                     ops.sample_filtered(logits, self._dev[0, :R], self._dev[1, :R], self._dev[2, :R], self._dev[3, :R],
-                                        self._dev[4, :R], ids)
+                                        self._dev[4, :R], ids, stash=self._stash if V > 32768 else None)
             self._ids_host[k, :R].copy_(ids, non_blocking=True)
         self._events[k].record()
         return k, R

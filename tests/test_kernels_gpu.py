@@ -444,7 +444,13 @@ def test_filtered_sample_is_the_host_sampler_s(V):
     plain_draw = torch.empty(R, dtype=torch.int32, device=DEV)
     ops().sample(logits, inv_t, f32(us), plain_draw)
     out.copy_(plain_draw)
-    ops().sample_filtered(logits, inv_t, f32(us), f32([f[0] for f in filt]), f32([f[1] for f in filt]), f32([f[2] for f in filt]), out)
+    args = (logits, inv_t, f32(us), f32([f[0] for f in filt]), f32([f[1] for f in filt]), f32([f[2] for f in filt]))
+    ops().sample_filtered(*args, out)
+    if V > 32768:
+        # with scratch for the probabilities (formed once instead of in every pass): the same draws
+        again = plain_draw.clone()
+        ops().sample_filtered(*args, again, stash=torch.empty(R * V, dtype=torch.int32, device=DEV))
+        assert torch.equal(again, out)
     assert out[R - 2] == plain_draw[R - 2] and out[R - 1] == plain_draw[R - 1] == int(torch.argmax(logits[R - 1]))
 
     class OneNumber:
