@@ -45,6 +45,14 @@ int fl_sample_filtered(const float* logits, const float* inv_temp, const float* 
                        const float* top_p, const float* min_p, int* out, int rows, int V, unsigned* stash,
                        hipStream_t stream);
 int fl_sample_filtered_max_k(void);
+// Penalties over the tokens a request has generated (counts[slot][V], 16-bit, one row per state slot) and
+// logit bias, in place on the step's logits before the draw; slot[r] < 0 (as a float): the row has none.
+int fl_sample_penalise(float* logits, int rows, int V, const unsigned short* counts, const float* slot,
+                       const float* repetition, const float* presence, const float* frequency, hipStream_t stream);
+int fl_sample_bias(float* logits, int V, int n, const float* row, const float* token, const float* value,
+                   hipStream_t stream);
+int fl_sample_count(unsigned short* counts, int V, int rows, const float* slot, const int* ids, hipStream_t stream);
+int fl_sample_history(unsigned short* counts, int V, int slot, const int* tokens, int n, hipStream_t stream);
 
 // ---- tuned bf16 kernels ----
 // nw_hint: waves per block that split K (0: chosen from the sizes)

@@ -123,18 +123,23 @@ class LLMEngine:
         on_device = self.options.gpu_sampler and all(s.request.params.device_ok for s in rows)
         logits = self.runner.step(entries)
         if on_device:
+            if any(PENDING in r.output and r.params.has_penalties and self._slot(r) is not None
+                   and not self.sampler.holds_history(self._slot(r), r) for r in (s.request for s in rows)):
+                finished += self.flush()              # the history is counted anew from tokens the host knows
             inv_t = [0.0 if s.request.params.is_greedy else 1.0 / s.request.params.temperature for s in rows]
             us = [0.0 if s.request.params.is_greedy else s.request.rng.next_f32() for s in rows]
             if rows:
-                handle = self.sampler.sample_async(logits, inv_t, us, [s.request.params.device_filters for s in rows])
+                requests = [s.request for s in rows]
+                handle = self.sampler.sample_async(logits, inv_t, us, [r.params.device_filters for r in requests],
+                                                   *self._histories_and_biases(requests))
             else:
                 handle = (0, 0)
             self.scheduler.advance(sched)
             finished += self.flush()                  # the step before; this one is running meanwhile
             self._in_flight = (sched, handle) if rows else None
             return finished
-        # Some request wants penalties or a bias: its logits go to the host sampler and nothing
-        # stays in flight.  Rows that the device can draw are still drawn there (by the same kernel,
+        # Some request wants what the device sampler does not take (a top-k beyond 2048, a long
+        # bias list): its logits go to the host sampler and nothing stays in flight.  Rows that the device can draw are still drawn there (by the same kernel,
         # from the same numbers of their own generators), so a request's tokens do not depend on
         # what its neighbours ask for.
         finished += self.flush()
@@ -146,7 +151,8 @@ class LLMEngine:
             inv_t = [0.0 if p.is_greedy else 1.0 / p.temperature for p in params]
             us = [0.0 if p.is_greedy else rows[i].request.rng.next_f32() for i, p in zip(on_dev, params)]
             picked = logits if on_dev == list(range(logits.shape[0])) else self._pick_rows(logits, on_dev)
-            for i, t in zip(on_dev, self.sampler.sample(picked, inv_t, us, [p.device_filters for p in params])):
+            for i, t in zip(on_dev, self.sampler.sample(picked, inv_t, us, [p.device_filters for p in params],
+                                                        *self._histories_and_biases([rows[i].request for i in on_dev]))):
                 sampled[rows[i].request.request_id] = t
         on_host = [i for i in live if i not in on_dev]
         if on_host:
@@ -155,6 +161,22 @@ class LLMEngine:
                 r = rows[i].request
                 sampled[r.request_id] = sample_host(host[i], r.params, r.output, r.rng)
         return finished + self.scheduler.commit(sched, sampled)
+
+    def _slot(self, request):
+        held = self.runner.manager.live.get(request.request_id)
+        return None if held is None else held.slot
+
+    def _histories_and_biases(self, requests):
+        """What the device sampler needs for penalties (the request's slot names its row of token
+        counts) and bias, per row; ``None`` where nobody asks."""
+        histories = biases = None
+        if any(r.params.has_penalties for r in requests):
+            # (a request that has just ended holds no slot any more; its row is drawn and dropped)
+            histories = [(self._slot(r), r, r.output, *r.params.penalties)
+                         if r.params.has_penalties and self._slot(r) is not None else None for r in requests]
+        if any(r.params.logit_bias for r in requests):
+            biases = [r.params.logit_bias for r in requests]
+        return histories, biases
 
     def _pick_rows(self, logits, idx):
         """Rows ``idx`` of the step's logits, gathered on the device for the device sampler."""

@@ -28,6 +28,10 @@ _SIGNATURES = {
     "fl_argmax": [P, P, I, I, P],
     "fl_sample": [P, P, P, P, I, I, P],
     "fl_sample_filtered": [P, P, P, P, P, P, P, I, I, P, P],
+    "fl_sample_penalise": [P, I, I, P, P, P, P, P, P],
+    "fl_sample_bias": [P, I, I, P, P, P, P],
+    "fl_sample_count": [P, I, I, P, P, P],
+    "fl_sample_history": [P, I, I, P, I, P],
 }
 
 

@@ -206,6 +206,46 @@ def argmax(logits, out):
     return out
 
 
+def _counts(counts, V):
+    if counts.dtype != torch.int16 or counts.dim() != 2 or counts.shape[1] != V or not counts.is_contiguous() or not counts.is_cuda:
+        raise KernelError(f"sample.counts: {counts.dtype} {tuple(counts.shape)}, want int16 [slots, {V}] on the device")
+    return counts.data_ptr()
+
+
+def sample_penalise(logits, counts, slot, repetition, presence, frequency):
+    """Repetition, presence and frequency penalties in place on ``logits`` [R, V] for the rows with a
+    history (``slot`` >= 0 as a float: row of ``counts``, int16 [slots, V], how often each token was
+    generated)."""
+    R, V = logits.shape
+    f = lambda t, name: _check(t, "sample_penalise." + name, torch.float32, (R,))
+    call("fl_sample_penalise", _check(logits, "sample_penalise.logits", torch.float32), R, V, _counts(counts, V),
+         f(slot, "slot"), f(repetition, "repetition"), f(presence, "presence"), f(frequency, "frequency"), stream_handle())
+    return logits
+
+
+def sample_bias(logits, rows, tokens, values):
+    """``logits[rows[j], tokens[j]] += values[j]`` (all float32 [n]; a pair occurs once)."""
+    V, n = logits.shape[1], rows.shape[0]
+    f = lambda t, name: _check(t, "sample_bias." + name, torch.float32, (n,))
+    call("fl_sample_bias", _check(logits, "sample_bias.logits", torch.float32), V, n, f(rows, "rows"), f(tokens, "tokens"),
+         f(values, "values"), stream_handle())
+    return logits
+
+
+def sample_count(counts, slot, ids):
+    """The tokens ``ids`` drawn for the rows with a history join it: ``counts[slot[r], ids[r]] += 1``."""
+    R, V = ids.shape[0], counts.shape[1]
+    call("fl_sample_count", _counts(counts, V), V, R, _check(slot, "sample_count.slot", torch.float32, (R,)),
+         _check(ids, "sample_count.ids", torch.int32, (R,)), stream_handle())
+
+
+def sample_history(counts, slot: int, tokens):
+    """Row ``slot`` of ``counts`` is zeroed and the ``tokens`` (int32 [n], may be empty) are counted."""
+    V, n = counts.shape[1], tokens.shape[0]
+    call("fl_sample_history", _counts(counts, V), V, int(slot),
+         _check(tokens, "sample_history.tokens", torch.int32, (n,)) if n else None, n, stream_handle())
+
+
 def sample_filtered(logits, inv_temp, uniform, top_k, top_p, min_p, out, stash=None):
     """The temperature draw through top-k, top-p and min-p for the rows that ask for them (``top_k``
     >= 1 as a float, 0 < ``top_p`` < 1, ``min_p`` > 0); other rows of ``out`` are not touched.

@@ -5,6 +5,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 
 DEVICE_TOP_K_MAX = 2048       # candidates the device sampler keeps (fl_sample_filtered_max_k)
+DEVICE_BIAS_MAX = 256         # logit-bias entries of one request that the device sampler takes
 
 
 @dataclass
@@ -45,9 +46,14 @@ class SamplingParams:
 
     @property
     def device_ok(self) -> bool:
-        """Greedy sampling, the temperature draw and the filters (top-k up to 2048, top-p, min-p) run
-        on the device; penalties and a bias need the request's history and the logits on the host."""
-        return not (self.has_penalties or self.logit_bias or (self.top_k is not None and self.top_k > DEVICE_TOP_K_MAX))
+        """Penalties, a bias of up to 256 entries, greedy sampling, the temperature draw and the filters
+        (top-k up to 2048, top-p, min-p) run on the device; what is beyond goes to the host sampler."""
+        return not ((self.logit_bias is not None and len(self.logit_bias) > DEVICE_BIAS_MAX)
+                    or (self.top_k is not None and self.top_k > DEVICE_TOP_K_MAX))
+
+    @property
+    def penalties(self) -> tuple:
+        return (self.repetition_penalty, self.presence_penalty, self.frequency_penalty)
 
     @property
     def device_filters(self) -> tuple:

@@ -207,7 +207,7 @@ def _plain_generate(d, prompt, n_new, temperature=0.0, seed=0, stop=(), **filter
         logits = pm.forward(cfg, w, toks)[-1].astype(np.float32)
         s = np.sort(logits)
         margins.append(float(s[-1] - s[-2]))
-        toks.append(pm.sample(logits, rng, temperature=temperature, **filters))
+        toks.append(pm.sample(logits, rng, temperature=temperature, history=toks[len(prompt):], **filters))
         if toks[-1] in stop:
             break
     return toks[len(prompt):], margins
@@ -254,8 +254,8 @@ def test_temperature_generation_through_the_entry_point(model_dirs):
 
 
 def test_a_request_s_tokens_do_not_depend_on_what_its_neighbours_ask_for(model_dirs):
-    """A seeded temperature request beside a neighbour with a filter (whose logits go to the host
-    sampler) draws the tokens it draws alone, and the plain sampler's."""
+    """A seeded temperature request beside a neighbour whose logits go to the host sampler (a top-k
+    beyond what the device keeps) draws the tokens it draws alone, and the plain sampler's."""
     from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
     d = model_dirs[("B", "float32")]
     prompts = list(rh.make_requests(384, [9, 14, 20], seed=23).values())
@@ -264,9 +264,11 @@ def test_a_request_s_tokens_do_not_depend_on_what_its_neighbours_ask_for(model_d
     alone = eng.generate(prompts[:1], mine)[0]
     assert alone == _plain_generate(d, prompts[0], 20, temperature=0.8, seed=500)[0]
     beside = eng.generate(prompts, [mine, SamplingParams(temperature=0.9, top_k=7, seed=501, max_tokens=20),
-                                    SamplingParams(temperature=0.0, repetition_penalty=1.3, max_tokens=12)])
+                                    SamplingParams(temperature=0.0, repetition_penalty=1.3, top_k=3000, max_tokens=12)])
+    assert not SamplingParams(top_k=3000).device_ok
     assert beside[0] == alone
     assert beside[1] == _plain_generate(d, prompts[1], 20, temperature=0.9, seed=501, top_k=7)[0]
+    assert beside[2] == _plain_generate(d, prompts[2], 12, repetition_penalty=1.3, top_k=3000)[0]
     # and with the device sampler switched off everything goes through the host sampler
     host = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", page_size=16, inflight_slots=3, prefill_chunk_tokens=32,
                                                     gpu_sampler=False))
@@ -295,6 +297,36 @@ def test_filtered_requests_stay_on_the_device(model_dirs, monkeypatch):
     assert any(seen_in_flight)
     for prompt, out, o in zip(prompts, outs, opts):
         assert out == _plain_generate(d, prompt, 16, **o)[0]
+
+
+def test_penalties_and_bias_stay_on_the_device(model_dirs, monkeypatch):
+    """Penalties over the generated tokens and a logit bias are applied on the device: the host
+    sampler is never called (it raises here), a step stays in flight, and the tokens are the plain
+    sampler's.  More requests than slots and so few pages that requests are pre-empted: a slot's
+    row of counts passes from request to request and is counted anew for a request that returns."""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    import flambeau_amd.engine.llm as llm
+
+    def no_host(*a, **k):
+        raise AssertionError("the host sampler was called")
+    monkeypatch.setattr(llm, "sample_host", no_host)
+    d = model_dirs[("B", "float32")]
+    prompts = list(rh.make_requests(384, [5, 23, 40, 12, 9, 17], seed=37).values())
+    opts = [dict(repetition_penalty=1.8), dict(temperature=0.8, presence_penalty=0.7, frequency_penalty=0.3, seed=611),
+            dict(logit_bias={3: 4.0, 200: 2.5, 9999: 1.0}), dict(temperature=0.9, repetition_penalty=0.7, top_k=20, seed=613),
+            dict(temperature=1.1, frequency_penalty=1.5, logit_bias={7: -3.0, 11: 6.0}, min_p=0.02, seed=614),
+            dict(temperature=0.7, seed=615)]
+    eng = LLMEngine.from_dir(str(d), EngineOptions(dtype="float32", page_size=16, inflight_slots=3, prefill_chunk_tokens=32,
+                                                   paged_kv=6))
+    seen_in_flight = []
+    step = eng.step
+    monkeypatch.setattr(eng, "step", lambda: (step(), seen_in_flight.append(eng._in_flight is not None))[0])
+    n_new = 24
+    outs = eng.generate(prompts, [SamplingParams(max_tokens=n_new, **o) for o in opts])
+    assert any(seen_in_flight) and eng.scheduler.n_preemptions > 0
+    for prompt, out, o in zip(prompts, outs, opts):
+        assert out == _plain_generate(d, prompt, n_new, **o)[0], o
+    assert not eng.runner.manager.live
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

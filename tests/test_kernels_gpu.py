@@ -413,6 +413,63 @@ def test_sample_is_the_inverse_cdf_in_index_order(V):
     assert bad <= 2
 
 
+@pytest.mark.parametrize("V", [97, 1000, 40000])
+def test_penalties_and_bias_are_the_host_sampler_s(V):
+    """Penalties from per-slot token counts and the bias triples against the host's rule, bit for bit:
+    rows with and without a history, neutral penalties, tokens seen several times, a slot that is
+    counted anew for another request, and the counts after a draw has joined them."""
+    from flambeau_amd.sampling.host import penalised
+    from flambeau_amd.sampling.params import SamplingParams
+    rng = np.random.default_rng(V + 1)
+    n_slots, R = 7, 6
+    slots = [2, -1, 0, 5, 1, 3]
+    params = [SamplingParams(repetition_penalty=1.7), SamplingParams(), SamplingParams(presence_penalty=0.6, frequency_penalty=0.35),
+              SamplingParams(repetition_penalty=0.8, frequency_penalty=1.25), SamplingParams(),
+              SamplingParams(repetition_penalty=1.3, presence_penalty=-0.4, logit_bias={1: 2.0, V - 1: -3.5, V + 5: 9.0})]
+    params[1] = SamplingParams(logit_bias={0: 1.5, 17: -0.25})
+    histories = [rng.integers(0, min(V, 40), int(n)).tolist() for n in (50, 0, 9, 200, 30, 0)]
+    histories[3][:3] = [V - 1, V - 1, 0]
+    counts = torch.randint(0, 9, (n_slots, V), dtype=torch.int16, device=DEV)       # what other requests left behind
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    f32 = lambda v: torch.tensor(np.asarray(v, dtype=np.float32), device=DEV)
+    for s, h in zip(slots, histories):
+        if s >= 0:
+            ops().sample_history(counts, s, i32(h))
+    for s, h in zip(slots, histories):
+        if s >= 0:
+            assert counts[s].tolist() == np.bincount(h, minlength=V).tolist()
+    assert counts[4].max() > 0 and counts[6].max() > 0                                # rows nobody took are untouched
+    logits = rnd(R, V, seed=21, scale=3.0)
+    want = [penalised(l, p, h) for l, p, h in zip(logits.cpu().numpy(), params, histories)]
+
+    def apply(l):
+        ops().sample_penalise(l, counts, f32(slots), f32([p.repetition_penalty for p in params]),
+                              f32([p.presence_penalty for p in params]), f32([p.frequency_penalty for p in params]))
+        triples = [(r, t, b) for r, p in enumerate(params) if p.logit_bias for t, b in p.logit_bias.items() if t < V]
+        ops().sample_bias(l, *(f32(list(c)) for c in zip(*triples)))
+        return l
+    got = apply(logits.clone())
+    assert torch.equal(got.cpu(), torch.tensor(np.stack(want)))
+    assert not torch.equal(got[0], logits[0]) and torch.equal(got[4], logits[4])
+    # the drawn tokens join the histories (a row without a slot counts nowhere; a token twice in a row adds up)
+    for draw in ([3, 5, 3, V - 1, 0, 8], [3, 5, 7, V - 1, 0, 8]):
+        before = counts.clone()
+        ops().sample_count(counts, f32(slots), i32(draw))
+        for s, h, t in zip(slots, histories, draw):
+            if s >= 0:
+                h.append(t)
+        changed = (counts != before).nonzero().tolist()
+        assert sorted(changed) == sorted([s, t] for s, t in zip(slots, draw) if s >= 0)
+    want = [penalised(l, p, h) for l, p, h in zip(logits.cpu().numpy(), params, histories)]
+    assert torch.equal(apply(logits.clone()).cpu(), torch.tensor(np.stack(want)))
+    # counts stop at 65,535
+    ops().sample_history(counts, 6, i32([4] * 3))
+    counts[6, 4] = -2                                                               # 65,534 as 16 bits
+    for _ in range(3):
+        ops().sample_count(counts, f32([6.0]), i32([4]))
+    assert int(counts[6, 4]) == -1
+
+
 @pytest.mark.parametrize("V", [97, 1000, 32768, 131072])
 def test_filtered_sample_is_the_host_sampler_s(V):
     """Top-k, top-p and min-p on the device against the host sampler (itself checked against the plain

@@ -38,10 +38,12 @@ def test_parameter_checks():
     with pytest.raises(ValueError):
         SamplingParams(top_k=0)
     assert SamplingParams().is_greedy and SamplingParams().device_ok
-    # filters run on the device (up to 2048 candidates); penalties and a bias need the host
+    # filters (up to 2048 candidates), penalties and a bias of up to 256 entries run on the device
     assert SamplingParams(temperature=1.0, top_p=0.9).device_ok and SamplingParams(temperature=1.0, top_k=2048).device_ok
     assert not SamplingParams(temperature=1.0, top_k=2049).device_ok
-    assert not SamplingParams(repetition_penalty=1.1).device_ok and not SamplingParams(logit_bias={3: 1.0}).device_ok
+    assert SamplingParams(repetition_penalty=1.1).device_ok and SamplingParams(logit_bias={3: 1.0}).device_ok
+    assert not SamplingParams(logit_bias={t: 1.0 for t in range(257)}).device_ok
+    assert SamplingParams(presence_penalty=0.5, frequency_penalty=0.25).penalties == (1.0, 0.5, 0.25)
     assert SamplingParams(temperature=1.0, top_p=0.9).device_filters == (2048, 0.9, 0.0)
     assert SamplingParams(temperature=1.0, top_k=7, min_p=0.1).device_filters == (7, 0.0, 0.1)
     assert SamplingParams(temperature=1.0, top_p=1.0).device_filters == (2048, 0.0, 0.0)
