@@ -58,20 +58,30 @@ struct SkinnyFusion {
 #define EPI_RESIDUAL 2
 #define EPI_ROPE 3               // rotate q and k, store q and the cache rows (rope_store.h)
 
-template <int MT, typename TOut, int EPI>
-__global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
+template <int MT, typename TOut, int EPI, int T>
+__global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ wp,
                                                            TOut* __restrict__ out, int M, int N, int K,
                                                            int n_steps, int out_cols, SkinnyFusion fu, RopeStore rs) {
     constexpr bool SWIGLU = EPI == EPI_SWIGLU;
-    extern __shared__ float red[];               // [NW][MT][64][4], then [NW * 4][16] for the row scale
+    static_assert(T == 1 || MT == 1, "several row groups per block only with one tile of tokens");
+    extern __shared__ float red[];               // [NW][MT * T][64][4], then [NW * 4][16] for the row scale
     const int nw = blockDim.x >> 6;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // the same for the whole wave: what depends on it is scalar
     const int li = lane & 15, g = lane >> 4;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    // tiles of this row group: [n_steps][64 lanes][8 values]
-    const bf16_t* wt = wp + ((size_t)blockIdx.x * n_steps * 64 + lane) * 8;
+    // the block's T row groups (the last block may hold fewer: it reads its last one again and drops the
+    // results); tiles of a row group: [n_steps][64 lanes][8 values]
+    const int groups = (N + 15) >> 4;
+    const int grp0 = blockIdx.x * T;
+    const int nt = min(T, groups - grp0);
+    const bf16_t* wt[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) wt[t] = wp + ((size_t)(grp0 + min((t + blockIdx.x) & (T - 1), nt - 1)) * n_steps * 64 + lane) * 8;
+    // wave t < nt finishes row group grp0 + t after the loop
+    const bool owner = wave < nt;
+    const int my_grp = grp0 + wave;
 
     // K in steps of 32; this wave's steps [s0, s1)
     const int per = (n_steps + nw - 1) / nw;
@@ -85,9 +95,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
         xok[mt] = tok < M;
         xrow[mt] = x + (size_t)min(tok, M - 1) * K + 8 * g;
     }
-    f32x4 acc[MT];
+    f32x4 acc[MT * T];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < MT * T; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     // row scale (one tile of tokens only): thread t fetches its share of the parts of token t % 16
     // (in fours where the number of parts allows 16-byte loads); the loads are in flight during
@@ -116,12 +126,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
             }
         }
     }
-    // epilogue 2: wave 0 fetches its part of the residual stream and of g before the loop
+    // epilogue 2: the wave that finishes a row group fetches its part of the residual stream and of g before the loop
     f32x4 r_in[MT], g_in = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) r_in[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    if (EPI == EPI_RESIDUAL && MT == 1 && wave == 0) {
-        const int f0 = blockIdx.x * 16 + 4 * g;
+    if (EPI == EPI_RESIDUAL && MT == 1 && owner) {
+        const int f0 = my_grp * 16 + 4 * g;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             if (f0 + r < N) g_in[r] = fu.g[f0 + r];
@@ -141,9 +151,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     TokenPlace place = {-1, 0};
     RopeAngles angles = {};
     const bool angles_early = EPI == EPI_ROPE && MT == 1 && rs.rot >= 8;
-    if (EPI == EPI_ROPE && MT == 1 && wave == 0 && li < M) {
+    if (EPI == EPI_ROPE && MT == 1 && owner && li < M) {
         place = rope_token_place(rs, li);
-        if (angles_early) angles = rope_angles(rs, li, blockIdx.x * 16 + 4 * g, g);
+        if (angles_early) angles = rope_angles(rs, li, my_grp * 16 + 4 * g, g);
     }
 
     int s = s0;
@@ -151,16 +161,40 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     // its data.  x beyond K does not exist (w is zero there): such chunks count as zero.
 #define FL_SKINNY_ITER(U)                                                                              \
     for (; s + U <= s1; s += U) {                                                                      \
-        bf16x8 a[U];                                                                                   \
-        _Pragma("unroll") for (int j = 0; j < U; ++j)                                                  \
-            a[j] = __builtin_nontemporal_load((const bf16x8*)(wt + (size_t)(s + j) * 512));            \
-        _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                            \
+        if constexpr (T == 1) {                                                                        \
+            bf16x8 a[U];                                                                               \
+            _Pragma("unroll") for (int j = 0; j < U; ++j)                                              \
+                a[j] = __builtin_nontemporal_load((const bf16x8*)(wt[0] + (size_t)(s + j) * 512));     \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                        \
+                bf16x8 b[U];                                                                           \
+                _Pragma("unroll") for (int j = 0; j < U; ++j)                                          \
+                    b[j] = (xok[mt] && (s + j) * 32 + 8 * g + 8 <= K)                                  \
+                               ? *(const bf16x8*)(xrow[mt] + (s + j) * 32) : zero;                     \
+                _Pragma("unroll") for (int j = 0; j < U; ++j)                                          \
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);   \
+            }                                                                                          \
+        } else {                                                                                       \
+            /* the same U steps of every row group in turn (U KB in a row each), x loaded once; the loads   \
+               of the next row group are issued before the products of this one (the scheduler is told to   \
+               leave that order alone: it would otherwise trade loads in flight for registers) */          \
             bf16x8 b[U];                                                                               \
+            bf16x8 a[2][U];                                                                            \
             _Pragma("unroll") for (int j = 0; j < U; ++j)                                              \
-                b[j] = (xok[mt] && (s + j) * 32 + 8 * g + 8 <= K)                                      \
-                           ? *(const bf16x8*)(xrow[mt] + (s + j) * 32) : zero;                         \
+                a[0][j] = __builtin_nontemporal_load((const bf16x8*)(wt[0] + (size_t)(s + j) * 512));  \
             _Pragma("unroll") for (int j = 0; j < U; ++j)                                              \
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);       \
+                b[j] = (xok[0] && (s + j) * 32 + 8 * g + 8 <= K)                                       \
+                           ? *(const bf16x8*)(xrow[0] + (s + j) * 32) : zero;                          \
+            _Pragma("unroll") for (int t = 0; t < T; ++t) {                                            \
+                if (t + 1 < T) {                                                                       \
+                    _Pragma("unroll") for (int j = 0; j < U; ++j)                                      \
+                        a[(t + 1) & 1][j] = __builtin_nontemporal_load(                                \
+                            (const bf16x8*)(wt[t + 1 < T ? t + 1 : 0] + (size_t)(s + j) * 512));       \
+                }                                                                                      \
+                __builtin_amdgcn_sched_barrier(0);                                                     \
+                _Pragma("unroll") for (int j = 0; j < U; ++j)                                          \
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t & 1][j], b[j], acc[t], 0, 0, 0); \
+                __builtin_amdgcn_sched_barrier(0);                                                     \
+            }                                                                                          \
         }                                                                                              \
     }
     FL_SKINNY_ITER(8)
@@ -171,8 +205,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 
     // add the waves' partial sums in wave order
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) *(f32x4*)(red + (((size_t)wave * MT + mt) * 64 + lane) * 4) = acc[mt];
-    float* ssred = red + (size_t)nw * MT * 256;                  // [MT][slices][16]
+    for (int i = 0; i < MT * T; ++i) {
+        const int slot = T == 1 ? i : ((i + blockIdx.x) & (T - 1));      // the row group that acc[i] belongs to
+        *(f32x4*)(red + (((size_t)wave * MT * T + slot) * 64 + lane) * 4) = acc[i];
+    }
+    float* ssred = red + (size_t)nw * MT * T * 256;              // [slices][16]
     if (MT == 1 && fu.in_ssq) {
         float t = 0.f;
 #pragma unroll
@@ -180,12 +217,14 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
         ssred[(threadIdx.x >> 4) * 16 + (threadIdx.x & 15)] = t;
     }
     __syncthreads();
-    if (wave == 0) {
+    if (owner) {
+        // (with T = 1 this is wave 0 and every tile of tokens; with T > 1 there is one tile of tokens and wave t takes row group t)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            f32x4 sum = *(f32x4*)(red + ((size_t)mt * 64 + lane) * 4);
+            const int mine = T == 1 ? mt : wave;
+            f32x4 sum = *(f32x4*)(red + ((size_t)mine * 64 + lane) * 4);
             for (int ww = 1; ww < nw; ++ww) {
-                const f32x4 v = *(f32x4*)(red + (((size_t)ww * MT + mt) * 64 + lane) * 4);
+                const f32x4 v = *(f32x4*)(red + (((size_t)ww * MT * T + mine) * 64 + lane) * 4);
                 sum += v;
             }
             // lane (token li, group g) holds rows 16*block + 4g .. 4g+3 of token mt*16 + li
@@ -202,11 +241,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
                 for (int r = 0; r < 4; ++r) sum[r] *= scale;
             }
             if (EPI == EPI_ROPE) {
-                const int f0 = blockIdx.x * 16 + 4 * g;
+                const int f0 = my_grp * 16 + 4 * g;
                 if (angles_early) rope_store4<true>(rs, tok, place, f0, g, sum, MT == 1 && tok < M && f0 < N, angles);
                 else rope_store4(rs, tok, place, f0, g, sum, MT == 1 && tok < M && f0 < N);
             } else if (EPI == EPI_RESIDUAL) {
-                const int f0 = blockIdx.x * 16 + 4 * g;
+                const int f0 = my_grp * 16 + 4 * g;
                 f32x4 nr;
                 float sq = 0.f;
 #pragma unroll
@@ -217,7 +256,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
                 sq += __shfl_xor(sq, 16, 64);
                 sq += __shfl_xor(sq, 32, 64);
                 if (tok < M) {
-                    if (g == 0) fu.out_ssq[(size_t)tok * gridDim.x + blockIdx.x] = sq;
+                    if (g == 0) fu.out_ssq[(size_t)tok * groups + my_grp] = sq;
                     if (f0 < N) {
                         float* pr = fu.resid + (size_t)tok * N + f0;
                         bf16_t* px = fu.xg + (size_t)tok * N + f0;
@@ -236,7 +275,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
                 f32x4 up;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) up[r] = __shfl_down(sum[r], 16, 64);      // lane g+1 holds the up rows
-                const int f0 = blockIdx.x * 8 + 2 * g;                                 // g even: features 8 b + 4 (g / 2)
+                const int f0 = my_grp * 8 + 2 * g;                                     // g even: features 8 b + 4 (g / 2)
                 if ((g & 1) == 0 && tok < M && f0 < out_cols) {
                     f32x4 act;
 #pragma unroll
@@ -249,7 +288,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
                     }
                 }
             } else {
-                const int f0 = blockIdx.x * 16 + 4 * g;
+                const int f0 = my_grp * 16 + 4 * g;
                 if (tok < M && f0 < N) {
                     TOut* p = out + (size_t)tok * N + f0;
                     if (N % 4 == 0 && f0 + 4 <= N) {
@@ -263,39 +302,69 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     }
 }
 
-static int skinny_waves(int N, int K, int nw_hint) {
+// Row groups per block.  Every block reads all of x, so with T row groups per block x crosses the chip T
+// times less often: nothing at one row, as much traffic as w itself at 16.  Against that, fewer and larger
+// blocks spread less evenly over the units.  Measured at 7B sizes (microseconds at 1 / 8 / 16 rows):
+// 384 row groups (q/k/v) T = 1: 11.3 / 13.0 / 16.3, T = 2: 10.3 / 11.1 / 12.8 (192 blocks: one per unit
+// instead of one or two); 1,792 row groups (gate/up) T = 1: 37.7 / 39.9 / 49.2, T = 2: 39.7 / 40.2 / 43.5,
+// T = 4: 41.4 / 40.8 / 42.0.  The results do not depend on T (K is split over the waves as before).
+static int skinny_tiles(int M, int N, int tiles_hint) {
+    if (M > 16) return 1;
+    if (tiles_hint > 0) return tiles_hint;
     const int groups = ceil_div(N, 16);
+    if (groups > 256 && groups <= 512) return 2;
+    if (M > 8 && groups >= 1024) return 4;
+    return 1;
+}
+
+static int skinny_waves(int N, int K, int nw_hint, int T) {
+    const int blocks = ceil_div(ceil_div(N, 16), T);
     const int n_steps = ceil_div(K, 32);
     // enough waves in flight to cover the memory latency: about 2048 and more over the chip
     int nw = 4;
-    while (nw < 16 && groups * nw < 2048) nw *= 2;
+    while (nw < 16 && blocks * nw < 2048) nw *= 2;
     if (nw_hint > 0) nw = nw_hint;
+    if (T > 1 && nw > 8) nw = 8;              // two sets of w registers: blocks of 512 threads at most
     while (nw > 1 && n_steps < nw * 2) nw /= 2;
-    return nw;
+    return nw < T ? T : nw;                   // wave t finishes row group t
 }
 
 // How many partial sums per token the row scale of a product of this shape can add.
 extern "C" int fl_gemm_skinny_scale_parts(int N, int K, int in_parts) {
-    const int slices = 4 * skinny_waves(N, K, 0);
+    int slices = 64;
+    for (int T = 1; T <= 4; T *= 2) slices = min(slices, 4 * skinny_waves(N, K, 0, T));
     return SKINNY_SCALE_LOADS * slices * ((in_parts & 3) == 0 ? 4 : 1);
 }
 
-template <int MT, typename TOut>
-static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
-                         int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs, hipStream_t stream) {
-    const int groups = ceil_div(N, 16);
+template <int MT, typename TOut, int T>
+static int launch_skinny_t(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
+                           int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs, hipStream_t stream) {
+    const int blocks = ceil_div(ceil_div(N, 16), T);
     const int n_steps = ceil_div(K, 32);
-    const int nw = skinny_waves(N, K, nw_hint);
-    const size_t lds = (size_t)nw * MT * 64 * 4 * sizeof(float) + (size_t)nw * 4 * 16 * sizeof(float);
+    const int nw = skinny_waves(N, K, nw_hint, T);
+    const size_t lds = (size_t)nw * MT * T * 64 * 4 * sizeof(float) + (size_t)nw * 4 * 16 * sizeof(float);
     if (epilogue == EPI_SWIGLU)
-        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else if (epilogue == EPI_RESIDUAL)
-        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else if (epilogue == EPI_ROPE)
-        gemm_skinny_kernel<MT, TOut, EPI_ROPE><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_ROPE, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else
-        gemm_skinny_kernel<MT, TOut, EPI_PLAIN><<<groups, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_PLAIN, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     return 0;
+}
+
+// hint: waves per block (0: chosen here) + 256 x row groups per block (0: chosen here)
+template <int MT, typename TOut>
+static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int hint,
+                         int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs, hipStream_t stream) {
+    const int nw_hint = hint & 255;
+    if constexpr (MT == 1) {
+        const int T = skinny_tiles(M, N, hint >> 8);
+        if (T == 4) return launch_skinny_t<1, TOut, 4>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream);
+        if (T == 2) return launch_skinny_t<1, TOut, 2>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream);
+    }
+    return launch_skinny_t<MT, TOut, 1>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream);
 }
 
 static int skinny_entry(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
@@ -303,7 +372,8 @@ static int skinny_entry(const void* x, const void* w_packed, void* out, int out_
                         hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
-    FL_CHECK(nw_hint >= 0 && nw_hint <= 16, "gemm_skinny: %d waves per block, at most 16", nw_hint);
+    FL_CHECK(nw_hint >= 0 && (nw_hint & 255) <= 16 && ((nw_hint >> 8) == 0 || (nw_hint >> 8) == 1 || (nw_hint >> 8) == 2 || (nw_hint >> 8) == 4),
+             "gemm_skinny: hint %d: at most 16 waves per block, and 1, 2 or 4 row groups", nw_hint);
     FL_CHECK(K % 8 == 0, "gemm_skinny: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(epilogue >= 0 && epilogue <= 3, "gemm_skinny: unknown epilogue %d", epilogue);
     FL_CHECK(epilogue != EPI_SWIGLU ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),

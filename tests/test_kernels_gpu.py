@@ -122,7 +122,40 @@ def test_gemm_skinny_against_plain(out_dtype, M, N, K):
     assert (got.double() - plain.double()).abs().max() < 2 * tol * scale
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 80, 96), (7, 37, 264), (16, 6144, 512), (12, 4112, 72), (9, 16400, 64)])
+def test_gemm_skinny_with_several_row_groups_per_block(M, N, K):
+    """One, two or four row groups per block (the last block holds fewer) and any number of waves give
+    the same numbers as long as K is split over the same number of waves; plain and SwiGLU epilogue."""
+    from flambeau_amd.kernels.packing import pack_weight
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=13), rnd(N, K, dtype=torch.bfloat16, seed=14, scale=0.05)
+    packed = pack_weight(w)
+    ref = x.double() @ w.double().T
+    for waves in (2, 4, 8):
+        outs = []
+        for groups in (1, 2, 4):
+            got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+            tuned().gemm_skinny(x, packed, got, waves + 256 * groups)
+            assert (got.double() - ref).abs().max() < 1e-5 * ref.abs().max()
+            outs.append(got)
+        if K // 32 >= 2 * waves:                      # (fewer steps than that: the kernel takes fewer waves)
+            assert torch.equal(outs[0], outs[1])
+            if waves >= 4:                            # (a block has at least one wave per row group)
+                assert torch.equal(outs[0], outs[2])
+    if N % 32 == 0:
+        gate, up = w[:N // 2].contiguous(), w[N // 2:].contiguous()
+        Wgu = tuned().prepare_gate_up(gate, up)
+        gr, ur = x.double() @ gate.double().T, x.double() @ up.double().T
+        ref_act = gr / (1 + torch.exp(-gr)) * ur
+        for groups in (1, 2, 4):
+            act = torch.full((M, N // 2), float("nan"), dtype=torch.float32, device=DEV)
+            tuned().gemm_skinny(x, Wgu.packed, act, 256 * groups, swiglu_rows=Wgu.packed_rows)
+            assert (act.double() - ref_act).abs().max() < 1e-5 * ref_act.abs().max()
+    with pytest.raises(Exception, match="row groups"):
+        tuned().gemm_skinny(x, packed, torch.empty(M, N, dtype=torch.float32, device=DEV), 256 * 3)
+
+
 @pytest.mark.parametrize("M,H,N2,I,eps", [(1, 4096, 6144, 512, 1e-5), (8, 4096, 32768, 14336, 1e-5), (16, 72, 40, 104, 1e-2),
+                                            (8, 5104, 6144, 96, 1e-5), (12, 5120, 28672, 256, 1e-5),
                                             (3, 136, 250, 40, 1e-6), (5, 64, 16, 8, 1e-5),
                                             (64, 4096, 6144, 14336, 1e-5), (17, 96, 40, 64, 1e-3), (40, 2080, 300, 160, 1e-5),
                                             (2048, 4096, 1024, 512, 1e-5), (300, 264, 152, 96, 1e-6), (129, 72, 40, 104, 1e-3),
@@ -691,6 +724,7 @@ def test_gemm_mid_refuses_what_it_cannot_do():
 
 
 @pytest.mark.parametrize("M,nh,nkv,hd,rot,ps,H", [(1, 32, 8, 128, 128, 16, 4096), (8, 4, 2, 16, 16, 8, 64), (16, 5, 5, 32, 16, 16, 80),
+                                                  (9, 33, 1, 144, 64, 16, 264),
                                                   (300, 6, 2, 64, 64, 16, 96), (2048, 32, 8, 128, 128, 16, 512),
                                                   (130, 3, 1, 48, 32, 32, 72), (70, 8, 8, 16, 16, 8, 40),
                                                   (64, 32, 8, 128, 128, 16, 4096), (17, 6, 2, 64, 32, 16, 96), (40, 5, 5, 32, 16, 8, 2048),
