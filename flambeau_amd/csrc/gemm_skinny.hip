@@ -58,13 +58,40 @@ struct SkinnyFusion {
 #define EPI_RESIDUAL 2
 #define EPI_ROPE 3               // rotate q and k, store q and the cache rows (rope_store.h)
 
-template <int MT, typename TOut, int EPI, int T>
+// x of eight steps of K for a wave's product, fetched by whole rows: load i brings rows 2 i and 2 i + 1
+// (512 bytes each, the lanes end to end, so that every cache line is asked for once and whole; a
+// 16-byte piece per row and lane touches every line of the rows in each of the eight loads), parked in
+// the wave's own piece of LDS and read back as the matrix instruction's operand.  Piece p (16 bytes) of
+// row 2 i + r lies in slot 32 r + (p + r + 2 i) % 32 of load i's kilobyte: the 16 lanes that read
+// together (one piece each of rows 0 .. 15) then hit 16 different groups of banks, and so do the 16
+// that write together.  XS = loads, rows 2 XS and beyond do not exist (rows from M on repeat row M - 1;
+// their columns of the product are never stored).
+template <int XS>
+__device__ __forceinline__ void skinny_x_staged(const bf16_t* __restrict__ x, int M, int K, int s, int lane, char* stage,
+                                                bf16x8 (&b)[8]) {
+    const int r = lane >> 5, p = lane & 31;
+    bf16x8 v[XS];
+#pragma unroll
+    for (int i = 0; i < XS; ++i)
+        v[i] = *(const bf16x8*)(x + (size_t)min(2 * i + r, M - 1) * K + (size_t)s * 32 + p * 8);
+#pragma unroll
+    for (int i = 0; i < XS; ++i)
+        *(bf16x8*)(stage + i * 1024 + (32 * r + ((p + r + 2 * i) & 31)) * 16) = v[i];
+    const int li = lane & 15, g = lane >> 4;
+    const int i = min(li >> 1, XS - 1), rr = li & 1;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        b[j] = *(const bf16x8*)(stage + i * 1024 + (32 * rr + ((4 * j + g + rr + 2 * i) & 31)) * 16);
+}
+
+template <int MT, typename TOut, int EPI, int T, int XS>
 __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ wp,
                                                            TOut* __restrict__ out, int M, int N, int K,
                                                            int n_steps, int out_cols, SkinnyFusion fu, RopeStore rs) {
     constexpr bool SWIGLU = EPI == EPI_SWIGLU;
     static_assert(T == 1 || MT == 1, "several row groups per block only with one tile of tokens");
+    static_assert(XS == 0 || MT == 1, "x through LDS only with one tile of tokens");
     extern __shared__ float red[];               // [NW][MT * T][64][4], then [NW * 4][16] for the row scale
     const int nw = blockDim.x >> 6;
     const int lane = threadIdx.x & 63;
@@ -78,7 +105,7 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
     const int nt = min(T, groups - grp0);
     const bf16_t* wt[T];
 #pragma unroll
-    for (int t = 0; t < T; ++t) wt[t] = wp + ((size_t)(grp0 + min((t + blockIdx.x) & (T - 1), nt - 1)) * n_steps * 64 + lane) * 8;
+    for (int t = 0; t < T; ++t) wt[t] = wp + ((size_t)(grp0 + min(t, nt - 1)) * n_steps * 64 + lane) * 8;
     // wave t < nt finishes row group grp0 + t after the loop
     const bool owner = wave < nt;
     const int my_grp = grp0 + wave;
@@ -156,6 +183,8 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
         if (angles_early) angles = rope_angles(rs, li, my_grp * 16 + 4 * g, g);
     }
 
+    // the wave's piece of LDS for x (behind the partial sums and the row scale's)
+    char* stage = (char*)(red + (size_t)nw * MT * T * 256 + (size_t)nw * 64) + (size_t)wave * XS * 1024;
     int s = s0;
     // iterations of U steps: every load of the iteration is issued before the first product needs
     // its data.  x beyond K does not exist (w is zero there): such chunks count as zero.
@@ -167,9 +196,13 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
                 a[j] = __builtin_nontemporal_load((const bf16x8*)(wt[0] + (size_t)(s + j) * 512));     \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                        \
                 bf16x8 b[U];                                                                           \
-                _Pragma("unroll") for (int j = 0; j < U; ++j)                                          \
-                    b[j] = (xok[mt] && (s + j) * 32 + 8 * g + 8 <= K)                                  \
-                               ? *(const bf16x8*)(xrow[mt] + (s + j) * 32) : zero;                     \
+                if constexpr (XS > 0 && U == 8) {                                                      \
+                    skinny_x_staged<XS>(x, M, K, s, lane, stage, b);                                   \
+                } else {                                                                               \
+                    _Pragma("unroll") for (int j = 0; j < U; ++j)                                      \
+                        b[j] = (xok[mt] && (s + j) * 32 + 8 * g + 8 <= K)                              \
+                                   ? *(const bf16x8*)(xrow[mt] + (s + j) * 32) : zero;                 \
+                }                                                                                      \
                 _Pragma("unroll") for (int j = 0; j < U; ++j)                                          \
                     acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);   \
             }                                                                                          \
@@ -181,9 +214,13 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
             bf16x8 a[2][U];                                                                            \
             _Pragma("unroll") for (int j = 0; j < U; ++j)                                              \
                 a[0][j] = __builtin_nontemporal_load((const bf16x8*)(wt[0] + (size_t)(s + j) * 512));  \
-            _Pragma("unroll") for (int j = 0; j < U; ++j)                                              \
-                b[j] = (xok[0] && (s + j) * 32 + 8 * g + 8 <= K)                                       \
-                           ? *(const bf16x8*)(xrow[0] + (s + j) * 32) : zero;                          \
+            if constexpr (XS > 0 && U == 8) {                                                          \
+                skinny_x_staged<XS>(x, M, K, s, lane, stage, b);                                       \
+            } else {                                                                                   \
+                _Pragma("unroll") for (int j = 0; j < U; ++j)                                          \
+                    b[j] = (xok[0] && (s + j) * 32 + 8 * g + 8 <= K)                                   \
+                               ? *(const bf16x8*)(xrow[0] + (s + j) * 32) : zero;                      \
+            }                                                                                          \
             _Pragma("unroll") for (int t = 0; t < T; ++t) {                                            \
                 if (t + 1 < T) {                                                                       \
                     _Pragma("unroll") for (int j = 0; j < U; ++j)                                      \
@@ -205,10 +242,7 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
 
     // add the waves' partial sums in wave order
 #pragma unroll
-    for (int i = 0; i < MT * T; ++i) {
-        const int slot = T == 1 ? i : ((i + blockIdx.x) & (T - 1));      // the row group that acc[i] belongs to
-        *(f32x4*)(red + (((size_t)wave * MT * T + slot) * 64 + lane) * 4) = acc[i];
-    }
+    for (int i = 0; i < MT * T; ++i) *(f32x4*)(red + (((size_t)wave * MT * T + i) * 64 + lane) * 4) = acc[i];
     float* ssred = red + (size_t)nw * MT * T * 256;              // [slices][16]
     if (MT == 1 && fu.in_ssq) {
         float t = 0.f;
@@ -302,19 +336,17 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
     }
 }
 
-// Row groups per block.  Every block reads all of x, so with T row groups per block x crosses the chip T
-// times less often: nothing at one row, as much traffic as w itself at 16.  Against that, fewer and larger
-// blocks spread less evenly over the units.  Measured at 7B sizes (microseconds at 1 / 8 / 16 rows):
-// 384 row groups (q/k/v) T = 1: 11.3 / 13.0 / 16.3, T = 2: 10.3 / 11.1 / 12.8 (192 blocks: one per unit
-// instead of one or two); 1,792 row groups (gate/up) T = 1: 37.7 / 39.9 / 49.2, T = 2: 39.7 / 40.2 / 43.5,
-// T = 4: 41.4 / 40.8 / 42.0.  The results do not depend on T (K is split over the waves as before).
+// Row groups per block.  Every block reads all of x, so with two row groups per block x crosses the chip
+// half as often; against that, fewer and larger blocks spread less evenly over the units.  Measured at 7B
+// sizes (microseconds at 1 / 8 / 16 rows, x by rows through LDS from 5 rows on): 384 row groups (q/k/v)
+// one per block 11.3 / 11.7 / 13.4, two 10.3 / 11.1 / 11.9 (192 blocks: one per unit instead of one or
+// two); 1,792 row groups (gate/up) one per block 37.7 / 38.3 / 41.8, two 39.7 / 40.8 / 41.1, four
+// 41.4 / 43.0 / 43.5.  The results do not depend on the choice (K is split over the waves as before).
 static int skinny_tiles(int M, int N, int tiles_hint) {
     if (M > 16) return 1;
     if (tiles_hint > 0) return tiles_hint;
     const int groups = ceil_div(N, 16);
-    if (groups > 256 && groups <= 512) return 2;
-    if (M > 8 && groups >= 1024) return 4;
-    return 1;
+    return groups > 256 && groups <= 512 ? 2 : 1;
 }
 
 static int skinny_waves(int N, int K, int nw_hint, int T) {
@@ -332,39 +364,49 @@ static int skinny_waves(int N, int K, int nw_hint, int T) {
 // How many partial sums per token the row scale of a product of this shape can add.
 extern "C" int fl_gemm_skinny_scale_parts(int N, int K, int in_parts) {
     int slices = 64;
-    for (int T = 1; T <= 4; T *= 2) slices = min(slices, 4 * skinny_waves(N, K, 0, T));
+    for (int T = 1; T <= 2; T *= 2) slices = min(slices, 4 * skinny_waves(N, K, 0, T));
     return SKINNY_SCALE_LOADS * slices * ((in_parts & 3) == 0 ? 4 : 1);
 }
 
-template <int MT, typename TOut, int T>
+template <int MT, typename TOut, int T, int XS>
 static int launch_skinny_t(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int nw_hint,
                            int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs, hipStream_t stream) {
     const int blocks = ceil_div(ceil_div(N, 16), T);
     const int n_steps = ceil_div(K, 32);
     const int nw = skinny_waves(N, K, nw_hint, T);
-    const size_t lds = (size_t)nw * MT * T * 64 * 4 * sizeof(float) + (size_t)nw * 4 * 16 * sizeof(float);
+    const size_t lds = (size_t)nw * MT * T * 64 * 4 * sizeof(float) + (size_t)nw * 4 * 16 * sizeof(float) + (size_t)nw * XS * 1024;
     if (epilogue == EPI_SWIGLU)
-        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else if (epilogue == EPI_RESIDUAL)
-        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else if (epilogue == EPI_ROPE)
-        gemm_skinny_kernel<MT, TOut, EPI_ROPE, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_ROPE, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     else
-        gemm_skinny_kernel<MT, TOut, EPI_PLAIN, T><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+        gemm_skinny_kernel<MT, TOut, EPI_PLAIN, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
     return 0;
 }
 
-// hint: waves per block (0: chosen here) + 256 x row groups per block (0: chosen here)
+// hint: waves per block (0: chosen here) + 256 x row groups per block (0: chosen here, 1 or 2) + 65536 if x is not to go through LDS
 template <int MT, typename TOut>
 static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K, int hint,
                          int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs, hipStream_t stream) {
     const int nw_hint = hint & 255;
     if constexpr (MT == 1) {
-        const int T = skinny_tiles(M, N, hint >> 8);
-        if (T == 4) return launch_skinny_t<1, TOut, 4>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream);
-        if (T == 2) return launch_skinny_t<1, TOut, 2>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream);
+        const int T = skinny_tiles(M, N, (hint >> 8) & 255);
+        // x through LDS from five rows on (four loads of two rows each, or eight), whole steps of K only; with
+        // fewer rows the pieces of a load lie in so few cache lines that the detour gains nothing
+        const int xs = (M <= 4 || K % 32 != 0 || (hint >> 16)) ? 0 : M <= 8 ? 4 : 8;
+#define FL_SK_T(T_)                                                                                                     \
+        switch (xs) {                                                                                                   \
+            case 4: return launch_skinny_t<1, TOut, T_, 4>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream); \
+            case 8: return launch_skinny_t<1, TOut, T_, 8>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream); \
+            default: return launch_skinny_t<1, TOut, T_, 0>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream); \
+        }
+        if (T == 2) { FL_SK_T(2) }
+        FL_SK_T(1)
+#undef FL_SK_T
     }
-    return launch_skinny_t<MT, TOut, 1>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream);
+    return launch_skinny_t<MT, TOut, 1, 0>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream);
 }
 
 static int skinny_entry(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
@@ -372,8 +414,11 @@ static int skinny_entry(const void* x, const void* w_packed, void* out, int out_
                         hipStream_t stream) {
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
-    FL_CHECK(nw_hint >= 0 && (nw_hint & 255) <= 16 && ((nw_hint >> 8) == 0 || (nw_hint >> 8) == 1 || (nw_hint >> 8) == 2 || (nw_hint >> 8) == 4),
-             "gemm_skinny: hint %d: at most 16 waves per block, and 1, 2 or 4 row groups", nw_hint);
+    {
+        const int tiles_hint = (nw_hint >> 8) & 255;
+        FL_CHECK(nw_hint >= 0 && (nw_hint & 255) <= 16 && tiles_hint <= 2 && (nw_hint >> 17) == 0,
+                 "gemm_skinny: hint %d: at most 16 waves per block, and 1 or 2 row groups", nw_hint);
+    }
     FL_CHECK(K % 8 == 0, "gemm_skinny: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(epilogue >= 0 && epilogue <= 3, "gemm_skinny: unknown epilogue %d", epilogue);
     FL_CHECK(epilogue != EPI_SWIGLU ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),

@@ -122,31 +122,31 @@ def test_gemm_skinny_against_plain(out_dtype, M, N, K):
     assert (got.double() - plain.double()).abs().max() < 2 * tol * scale
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 80, 96), (7, 37, 264), (16, 6144, 512), (12, 4112, 72), (9, 16400, 64)])
+@pytest.mark.parametrize("M,N,K", [(1, 80, 96), (7, 48, 1024), (5, 37, 264), (16, 6144, 512), (12, 4112, 72), (9, 16400, 2560), (8, 4096, 14336)])
 def test_gemm_skinny_with_several_row_groups_per_block(M, N, K):
-    """One, two or four row groups per block (the last block holds fewer) and any number of waves give
-    the same numbers as long as K is split over the same number of waves; plain and SwiGLU epilogue."""
+    """One or two row groups per block (the last block may hold one), x fetched piece by piece or by
+    rows through LDS, and any number of waves give the same numbers as long as K is split over the
+    same number of waves; plain and SwiGLU epilogue."""
     from flambeau_amd.kernels.packing import pack_weight
     x, w = rnd(M, K, dtype=torch.bfloat16, seed=13), rnd(N, K, dtype=torch.bfloat16, seed=14, scale=0.05)
     packed = pack_weight(w)
     ref = x.double() @ w.double().T
     for waves in (2, 4, 8):
         outs = []
-        for groups in (1, 2, 4):
-            got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
-            tuned().gemm_skinny(x, packed, got, waves + 256 * groups)
-            assert (got.double() - ref).abs().max() < 1e-5 * ref.abs().max()
-            outs.append(got)
+        for groups in (1, 2):
+            for direct_x in (0, 1):
+                got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+                tuned().gemm_skinny(x, packed, got, waves + 256 * groups + 65536 * direct_x)
+                assert (got.double() - ref).abs().max() < 1e-5 * ref.abs().max()
+                outs.append(got)
         if K // 32 >= 2 * waves:                      # (fewer steps than that: the kernel takes fewer waves)
-            assert torch.equal(outs[0], outs[1])
-            if waves >= 4:                            # (a block has at least one wave per row group)
-                assert torch.equal(outs[0], outs[2])
+            assert all(torch.equal(outs[0], o) for o in outs[1:])
     if N % 32 == 0:
         gate, up = w[:N // 2].contiguous(), w[N // 2:].contiguous()
         Wgu = tuned().prepare_gate_up(gate, up)
         gr, ur = x.double() @ gate.double().T, x.double() @ up.double().T
         ref_act = gr / (1 + torch.exp(-gr)) * ur
-        for groups in (1, 2, 4):
+        for groups in (1, 2):
             act = torch.full((M, N // 2), float("nan"), dtype=torch.float32, device=DEV)
             tuned().gemm_skinny(x, Wgu.packed, act, 256 * groups, swiglu_rows=Wgu.packed_rows)
             assert (act.double() - ref_act).abs().max() < 1e-5 * ref_act.abs().max()
