@@ -108,14 +108,14 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
 #pragma unroll
         for (int s = 0; s < QS; ++s) {
             const int d = min(32 * s + 8 * g, hd - 8);       // head dims beyond hd: q is zero there
-            f.xa[s] = *(const bf16x8*)(rowa + d);
-            f.xb[s] = *(const bf16x8*)(rowb + d);
+            f.xa[s] = __builtin_nontemporal_load((const bf16x8*)(rowa + d));
+            f.xb[s] = __builtin_nontemporal_load((const bf16x8*)(rowb + d));
         }
         const bf16_t* vrow = kv + cache_v_offset(cache, pv, kvh, row_of(vk), 0);
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
             const int d = min(16 * t + li, hd - 1);          // rows beyond hd are never stored
-            f.wv[t] = *(const bf16x8*)(vrow + (size_t)d * ps);
+            f.wv[t] = __builtin_nontemporal_load((const bf16x8*)(vrow + (size_t)d * ps));
         }
     };
     auto compute = [&](const Chunk& f, int c) {
