@@ -7,7 +7,8 @@
 //    order, tiles of one row group following each other along k.  A wave's load instruction
 //    then reads one whole kilobyte, and its 8 loads per iteration 8 KB in a row (measured:
 //    6.2 TB/s against 5.3 TB/s for 16 row pieces of 64 B per instruction);
-//  * a block owns 16 consecutive output features (a row group); its NW waves split K between
+//  * a block owns 16 consecutive output features (a row group), or two such groups where that
+//    spreads the blocks better over the units (skinny_tiles); its NW waves split K between
 //    them and add their partial sums through LDS in a fixed order (no atomics: the result
 //    does not depend on timing);
 //  * a wave keeps 8 16-byte loads of w in flight per lane before it consumes them; w is loaded
@@ -15,7 +16,8 @@
 //  * the arithmetic is v_mfma_f32_16x16x32_bf16 with w as the A operand (16 features x 32 k)
 //    and x as the B operand (32 k x 16 tokens): C[feature][token] leaves each lane with four
 //    consecutive features of one token, i.e. one 16-byte store.  Rows of x beyond M are not
-//    loaded.  With MT > 1 the same w registers feed MT token tiles.
+//    loaded.  With MT > 1 the same w registers feed MT token tiles.  Every block reads all of x:
+//    from 5 rows on that is worth fetching by whole rows (skinny_x_staged);
 //
 // Two fusions with the norm around a product save a kernel each in a decode step:
 //  * epilogue 2 (residual): instead of storing the product the block adds it to the residual
