@@ -55,6 +55,7 @@ struct SkinnyFusion {
 };
 
 #define SKINNY_SCALE_LOADS 4     // loads of partial sums per thread for the row scale
+#define SKINNY_LDS_MAX (160 * 1024)
 #define EPI_PLAIN 0
 #define EPI_SWIGLU 1
 #define EPI_RESIDUAL 2
@@ -377,14 +378,24 @@ static int launch_skinny_t(const bf16_t* x, const bf16_t* wp, TOut* out, int M, 
     const int n_steps = ceil_div(K, 32);
     const int nw = skinny_waves(N, K, nw_hint, T);
     const size_t lds = (size_t)nw * MT * T * 64 * 4 * sizeof(float) + (size_t)nw * 4 * 16 * sizeof(float) + (size_t)nw * XS * 1024;
-    if (epilogue == EPI_SWIGLU)
-        gemm_skinny_kernel<MT, TOut, EPI_SWIGLU, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
-    else if (epilogue == EPI_RESIDUAL)
-        gemm_skinny_kernel<MT, TOut, EPI_RESIDUAL, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
-    else if (epilogue == EPI_ROPE)
-        gemm_skinny_kernel<MT, TOut, EPI_ROPE, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
-    else
-        gemm_skinny_kernel<MT, TOut, EPI_PLAIN, T, XS><<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);
+    // (a launch may ask for more than 64 KB of LDS once the kernel has been told so)
+#define FL_SK_LAUNCH(EPI_)                                                                                         \
+    {                                                                                                              \
+        auto* kernel = gemm_skinny_kernel<MT, TOut, EPI_, T, XS>;                                                  \
+        static bool raised = false;                                                                                \
+        if (lds > 64 * 1024 && !raised) {                                                                          \
+            const hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                                     SKINNY_LDS_MAX);                                              \
+            FL_CHECK(e == hipSuccess, "gemm_skinny: hipFuncSetAttribute failed: %s", hipGetErrorString(e));         \
+            raised = true;                                                                                         \
+        }                                                                                                          \
+        kernel<<<blocks, nw * 64, lds, stream>>>(x, wp, out, M, N, K, n_steps, out_cols, fu, rs);                  \
+    }
+    if (epilogue == EPI_SWIGLU) FL_SK_LAUNCH(EPI_SWIGLU)
+    else if (epilogue == EPI_RESIDUAL) FL_SK_LAUNCH(EPI_RESIDUAL)
+    else if (epilogue == EPI_ROPE) FL_SK_LAUNCH(EPI_ROPE)
+    else FL_SK_LAUNCH(EPI_PLAIN)
+#undef FL_SK_LAUNCH
     return 0;
 }
 
@@ -397,7 +408,8 @@ static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, in
         const int T = skinny_tiles(M, N, (hint >> 8) & 255);
         // x through LDS from five rows on (four loads of two rows each, or eight), whole steps of K only; with
         // fewer rows the pieces of a load lie in so few cache lines that the detour gains nothing
-        const int xs = (M <= 4 || K % 32 != 0 || (hint >> 16)) ? 0 : M <= 8 ? 4 : 8;
+        int xs = (M <= 4 || K % 32 != 0 || (hint >> 16)) ? 0 : M <= 8 ? 4 : 8;
+        if ((size_t)skinny_waves(N, K, nw_hint, T) * (T * 1024 + 256 + xs * 1024) > SKINNY_LDS_MAX) xs = 0;
 #define FL_SK_T(T_)                                                                                                     \
         switch (xs) {                                                                                                   \
             case 4: return launch_skinny_t<1, TOut, T_, 4>(x, wp, out, M, N, K, nw_hint, epilogue, out_cols, fu, rs, stream); \
