@@ -1,7 +1,10 @@
 // Split-K grouped-query attention over the paged cache for single query rows (decode rows, and
 // the rows of short prompt portions): bf16 storage, float arithmetic, matrix cores.
 //
-// Work item = (query row, kv head, split); a query row comes as (row, position, request, 0).  A
+// Work item = (query row, kv head, split); a query row comes as (row, position, request, 0), or, with
+// splits of its own, once per split as (row, position, request, split + 256 * splits): the caller
+// then gives long contexts more splits than short ones, and the blocks take about equally long
+// (with one number of splits for all, the longest context of a ragged batch ends the kernel alone).  A
 // block of four waves handles the (up to 16) query heads that share one kv head over the keys of
 // its split, 32 keys per wave at a time:
 //
@@ -45,10 +48,15 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
     __shared__ float s_m[DEC_WAVES][16], s_l[DEC_WAVES][16];
     __shared__ f32x4 s_o[DEC_WAVES - 1][DT][64];     // wave 0 keeps its own in registers
 
-    const int item = blockIdx.x;
-    const int kvh = blockIdx.y / q_tiles, qt = blockIdx.y % q_tiles;
-    const int split = blockIdx.z;
+    // (the items are the slow index of the grid: the places of a list that no row uses come last)
+    const int item = blockIdx.y;
+    const int kvh = blockIdx.x / q_tiles, qt = blockIdx.x % q_tiles;
     const int4 it = items[item];
+    if (it.x < 0) return;                              // a place in the list that no row uses
+    // an item with splits of its own says which split it is; its partial result lies in the slot of the item
+    const bool own_splits = it.w != 0;
+    const int split = own_splits ? (it.w & 255) : (int)blockIdx.z;
+    if (own_splits) n_split = it.w >> 8;
     const int token = it.x, p = it.y;
     const int hd = cache.head_dim, ps = cache.page_size;
     const int G = nh / cache.n_kv_heads;
@@ -248,7 +256,7 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
                 }
             }
         } else if (head_ok) {
-            const size_t slot = ((size_t)item * nh + head) * n_split + split;
+            const size_t slot = own_splits ? (size_t)item * nh + head : ((size_t)item * nh + head) * n_split + split;
             if (g == 0) { part_ml[slot * 2] = mm; part_ml[slot * 2 + 1] = ll; }
             float* prow = part_o + slot * HDP;
 #pragma unroll
@@ -274,6 +282,22 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
                       n_split);
 }
 
+// The same for items with splits of their own, which lie nh slots apart: one block per (row, head); firsts[r] =
+// (row, position, request, index of the row's first item).
+__global__ __launch_bounds__(256) void attn_decode_merge_items_kernel(const float* __restrict__ part_o,
+                                                                      const float* __restrict__ part_ml,
+                                                                      bf16_t* __restrict__ out,
+                                                                      const int4* __restrict__ items,
+                                                                      const int4* __restrict__ firsts, int nh,
+                                                                      int hd, int hdp) {
+    const int head = blockIdx.y;
+    const int4 row = firsts[blockIdx.x];
+    const int first = row.w, n_split = items[first].w >> 8;
+    if (n_split <= 1) return;
+    attn_merge_splits(part_o, part_ml, out + ((size_t)row.x * nh + head) * hd, (size_t)first * nh + head, hd, hdp, n_split,
+                      (size_t)nh);
+}
+
 extern "C" int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats,
                                         long* ml_floats) {
     const int hdp = ceil_div(hd, 32) * 32;
@@ -285,7 +309,8 @@ extern "C" int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split
 static int attn_decode_launch(const char* who, const void* q, void* out, float* part_o, float* part_ml,
                               const void* cache_base, const int* items, int n_items, const int* block_table,
                               int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
-                              float scale, int window, int n_split, hipStream_t stream) {
+                              float scale, int window, int n_split, hipStream_t stream, bool own_splits = false,
+                              const int* firsts = nullptr, int n_rows = 0) {
     FL_CHECK(n_items >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "%s: bad head counts %d/%d", who, nh, nkv);
     FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "%s: head size %d must be a multiple of 8 up to 256", who, hd);
     FL_CHECK(page_size % 8 == 0, "%s: page size %d must be a multiple of 8", who, page_size);
@@ -300,7 +325,8 @@ static int attn_decode_launch(const char* who, const void* q, void* out, float* 
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
     const int G = nh / nkv;
     const int q_tiles = ceil_div(G, 16);
-    dim3 grid(n_items, nkv * q_tiles, n_split);
+    FL_CHECK(n_items <= 65535, "%s: %d items, at most 65535", who, n_items);
+    dim3 grid(nkv * q_tiles, n_items, own_splits ? 1 : n_split);
     const int hdp = ceil_div(hd, 32) * 32;
 #define FL_DEC(HDP_)                                                                                  \
     attn_decode_kernel<HDP_><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, part_ml, c,       \
@@ -318,7 +344,15 @@ static int attn_decode_launch(const char* who, const void* q, void* out, float* 
     }
 #undef FL_DEC
     FL_LAUNCH_CHECK();
-    if (n_split > 1) {
+    if (own_splits) {
+        if (firsts && n_rows > 0) {              // (without: the caller knows that no row has more than one split)
+            FL_CHECK((uintptr_t)firsts % 16 == 0, "%s: the rows' first items must be 16-byte aligned", who);
+            dim3 mg(n_rows, nh);
+            attn_decode_merge_items_kernel<<<mg, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, (const int4*)items,
+                                                                   (const int4*)firsts, nh, hd, hdp);
+            FL_LAUNCH_CHECK();
+        }
+    } else if (n_split > 1) {
         dim3 mg(n_items, nh);
         attn_decode_merge_kernel<<<mg, 256, 0, stream>>>(
             part_o, part_ml, (bf16_t*)out, (const int4*)items, nh, hd, hdp, n_split);
@@ -333,6 +367,20 @@ extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* pa
                               float scale, int window, int n_split, hipStream_t stream) {
     return attn_decode_launch("attn_decode", q, out, part_o, part_ml, cache_base, items, n_items, block_table, max_blocks,
                               nh, nkv, hd, page_size, n_pages, scale, window, n_split, stream);
+}
+
+// Items with splits of their own: items[i] = (row, position, request, split + 256 * splits), the splits of
+// a row one after the other from split 0 on (up to 255), row < 0 for a place that is not used.  part_o
+// holds n_items * nh * (head size rounded up to 32) floats, part_ml n_items * nh * 2.  firsts[r] = (row,
+// position, request, index of the row's first item) for the n_rows rows; without it no row has more
+// than one split (a list with a place per row and no more) and the kernel that merges is left out.
+extern "C" int fl_attn_decode_items(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
+                                    const int* items, int n_items, const int* block_table, int max_blocks, int nh,
+                                    int nkv, int hd, int page_size, int n_pages, float scale, int window,
+                                    const int* firsts, int n_rows, hipStream_t stream) {
+    FL_CHECK(!firsts || (part_o && part_ml), "attn_decode_items: needs a workspace");
+    return attn_decode_launch("attn_decode_items", q, out, part_o, part_ml, cache_base, items, n_items, block_table, max_blocks,
+                              nh, nkv, hd, page_size, n_pages, scale, window, 1, stream, true, firsts, n_rows);
 }
 
 // ---- the same without any allocation: the splits' partial results go to an array that is part of

@@ -8,16 +8,18 @@
 #pragma once
 #include "common.h"
 
+// Split s lies in slot base + s * stride.
 __device__ __forceinline__ void attn_merge_splits(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                  bf16_t* __restrict__ out_row, size_t base, int hd, int hdp, int n_split) {
+                                                  bf16_t* __restrict__ out_row, size_t base, int hd, int hdp, int n_split,
+                                                  size_t stride = 1) {
     __shared__ float s_f[256];       // exp(m_s - m_max) per split (n_split <= 256)
     __shared__ float s_l[256];
     __shared__ float s_inv;
     const int t = threadIdx.x;
     float ms = -INFINITY, ls = 0.f;
     if (t < n_split) {
-        ms = part_ml[(base + t) * 2];
-        ls = part_ml[(base + t) * 2 + 1];
+        ms = part_ml[(base + t * stride) * 2];
+        ls = part_ml[(base + t * stride) * 2 + 1];
     }
     s_f[t] = ms;
     __syncthreads();
@@ -42,11 +44,11 @@ __device__ __forceinline__ void attn_merge_splits(const float* __restrict__ part
         for (; s + 8 <= n_split; s += 8) {
             float v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = part_o[(base + s + u) * hdp + d];
+            for (int u = 0; u < 8; ++u) v[u] = part_o[(base + (s + u) * stride) * hdp + d];
 #pragma unroll
             for (int u = 0; u < 8; ++u) acc += v[u] * s_f[s + u];
         }
-        for (; s < n_split; ++s) acc += part_o[(base + s) * hdp + d] * s_f[s];
+        for (; s < n_split; ++s) acc += part_o[(base + s * stride) * hdp + d] * s_f[s];
         out_row[d] = (bf16_t)(acc * inv);
     }
 }

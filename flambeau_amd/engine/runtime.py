@@ -143,6 +143,16 @@ class Runtime:
             return tuned.attention(self, q, out, kv, step, table, n_heads, scale, window)
         return ops.attn_plain(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window)
 
+    def attention_metadata(self, batch, mixers):
+        """The attention kernels' work lists for a batch (integer arrays for the step's upload): the
+        rows and tiles, and for the tuned single-row kernel the rows with splits of their own, one
+        list per shape (blocks per row, window) among ``mixers``."""
+        from ..kernels import tuned
+        shapes = ()
+        if self.tuned:
+            shapes = sorted({(tuned.decode_blocks_per_row(m.n_heads, m.n_kv_heads), m.window or 0) for m in mixers})
+        return tuned.attention_metadata(batch, shapes)
+
     def attention_splits(self, batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int):
         """What the attention kernels of this runtime decide from the contexts' lengths (part of a
         recorded step's key); nothing for the plain kernels."""

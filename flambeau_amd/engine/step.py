@@ -55,6 +55,8 @@ class ModelRunner:
         self.manager = CacheManager(self.storage.group_specs, n_pages, page_size, max_slots, self.max_seq_len)
         self.max_logit_rows = max_logit_rows or self.rt.max_batch_tokens
         self._mixer_classes = model.mixer_classes()
+        by_class = getattr(model, "mixers_by_class", lambda: {})()
+        self._mixers_of = {c: by_class.get(c, []) for c in self._mixer_classes}
         self._meta_capacity = 0
         self._meta_host = None
         self._meta_dev = None
@@ -196,7 +198,10 @@ class ModelRunner:
                  ("logit_rows", np.asarray(rows, dtype=np.int32))]
         parts += [(f"table{g}", t) for g, t in enumerate(tables)]
         for cls in self._mixer_classes:
-            for name, arr in cls.step_metadata(batch).items():
+            # (a class that wants to see its mixers, for their sizes, has step_metadata_for)
+            wanted = (cls.step_metadata_for(batch, self._mixers_of[cls]) if hasattr(cls, "step_metadata_for")
+                      else cls.step_metadata(batch))
+            for name, arr in wanted.items():
                 parts.append(("extra:" + name, np.ascontiguousarray(arr, dtype=np.int32)))
         return batch, parts
 

@@ -40,6 +40,7 @@ register_signatures({
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, P, I, P],
     "fl_attn_prefill_splits": [I, I, I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
+    "fl_attn_decode_items": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P, I, P],
 })
 
 SKINNY_MAX_ROWS = 64     # rows the decode kernels take
@@ -463,18 +464,23 @@ def prepare_gate_up(gate: torch.Tensor, up: torch.Tensor) -> Weight:
 # Rows of portions up to this length are treated as single query rows by the split-K kernel;
 # longer portions go to the tiled prefill kernel.
 SHORT_PORTION = 8
-DECODE_TARGET_BLOCKS = 512           # two blocks per compute unit (measured best at 1, 8 and 64 rows)
+DECODE_TARGET_BLOCKS = 512           # two blocks per compute unit
+DECODE_EVEN_BLOCKS = 256             # one per unit: enough when all rows have about the same number of keys
 DECODE_MIN_KEYS_PER_SPLIT = 128
+DECODE_MAX_SPLITS = 64
 
 
 PREFILL_TILE = 64        # query tokens per block of the tiled kernel
 
 
-def attention_metadata(batch) -> dict:
+def attention_metadata(batch, shapes=()) -> dict:
     """Work lists for the attention kernels of one batch: ``attn_rows`` = (row, position, request,
     0) of the rows that run as single queries (decode rows and rows of short portions);
     ``attn_tiles`` = (request, first row, rows, index of the first row among all rows of tiles) for
-    every 64 rows of the longer portions."""
+    every 64 rows of the longer portions.  For every ``(blocks per row, window)`` in ``shapes`` (blocks
+    that the single-row kernel runs per row and split: kv heads x tiles of 16 query heads) a list
+    ``attn_items/<blocks>/<window>`` of the same rows with splits of their own and a list
+    ``attn_item_rows/<blocks>/<window>`` of where each row's items begin (``balanced_items``)."""
     import numpy as np
     rows, tiles = [], []
     n_tile_rows = 0
@@ -486,8 +492,74 @@ def attention_metadata(batch) -> dict:
                 cnt = min(PREFILL_TILE, ql - off)
                 tiles.append((s, q0 + off, cnt, n_tile_rows))
                 n_tile_rows += cnt
-    return {"attn_rows": np.asarray(rows, dtype=np.int32).reshape(-1, 4),
-            "attn_tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 4)}
+    rows = np.asarray(rows, dtype=np.int32).reshape(-1, 4)
+    out = {"attn_rows": rows, "attn_tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 4)}
+    for per_row, window in shapes:
+        out[f"attn_items/{per_row}/{window}"], out[f"attn_item_rows/{per_row}/{window}"] = balanced_items(rows, per_row, window)
+    return out
+
+
+def decode_blocks_per_row(n_heads: int, n_kv_heads: int) -> int:
+    return n_kv_heads * -(-(n_heads // n_kv_heads) // 16)
+
+
+def decode_item_budget(n_rows: int, blocks_per_row: int) -> int:
+    """Places in the list of items for ``n_rows`` single rows: four per row, and what gives the chip
+    ``DECODE_TARGET_BLOCKS`` blocks at least.  Depends on the batch's shape only, so a recorded step
+    keeps its grid while the contexts grow; places that a step does not use cost next to nothing
+    (their blocks come last and end at once)."""
+    return max(n_rows, min(max(DECODE_TARGET_BLOCKS // max(1, blocks_per_row), 4 * n_rows), n_rows * DECODE_MAX_SPLITS))
+
+
+def balanced_items(rows, blocks_per_row: int, window: int = 0, budget: int | None = None):
+    """``rows`` (row, position, request, 0) with splits of their own: every row gets splits in
+    proportion to the keys it sees (a split of 128 keys at least, 64 splits at most), so that the blocks
+    of a ragged batch take about equally long.  Returns ``(items, firsts)``: ``items`` = (row,
+    position, request, split + 256 * splits), a row's splits one after the other, the list filled up
+    to ``decode_item_budget`` with row -1; ``firsts`` = (row, position, request, index of the row's
+    first item), one per row, for the kernel that merges."""
+    import numpy as np
+    n = rows.shape[0]
+    if budget is None:
+        budget = decode_item_budget(n, blocks_per_row)
+    items = np.full((budget, 4), -1, dtype=np.int32)
+    firsts = rows.copy()
+    if n == 0:
+        return items, firsts
+    keys = rows[:, 1].astype(np.int64) + 1
+    if window:
+        keys = np.minimum(keys, window)
+    most = np.minimum(-(-keys // DECODE_MIN_KEYS_PER_SPLIT), DECODE_MAX_SPLITS)
+    # How many places to use.  Rows of about one length: a block per unit is enough (measured at 1 to 64
+    # rows of 2,100 keys: 256 blocks, or one per row and kv head if that is more, beat 512 and 1,024).  A
+    # ragged batch: all places, since many short blocks spread over the units as they finish (55 rows of
+    # 128 to 4,600 keys: 136 us with a place per row, 100 with two, 94 with four per row).
+    ragged = int(keys.max()) * n > 1.5 * int(keys.sum())
+    use = budget if ragged else min(budget, max(n, DECODE_EVEN_BLOCKS // max(1, blocks_per_row)))
+    splits = np.clip(keys * use // max(int(keys.sum()), 1), 1, most)
+    # what rounding down and the caps left over goes to the rows whose splits are longest; what the
+    # least of one split per row took too much comes from the rows whose splits are shortest
+    left = use - int(splits.sum())
+    while left > 0:
+        room = splits < most
+        if not room.any():
+            break
+        take = np.argsort(-np.where(room, keys / splits, 0.0), kind="stable")[:left]
+        take = take[room[take]]
+        splits[take] += 1
+        left -= take.size
+    while left < 0:
+        give = np.argsort(np.where(splits > 1, keys / splits, np.inf), kind="stable")[:-left]
+        give = give[splits[give] > 1]
+        splits[give] -= 1
+        left += give.size
+    first = np.concatenate(([0], np.cumsum(splits)[:-1]))
+    which = np.repeat(np.arange(n), splits)
+    total = int(splits.sum())
+    items[:total, :3] = rows[which, :3]
+    items[:total, 3] = (np.arange(total) - first[which]) + 256 * splits[which]
+    firsts[:, 3] = first
+    return items, firsts
 
 
 def decode_splits(n_items: int, n_kv_heads: int, group: int, max_ctx: int) -> int:
@@ -499,24 +571,30 @@ def decode_splits(n_items: int, n_kv_heads: int, group: int, max_ctx: int) -> in
     return int(min(by_blocks, by_keys, 64))
 
 
-def attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, part_o=None, part_ml=None):
+def attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, part_o=None, part_ml=None, firsts=None):
     """Attention of single query rows; ``rows[i] = (row of q and out, position, index of the request's
-    row in ``table``, 0)``."""
+    row in ``table``, 0)``, every row's keys in ``n_split`` parts; or, with ``n_split`` = 0, rows with
+    splits of their own as ``balanced_items`` lists them, with its list ``firsts`` of where each row's
+    items begin (``None``: no row has more than one split, nothing is merged)."""
     n = q.shape[0]
     hd = cache.head_dim
     n_items = rows.shape[0]
-    if n_split > 1:
-        hdp = -(-hd // 32) * 32
-        need_o, need_ml = n_items * n_heads * n_split * hdp, n_items * n_heads * n_split * 2
-        if part_o is None or part_o.numel() < need_o or part_ml is None or part_ml.numel() < need_ml:
+    hdp = -(-hd // 32) * 32
+    if n_split > 1 or (n_split == 0 and firsts is not None):
+        slots = n_items * n_heads * max(n_split, 1)
+        if part_o is None or part_o.numel() < slots * hdp or part_ml is None or part_ml.numel() < slots * 2:
             raise KernelError("attn_decode: workspace too small for the splits")
-    call("fl_attn_decode", _check(q, "attn.q", torch.bfloat16, (n, n_heads * hd)),
-         _check(out, "attn.out", torch.bfloat16, (n, n_heads * hd)),
-         _check(part_o, "attn.part_o", torch.float32) if part_o is not None else None,
-         _check(part_ml, "attn.part_ml", torch.float32) if part_ml is not None else None,
-         _check(cache.pool, "attn.cache", torch.bfloat16), _check(rows, "attn.rows", torch.int32, (n_items, 4)), n_items,
-         _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads,
-         hd, cache.page_size, cache.n_pages, float(scale), int(window), int(n_split), stream_handle())
+    head = (_check(q, "attn.q", torch.bfloat16, (n, n_heads * hd)), _check(out, "attn.out", torch.bfloat16, (n, n_heads * hd)),
+            _check(part_o, "attn.part_o", torch.float32) if part_o is not None else None,
+            _check(part_ml, "attn.part_ml", torch.float32) if part_ml is not None else None,
+            _check(cache.pool, "attn.cache", torch.bfloat16), _check(rows, "attn.rows", torch.int32, (n_items, 4)), n_items,
+            _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads,
+            hd, cache.page_size, cache.n_pages, float(scale), int(window))
+    if n_split == 0:
+        call("fl_attn_decode_items", *head, _check(firsts, "attn.firsts", torch.int32, (None, 4)) if firsts is not None else None,
+             firsts.shape[0] if firsts is not None else 0, stream_handle())
+    else:
+        call("fl_attn_decode", *head, int(n_split), stream_handle())
     return out
 
 
@@ -567,9 +645,11 @@ def prefill_supported(cache, table) -> bool:
     return decode_supported(cache) and ps >= 8 and ps & (ps - 1) == 0 and table.shape[1] <= PREFILL_MAX_PAGES
 
 
-def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int):
+def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int, with_items: bool = True):
     """``(parts of the keys for the tiled kernel, for the single-row kernel)`` for a batch: everything
-    that ``attention`` decides from the contexts' lengths (the rest follows from the batch's shape)."""
+    that ``attention`` decides from the contexts' lengths (the rest follows from the batch's shape).
+    ``with_items``: the single rows come with splits of their own (``balanced_items``), which are
+    data of the step and decide nothing here (0 stands for that)."""
     n_tiles = sum(-(-ql // PREFILL_TILE) for ql in batch.q_lens if ql > SHORT_PORTION)
     n_items = sum(ql for ql in batch.q_lens if ql <= SHORT_PORTION)
     p_split = n_split = 1
@@ -577,12 +657,12 @@ def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window
         # few tiles before a long context: the keys are split too, so that the chip has blocks enough
         longest = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + PREFILL_TILE)
         p_split = attn_prefill_splits(n_tiles, n_heads, n_kv_heads, head_dim, longest)
-    if n_items:
+    if n_items and not with_items:
         max_ctx = batch.ctx_bound or batch.max_ctx_len
         if window:
             max_ctx = min(max_ctx, window + 32)
         n_split = decode_splits(n_items, n_kv_heads, n_heads // n_kv_heads, max_ctx)
-    return p_split, n_split
+    return p_split, (0 if n_items and with_items else n_split)
 
 
 def attention(rt, q, out, cache, step, table, n_heads, scale, window):
@@ -593,10 +673,12 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
     batch = step.host
     if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table)):
         return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
+    items = step.extra.get(f"attn_items/{decode_blocks_per_row(n_heads, cache.n_kv_heads)}/{window or 0}")
     key = ("attention_splits", n_heads, cache.n_kv_heads, cache.head_dim, window)
     splits = step.scratch.get(key)
     if splits is None:
-        splits = step.scratch[key] = attention_splits(batch, n_heads, cache.n_kv_heads, cache.head_dim, window)
+        splits = step.scratch[key] = attention_splits(batch, n_heads, cache.n_kv_heads, cache.head_dim, window,
+                                                       with_items=items is not None)
     p_split, n_split = splits
     if tiles.shape[0]:
         p_o = p_ml = None
@@ -606,7 +688,20 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
             p_o = rt.buffer("attn_tile_part_o", n_rows * n_heads * p_split, hdp, torch.float32, max_rows=1 << 24)
             p_ml = rt.buffer("attn_tile_part_ml", n_rows * n_heads * p_split, 2, torch.float32, max_rows=1 << 24)
         attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window, n_split=p_split, part_o=p_o, part_ml=p_ml)
-    if rows.shape[0]:
+    if rows.shape[0] and items is not None:
+        # rows with splits of their own; the list's length follows from the number of rows alone
+        # (a list with a place per row and no more: no row is ever split, nothing to merge)
+        firsts = step.extra.get(f"attn_item_rows/{decode_blocks_per_row(n_heads, cache.n_kv_heads)}/{window or 0}")
+        if items.shape[0] <= rows.shape[0]:
+            firsts = None
+        part_o = part_ml = None
+        if firsts is not None:
+            hdp = -(-cache.head_dim // 32) * 32
+            slots = items.shape[0] * n_heads
+            part_o = rt.buffer("attn_part_o", slots, hdp, torch.float32, max_rows=1 << 24)
+            part_ml = rt.buffer("attn_part_ml", slots, 2, torch.float32, max_rows=1 << 24)
+        attn_decode(q, out, cache, items, table, n_heads, scale, window, 0, part_o, part_ml, firsts=firsts)
+    elif rows.shape[0]:
         part_o = part_ml = None
         if n_split > 1:
             hdp = -(-cache.head_dim // 32) * 32

@@ -150,12 +150,15 @@ class DecoderModel:
         return tuple(m.step_signature(batch) for m in self._signature_mixers)
 
     def mixer_classes(self):
-        seen = []
+        return list(self.mixers_by_class())
+
+    def mixers_by_class(self) -> dict:
+        """The model's mixers, grouped by their class in the order of first appearance."""
+        found = {}
         for b in self.blocks:
             for m in getattr(b, "mixers", lambda: [])():
-                if type(m) not in seen:
-                    seen.append(type(m))
-        return seen
+                found.setdefault(type(m), []).append(m)
+        return found
 
     # ------------------------------------------------------------ the forward pass of one batch
     def forward(self, step, caches, max_logit_rows: int):

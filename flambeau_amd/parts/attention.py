@@ -62,6 +62,10 @@ class PagedGQAAttention(Mixer):
         from ..kernels import tuned
         return tuned.attention_metadata(batch)
 
+    @classmethod
+    def step_metadata_for(cls, batch, mixers):
+        return mixers[0].rt.attention_metadata(batch, mixers) if mixers else cls.step_metadata(batch)
+
     def bind(self, weights, rt):
         self.rt = rt
         w_qkv = torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0)

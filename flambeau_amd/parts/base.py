@@ -254,7 +254,10 @@ class Mixer(Part):
     @classmethod
     def step_metadata(cls, batch: HostBatch) -> dict:
         """Integer arrays (numpy int32) this kind of mixer wants on the device for the batch,
-        uploaded with the rest of the step's metadata and found in ``StepState.extra``."""
+        uploaded with the rest of the step's metadata and found in ``StepState.extra``.  A class
+        whose arrays depend on its mixers' sizes defines ``step_metadata_for(cls, batch, mixers)``
+        (``mixers``: the model's mixers of this class) instead; the shapes of the arrays may depend
+        on the batch's shape only."""
         return {}
 
     def step_signature(self, batch: HostBatch):

@@ -596,6 +596,44 @@ def test_attn_decode_against_plain_and_reference(nh, nkv, hd, ps, window, n_spli
     assert (out.double() - plain.double()).abs().max() < 1.5e-2 * top
 
 
+@pytest.mark.parametrize("nh,nkv,hd,ps,window", [(32, 8, 128, 16, 0), (4, 2, 16, 8, 16), (6, 1, 24, 16, 0), (20, 1, 64, 8, 0),
+                                                (8, 4, 256, 32, 100), (40, 2, 32, 16, 0)])
+def test_attn_decode_with_splits_per_row(nh, nkv, hd, ps, window):
+    """Rows with splits of their own (long contexts many, short ones one, unused places in the list):
+    the reference's result, and exactly the uniform kernel's where a row has one split."""
+    seqs = [(1500, 1), (33, 1), (ps * 3, 1), (1, 1), (257, 3), (640, 2), (32, 1), (31, 1)]
+    case = build_attention_case(torch.bfloat16, nh, nkv, hd, ps, seqs, seed=9)
+    n = case["n"]
+    scale = 1 / math.sqrt(hd)
+    q2 = case["q"].reshape(n, nh * hd)
+    rows = decode_rows(case, range(n))
+    per_row = tuned().decode_blocks_per_row(nh, nkv)
+    items_host, firsts_host = tuned().balanced_items(rows.cpu().numpy(), per_row, window)
+    splits = {int(r): int(w) >> 8 for r, _, _, w in items_host if r >= 0}
+    assert len(items_host) == tuned().decode_item_budget(n, per_row) and set(splits) == set(range(n))
+    assert (max(splits.values()) > 1 or 0 < window < 256) and min(splits.values()) == 1
+    assert (items_host[:, 0] < 0).any() == (sum(splits.values()) < len(items_host))
+    items, firsts = torch.tensor(items_host, device=DEV), torch.tensor(firsts_host, device=DEV)
+    assert all(items_host[f, 0] == r and items_host[f, 3] & 255 == 0 for r, _, _, f in firsts_host)
+    hdp = -(-hd // 32) * 32
+    part_o = torch.full((len(items_host) * nh * hdp,), float("nan"), dtype=torch.float32, device=DEV)
+    part_ml = torch.full((len(items_host) * nh * 2,), float("nan"), dtype=torch.float32, device=DEV)
+    out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    tuned().attn_decode(q2, out, case["cache"], items, case["table"], nh, scale, window, 0, part_o, part_ml, firsts=firsts)
+    ref = attention_case_ref(case, scale, window)
+    assert (out.double().reshape(n, nh, hd) - ref).abs().max() < 1e-2 * ref.abs().max()
+    whole = torch.empty_like(out)
+    tuned().attn_decode(q2, whole, case["cache"], rows, case["table"], nh, scale, window, 1)
+    one = [r for r, k in splits.items() if k == 1]
+    assert torch.equal(out[one], whole[one])
+    # a list with a place per row: nothing to merge, no workspace
+    plain_items = rows.clone()
+    plain_items[:, 3] = 256
+    again = torch.full_like(out, float("nan"))
+    tuned().attn_decode(q2, again, case["cache"], plain_items, case["table"], nh, scale, window, 0)
+    assert torch.equal(again, whole)
+
+
 def test_attn_decode_subset_of_rows_leaves_the_others_alone():
     nh, nkv, hd, ps = 8, 2, 64, 16
     case = build_attention_case(torch.bfloat16, nh, nkv, hd, ps, [(40, 4), (90, 1)], seed=4)
