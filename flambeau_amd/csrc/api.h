@@ -139,7 +139,7 @@ int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, cons
 // fl_attn_decode with splits per row: items[i] = (row, position, request, split + 256 * splits), a row's
 // splits one after the other from split 0 on (up to 255 of them; 1: no split), row < 0: unused place.
 // part_o: n_items * nh * (hd rounded up to 32) floats, part_ml: n_items * nh * 2.  firsts[r] = (row,
-// position, request, index of the row's first item), n_rows of them; null: every row has one split,
+// index of the row's first item, its splits, 0), n_rows of them; null: every row has one split,
 // nothing is merged (and no workspace needed).
 int fl_attn_decode_items(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                          const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv,

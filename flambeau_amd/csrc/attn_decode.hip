@@ -283,7 +283,7 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
 }
 
 // The same for items with splits of their own, which lie nh slots apart: one block per (row, head); firsts[r] =
-// (row, position, request, index of the row's first item).
+// (row, index of the row's first item, its splits, 0).
 __global__ __launch_bounds__(256) void attn_decode_merge_items_kernel(const float* __restrict__ part_o,
                                                                       const float* __restrict__ part_ml,
                                                                       bf16_t* __restrict__ out,
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(256) void attn_decode_merge_items_kernel(const floa
                                                                       int hd, int hdp) {
     const int head = blockIdx.y;
     const int4 row = firsts[blockIdx.x];
-    const int first = row.w, n_split = items[first].w >> 8;
+    const int first = row.y, n_split = row.z;
     if (n_split <= 1) return;
     attn_merge_splits(part_o, part_ml, out + ((size_t)row.x * nh + head) * hd, (size_t)first * nh + head, hd, hdp, n_split,
                       (size_t)nh);
@@ -372,7 +372,7 @@ extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* pa
 // Items with splits of their own: items[i] = (row, position, request, split + 256 * splits), the splits of
 // a row one after the other from split 0 on (up to 255), row < 0 for a place that is not used.  part_o
 // holds n_items * nh * (head size rounded up to 32) floats, part_ml n_items * nh * 2.  firsts[r] = (row,
-// position, request, index of the row's first item) for the n_rows rows; without it no row has more
+// index of the row's first item, its splits, 0) for the n_rows rows; without it no row has more
 // than one split (a list with a place per row and no more) and the kernel that merges is left out.
 extern "C" int fl_attn_decode_items(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                                     const int* items, int n_items, const int* block_table, int max_blocks, int nh,

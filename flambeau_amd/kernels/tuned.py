@@ -516,14 +516,14 @@ def balanced_items(rows, blocks_per_row: int, window: int = 0, budget: int | Non
     proportion to the keys it sees (a split of 128 keys at least, 64 splits at most), so that the blocks
     of a ragged batch take about equally long.  Returns ``(items, firsts)``: ``items`` = (row,
     position, request, split + 256 * splits), a row's splits one after the other, the list filled up
-    to ``decode_item_budget`` with row -1; ``firsts`` = (row, position, request, index of the row's
-    first item), one per row, for the kernel that merges."""
+    to ``decode_item_budget`` with row -1; ``firsts`` = (row, index of the row's first item, its
+    splits, 0), one per row, for the kernel that merges."""
     import numpy as np
     n = rows.shape[0]
     if budget is None:
         budget = decode_item_budget(n, blocks_per_row)
     items = np.full((budget, 4), -1, dtype=np.int32)
-    firsts = rows.copy()
+    firsts = np.zeros((n, 4), dtype=np.int32)
     if n == 0:
         return items, firsts
     keys = rows[:, 1].astype(np.int64) + 1
@@ -558,7 +558,7 @@ def balanced_items(rows, blocks_per_row: int, window: int = 0, budget: int | Non
     total = int(splits.sum())
     items[:total, :3] = rows[which, :3]
     items[:total, 3] = (np.arange(total) - first[which]) + 256 * splits[which]
-    firsts[:, 3] = first
+    firsts[:, 0], firsts[:, 1], firsts[:, 2] = rows[:, 0], first, splits
     return items, firsts
 
 

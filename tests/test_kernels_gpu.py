@@ -614,7 +614,7 @@ def test_attn_decode_with_splits_per_row(nh, nkv, hd, ps, window):
     assert (max(splits.values()) > 1 or 0 < window < 256) and min(splits.values()) == 1
     assert (items_host[:, 0] < 0).any() == (sum(splits.values()) < len(items_host))
     items, firsts = torch.tensor(items_host, device=DEV), torch.tensor(firsts_host, device=DEV)
-    assert all(items_host[f, 0] == r and items_host[f, 3] & 255 == 0 for r, _, _, f in firsts_host)
+    assert all(items_host[f, 0] == r and items_host[f, 3] == 256 * k for r, f, k, _ in firsts_host)
     hdp = -(-hd // 32) * 32
     part_o = torch.full((len(items_host) * nh * hdp,), float("nan"), dtype=torch.float32, device=DEV)
     part_ml = torch.full((len(items_host) * nh * 2,), float("nan"), dtype=torch.float32, device=DEV)

@@ -28,7 +28,7 @@ def test_every_row_gets_consecutive_splits_within_the_budget():
             assert [w & 255 for w in ws] == list(range(k)) and all(w >> 8 == k for w in ws)
             keys = min(pos[r] + 1, window) if window else pos[r] + 1
             assert 1 <= k <= tuned.DECODE_MAX_SPLITS and (k == 1 or keys / k > tuned.DECODE_MIN_KEYS_PER_SPLIT / 2)
-        assert all(items[f, 0] == r and items[f, 3] & 255 == 0 for r, _, _, f in firsts)
+        assert all(items[f, 0] == r and items[f, 3] == 256 * k for r, f, k, _ in firsts)
 
 
 def test_long_contexts_get_the_splits_of_a_ragged_batch():
@@ -48,4 +48,4 @@ def test_long_contexts_get_the_splits_of_a_ragged_batch():
     # no rows, one row
     assert tuned.balanced_items(rows[:0], 8)[0].shape == (0, 4)
     one, first = tuned.balanced_items(rows[:1], 8)
-    assert (one[:, 0] >= 0).sum() == 32 and first[0, 3] == 0
+    assert (one[:, 0] >= 0).sum() == 32 and first[0].tolist() == [0, 0, 32, 0]
