@@ -530,12 +530,14 @@ def balanced_items(rows, blocks_per_row: int, window: int = 0, budget: int | Non
     if window:
         keys = np.minimum(keys, window)
     most = np.minimum(-(-keys // DECODE_MIN_KEYS_PER_SPLIT), DECODE_MAX_SPLITS)
-    # How many places to use.  Rows of about one length: a block per unit is enough (measured at 1 to 64
-    # rows of 2,100 keys: 256 blocks, or one per row and kv head if that is more, beat 512 and 1,024).  A
-    # ragged batch: all places, since many short blocks spread over the units as they finish (55 rows of
-    # 128 to 4,600 keys: 136 us with a place per row, 100 with two, 94 with four per row).
+    # How many places to use.  Rows of about one length: a block per unit is enough (measured at 16 to 64
+    # rows of 2,100 keys: 256 blocks, or one per row and kv head if that is more, beat 512 and 1,024; up
+    # to 8 rows, two per unit were 1 % of a 7B decode step faster).  A ragged batch: all places, since
+    # many short blocks spread over the units as they finish (55 rows of 128 to 4,600 keys: 136 us with
+    # a place per row, 100 with two, 94 with four per row).
     ragged = int(keys.max()) * n > 1.5 * int(keys.sum())
-    use = budget if ragged else min(budget, max(n, DECODE_EVEN_BLOCKS // max(1, blocks_per_row)))
+    even_blocks = DECODE_TARGET_BLOCKS if n * blocks_per_row <= DECODE_TARGET_BLOCKS // 8 else DECODE_EVEN_BLOCKS
+    use = budget if ragged else min(budget, max(n, even_blocks // max(1, blocks_per_row)))
     splits = np.clip(keys * use // max(int(keys.sum()), 1), 1, most)
     # what rounding down and the caps left over goes to the rows whose splits are longest; what the
     # least of one split per row took too much comes from the rows whose splits are shortest

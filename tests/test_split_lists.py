@@ -42,10 +42,12 @@ def test_long_contexts_get_the_splits_of_a_ragged_batch():
     assert longest < 2.0 * sum(p + 1 for p in pos) / len(items) + tuned.DECODE_MIN_KEYS_PER_SPLIT
     # rows of one length share a block per unit and no more; 64 of them get a split each
     even, _ = tuned.balanced_items(np.array([[i, 2099, i, 0] for i in range(8)], dtype=np.int32), 8)
-    assert [int(w) >> 8 for r, _, _, w in even if r >= 0 and w & 255 == 0] == [4] * 8
+    assert [int(w) >> 8 for r, _, _, w in even if r >= 0 and w & 255 == 0] == [8] * 8
+    even, _ = tuned.balanced_items(np.array([[i, 2099, i, 0] for i in range(16)], dtype=np.int32), 8)
+    assert [int(w) >> 8 for r, _, _, w in even if r >= 0 and w & 255 == 0] == [2] * 16
     many, _ = tuned.balanced_items(np.array([[i, 2099, i, 0] for i in range(64)], dtype=np.int32), 8)
     assert len(many) == 256 and (many[:64, 3] == 256).all() and (many[64:, 0] < 0).all()
     # no rows, one row
     assert tuned.balanced_items(rows[:0], 8)[0].shape == (0, 4)
     one, first = tuned.balanced_items(rows[:1], 8)
-    assert (one[:, 0] >= 0).sum() == 32 and first[0].tolist() == [0, 0, 32, 0]
+    assert (one[:, 0] >= 0).sum() == 63 and first[0].tolist() == [0, 0, 63, 0]
