@@ -20,8 +20,11 @@
 //
 // The four waves' states are merged through LDS; with more than one split the block writes a
 // partial (max, sum, O) and a second kernel merges the splits (same rule: exp(m_c - m_max)).
-// (Merging in the block that finishes last was tried and is far slower here: it needs a
-// device-wide release fence in every block, which writes the L2 back, one block after the other.)
+// (Merging in the block that finishes last was tried twice: with a device-wide release fence in every
+// block it is far slower, since each fence writes the L2 back, one block after the other; with
+// device-scope loads and stores and a relaxed counter instead of fences it takes as long as the second
+// kernel that it saves.)  Keys and values are loaded with the non-temporal hint: a step reads each
+// byte of them once, and streaming reads are a tenth faster with the hint.
 // Which keys a row sees depends on its own position only: [max(0, p - window + 1), p].
 //
 // Reference: crates/kernels-hip/src/kernels/attention_decode_f16_paged.cu:49-158 (paged decode),
@@ -34,8 +37,8 @@
 #define DEC_WAVES 4
 #define DEC_CHUNK 32
 
-// items[i] = (row of q and out, position, request, 0): everything a block needs to find its keys
-// comes with one load.
+// items[i] = (row of q and out, position, request, 0 or split + 256 * splits): everything a block needs
+// to find its keys comes with one load.
 template <int HDP>
 __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* part_o,
