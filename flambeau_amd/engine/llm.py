@@ -124,7 +124,7 @@ class LLMEngine:
         logits = self.runner.step(entries)
         if on_device:
             if any(PENDING in r.output and r.params.has_penalties and self._slot(r) is not None
-                   and not self.sampler.holds_history(self._slot(r), r) for r in (s.request for s in rows)):
+                   and not self.sampler.holds_history(self._slot(r), r, len(r.output)) for r in (s.request for s in rows)):
                 finished += self.flush()              # the history is counted anew from tokens the host knows
             inv_t = [0.0 if s.request.params.is_greedy else 1.0 / s.request.params.temperature for s in rows]
             us = [0.0 if s.request.params.is_greedy else s.request.rng.next_f32() for s in rows]

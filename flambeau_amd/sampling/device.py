@@ -28,7 +28,7 @@ class DeviceSampler:
         self._bias_host = torch.zeros((2, 3, max_rows * BIAS_MAX), dtype=torch.float32, pin_memory=True)
         self._bias_dev = torch.zeros((3, max_rows * BIAS_MAX), dtype=torch.float32, device=device)
         self._counts = None          # int16 [max_rows, V]: how often a slot's request generated each token
-        self._owner = {}             # slot -> the request whose history the slot's row holds
+        self._owner = {}             # slot -> (the request whose history the slot's row holds, tokens counted)
         self.ids = torch.empty(max_rows, dtype=torch.int32, device=device)     # the last draw, on the device
         self._ids_host = torch.empty((2, max_rows), dtype=torch.int32, pin_memory=True)
         self._events = [torch.cuda.Event(), torch.cuda.Event()]
@@ -49,11 +49,12 @@ class DeviceSampler:
             slot, owner, generated, rp, pp, fp = hist
             if not 0 <= slot < self.max_rows:
                 raise ValueError(f"history slot {slot}, the sampler has {self.max_rows}")
-            if self._owner.get(slot) is not owner:
-                # the row holds another request's counts: count what this one has generated so far
+            if not self.holds_history(slot, owner, len(generated)):
+                # the row holds another request's counts, or this request's from before it generated
+                # tokens in another slot: count what it has generated so far
                 tokens = torch.tensor(list(generated), dtype=torch.int32).to(self.device)
                 ops.sample_history(self._counts, slot, tokens)
-                self._owner[slot] = owner
+            self._owner[slot] = (owner, len(generated) + 1)      # this draw joins the row
             h[5, i], h[6, i], h[7, i], h[8, i] = slot, rp, pp, fp
         for a in range(5, 9):
             self._dev[a, :R].copy_(self._host[k, a, :R], non_blocking=True)
@@ -73,9 +74,12 @@ class DeviceSampler:
                 self._bias_dev[a, :n].copy_(self._bias_host[k, a, :n], non_blocking=True)
             ops.sample_bias(logits, *(self._bias_dev[a, :n] for a in range(3)))
 
-    def holds_history(self, slot: int, owner) -> bool:
-        """Whether ``slot``'s row of counts is ``owner``'s (else the next draw counts its tokens anew)."""
-        return self._owner.get(slot) is owner
+    def holds_history(self, slot: int, owner, n_generated: int) -> bool:
+        """Whether ``slot``'s row of counts holds exactly the ``n_generated`` tokens that ``owner`` has
+        generated (else the next draw counts its tokens anew): the row is the request's, and the
+        request has drawn every token since in this slot."""
+        held = self._owner.get(slot)
+        return held is not None and held[0] is owner and held[1] == n_generated
 
     def sample_async(self, logits, inv_temps, uniforms, filters=None, histories=None, biases=None):
         """Enqueue the draw for ``logits`` float32 [R, V] (per row ``inv_temp``, <= 0: argmax, and a

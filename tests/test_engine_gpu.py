@@ -329,6 +329,32 @@ def test_penalties_and_bias_stay_on_the_device(model_dirs, monkeypatch):
     assert not eng.runner.manager.live
 
 
+def test_the_sampler_s_history_follows_a_request_through_slots():
+    """A request that is pre-empted comes back in whatever slot is free: its row of token counts is
+    taken over when it kept drawing in the same slot and counted anew otherwise, also when it returns
+    to a slot whose row still holds its counts from before it drew tokens elsewhere."""
+    from flambeau_amd import SamplingParams
+    from flambeau_amd.sampling.device import DeviceSampler
+    from flambeau_amd.sampling.host import penalised
+    V = 50
+    sampler = DeviceSampler(torch.device("cuda:0"), 4)
+    rng = np.random.default_rng(3)
+    p = SamplingParams(repetition_penalty=1.5, presence_penalty=0.3, frequency_penalty=0.2)
+
+    class Req:
+        def __init__(self): self.output = []
+    a, b = Req(), Req()
+    for slot, req, counted_anew in [(0, a, True), (0, a, False), (1, b, True), (2, a, True), (2, a, False), (0, a, True),
+                                    (0, a, False), (1, b, False), (0, b, True), (2, a, True)]:
+        logits = rng.normal(0, 2, (1, V)).astype(np.float32)
+        assert sampler.holds_history(slot, req, len(req.output)) == (not counted_anew)
+        tok = sampler.sample(torch.tensor(logits, device="cuda:0"), [0.0], [0.0], None, [(slot, req, req.output, *p.penalties)])[0]
+        assert tok == int(np.argmax(penalised(logits[0], p, req.output)))
+        req.output.append(tok)
+        assert sampler._counts[slot].cpu().numpy().tolist() == np.bincount(req.output, minlength=V).tolist()
+    assert len(a.output) == 7 and len(b.output) == 3
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_stop_tokens_end_requests_while_the_next_step_is_in_flight(model_dirs, dtype):
     """The engine runs one step ahead of the host: when a stop id (or one of several end-of-sequence
