@@ -62,8 +62,10 @@ class ModelRunner:
         self._meta_dev = None
         self._meta_copied = None     # event: the last metadata copy has left the pinned buffer
         # steps of single tokens replay a captured graph per batch-size bucket, if every mixer
-        # of the model says that running a step twice leaves the same cache (graph_safe)
-        self.decode_graphs = bool(decode_graphs) and all(getattr(c, "graph_safe", False) for c in self._mixer_classes)
+        # of the model says that running a step twice leaves the same cache (graph_safe) and every part
+        # of it can be captured (a part that is not replayable may call what a capture does not allow)
+        self.decode_graphs = (bool(decode_graphs) and all(getattr(c, "graph_safe", False) for c in self._mixer_classes)
+                              and getattr(model, "capturable", lambda: True)())
         self.max_graph_batch = min(max_graph_batch, max_slots)
         self._graphs: dict[int, "_GraphedStep"] = {}
         # ids drawn on the device in the step before (the sampler's output buffer); entries with

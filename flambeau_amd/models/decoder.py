@@ -125,6 +125,12 @@ class DecoderModel:
         final norm and head must be; a block that is not runs as it is between the recorded stretches."""
         return all(self._part_replayable(p) for p in (self.embedding, self.final_norm, self.head))
 
+    def capturable(self) -> bool:
+        """True if a whole step of this model can go into a device graph: every part only enqueues
+        launches of the kernel library (``Part.replayable``), the blocks included (a part that calls
+        other libraries or waits for the device cannot be captured)."""
+        return self.replayable() and all(self._part_replayable(b) for b in self.blocks)
+
     @staticmethod
     def _part_replayable(part) -> bool:
         todo = [part]

@@ -508,6 +508,34 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
     rh.compare(rh.run_in_process(runner, rh.trace_mixed(reqs, seed=3, max_live=3)), reqs, ref, dtype, "toy again")
 
 
+def test_a_part_that_cannot_be_captured_keeps_decode_steps_out_of_graphs(tmp_path):
+    """All mixers are attention (a padded decode step could replay a device graph), but one layer's
+    feed-forward is the toy that calls torch and looks at its routing on the host: such a model's
+    decode steps are not captured (a capture refuses those calls); its other blocks are still
+    recorded, and every cutting gives the plain numbers."""
+    import replay_helpers as rh
+    from flambeau_amd.engine import ModelRunner, load_model
+    from flambeau_amd.weights import write_random_model
+    _register_toys()
+    cfg = dict(architectures=["ToyStateLM"], hidden_size=32, vocab_size=70, layer_kinds=["attn", "attn"],
+               ffn_kinds=["swiglu", "routed"], decay=0.8, rate=0.3, max_position_embeddings=128)
+    d = write_random_model(cfg, tmp_path / "toy2", seed=6, std=0.15, gain_std=0.05, store_dtype=torch.float32)
+    model, _ = load_model(d, dtype="float32", max_batch_tokens=128)
+    assert not model.capturable() and model.replayable()
+    runner = ModelRunner(model, n_pages=14, page_size=8, max_slots=3, max_logit_rows=128)
+    assert not runner.decode_graphs and runner.step_programs
+    w = {k: v for k, v in pm.read_safetensors(d / "model.safetensors").items()}
+    reqs = rh.make_requests(70, [21, 9, 33, 14], seed=8)
+    ref = {rid: _toy_plain(cfg, w, toks) for rid, toks in reqs.items()}
+    for mode, steps in [("tail", rh.trace_tail(reqs, tail=12)), ("mixed", rh.trace_mixed(reqs, seed=2, max_live=3, max_portion=9, decode_tail=6))]:
+        rh.compare(rh.run_in_process(runner, steps), reqs, ref, "float32", f"toy {mode}")
+    assert runner.n_replayed > 5
+    # the built-in architecture's parts can all be captured
+    from flambeau_amd.engine import random_model
+    from tiny_configs import TINY
+    assert random_model(TINY["A"]["config"], 1, dtype="bfloat16")[0].capturable()
+
+
 def test_unknown_part_names_the_known_ones():
     from flambeau_amd.parts import MIXERS, PartSpec
     with pytest.raises(KeyError, match="paged_gqa_attention"):
