@@ -62,8 +62,8 @@ def sample_host(logits: np.ndarray, params: SamplingParams, history, rng: Xoshir
         ids, kept = order[:end], probs[:end]
     else:
         ids, kept = None, p
-    u = np.float32(rng.next_f32()) * kept.sum(dtype=np.float32)
-    walk = np.cumsum(kept, dtype=np.float32)
+    walk = np.cumsum(kept, dtype=np.float32)              # (the sum of the kept ones is added up in their order, as the walk is)
+    u = np.float32(rng.next_f32()) * walk[-1]
     idx = int(np.searchsorted(walk, u, side="left"))      # first i with u - walk[i] <= 0
     idx = min(idx, kept.shape[0] - 1)
     return int(idx if ids is None else ids[idx])

@@ -381,7 +381,10 @@ def sample(logits, rng: Xoshiro, temperature=0.0, top_k=None, top_p=None, min_p=
             end = max(drop, 1)
         ids = order[:end]
     kept = p[ids]
-    u = np.float32(rng.next_f32()) * kept.sum(dtype=np.float32)
+    total = np.float32(0.0)
+    for pv in kept:                      # summed in order (sampling.rs:736), not pairwise
+        total = np.float32(total + pv)
+    u = np.float32(rng.next_f32()) * total
     for tok, pv in zip(ids, kept):
         u -= pv
         if u <= 0.0:
