@@ -139,9 +139,9 @@ class LLMEngine:
             self._in_flight = (sched, handle) if rows else None
             return finished
         # Some request wants what the device sampler does not take (a top-k beyond 2048, a long
-        # bias list): its logits go to the host sampler and nothing stays in flight.  Rows that the device can draw are still drawn there (by the same kernel,
-        # from the same numbers of their own generators), so a request's tokens do not depend on
-        # what its neighbours ask for.
+        # bias list): its logits go to the host sampler and nothing stays in flight.  Rows that the
+        # device can draw are still drawn there (by the same kernel, from the same numbers of their
+        # own generators), so a request's tokens do not depend on what its neighbours ask for.
         finished += self.flush()
         sampled = {}
         live = [i for i, s in enumerate(rows) if s.request.status != "finished"]   # (a stop token of the step before may just have ended one)
