@@ -132,6 +132,9 @@ int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* out, float* 
 int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K, float* resid,
                            const float* g, void* xg, float* out_ssq, hipStream_t stream);
 int fl_gemm_tiled_parts(int M, int N, int K);
+// The K-splits left apart in workspace[fl_gemm_tiled_splits(M, N, K)][M][N], each scaled by in_ssq's row scale.
+int fl_gemm_tiled_partials(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                           const float* in_ssq, int in_parts, float eps, hipStream_t stream);
 int fl_gemm_tiled_residual_parts(int M, int N, int K);
 int fl_attn_decode(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
                    const int* items, int n_items, const int* block_table, int max_blocks, int nh, int nkv, int hd, int page_size,

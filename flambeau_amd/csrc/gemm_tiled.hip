@@ -598,6 +598,26 @@ extern "C" int fl_gemm_tiled_residual_parts(int M, int N, int K) {
     return fl_gemm_tiled_splits(M, N, K) > 1 ? fl_gemm_mid_parts(N) : fl_gemm_tiled_parts(M, N, K);
 }
 
+// The K-splits of x w^T left apart: workspace[splits][M][N] (splits = fl_gemm_tiled_splits(M, N, K), at
+// least one) for a kernel that adds them with work of its own (the rotation kernel does).  in_ssq as
+// in fl_gemm_tiled_scaled: every part is scaled, so that their sum is.
+extern "C" int fl_gemm_tiled_partials(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
+                                      const float* in_ssq, int in_parts, float eps, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_partials: bad sizes M=%d N=%d K=%d", M, N, K);
+    FL_CHECK(K % 8 == 0, "gemm_tiled_partials: K=%d is no multiple of 8 (16-byte loads)", K);
+    FL_CHECK(workspace && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)workspace % 16 == 0),
+             "gemm_tiled_partials: operands must be 16-byte aligned");
+    FL_CHECK(!in_ssq || in_parts > 0, "gemm_tiled_partials: a row scale over %d parts", in_parts);
+    if (M == 0) return 0;
+    const int n_steps = ceil_div(K, 32);
+    const TilePlan plan = tiled_plan(M, N, K, true, 0, 0);
+    const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
+    launch_tiled<float, TG_PLAIN>(plan.variant, plan.splits, stream, (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
+                                  n_steps, ceil_div(n_steps, plan.splits), N, RopeStore{}, fu);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+
 // The joined q/k/v projection of many rows with its rows in paired order: q is rotated and written to
 // q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens' positions; cs[M,
 // rot / 2, 2] are the step's cosines and sines.  K is never split here (for shapes whose K the plain

@@ -75,6 +75,7 @@ const Known g_known[] = {
     FL_KNOWN(fl_gemm_tiled), FL_KNOWN(fl_gemm_skinny_rope), FL_KNOWN(fl_gemm_tiled_rope), FL_KNOWN(fl_gemm_tiled_scaled),
     FL_KNOWN(fl_gemm_tiled_residual), FL_KNOWN(fl_attn_decode), FL_KNOWN(fl_attn_decode_static), FL_KNOWN(fl_attn_prefill),
     FL_KNOWN(fl_gemm_mid_ex), FL_KNOWN(fl_gemm_tiled_ex), FL_KNOWN(fl_gemm_tiled_residual_ex), FL_KNOWN(fl_gemm_tiled_rope_ex), FL_KNOWN(fl_attn_decode_items),
+    FL_KNOWN(fl_gemm_tiled_partials),
 };
 #undef FL_KNOWN
 

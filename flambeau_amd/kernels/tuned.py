@@ -31,6 +31,7 @@ register_signatures({
     "fl_gemm_mid_residual": [P, P, P, I, I, I, P, P, P, P, P],
     "fl_gemm_mid_parts": [I],
     "fl_gemm_mid_partials": [P, P, P, I, I, I, P, I, F, P],
+    "fl_gemm_tiled_partials": [P, P, P, I, I, I, P, I, F, P],
     "fl_gemm_mid_ex": [P, P, P, P, I, I, I, I, I, I, P, I, F, I, I, P],
     "fl_gemm_tiled_ex": [P, P, P, P, I, I, I, I, I, I, P, I, F, I, I, P],
     "fl_gemm_tiled_residual_ex": [P, P, P, I, I, I, P, P, P, P, I, P],
@@ -183,12 +184,19 @@ def gemm_rope_store(x, w: Weight, store: RopeStore, rt=None) -> bool:
         x, scale = _rows_for(x, w, rt)
         gemm_skinny_rope(x, w.packed, w.rows, store, row_scale=scale)
         return True
-    # many rows: the tiled product rotates and stores itself where its K is not split (where it is, the
-    # split product, the kernel that adds the splits and the rotation kernel together are faster:
-    # 45 + 9 + 13 us against 82 at 7B sizes and 512 rows)
-    if M > SKINNY_MAX_ROWS and K % 8 == 0 and gemm_tiled_splits(M, w.rows, K) == 1:
+    # many rows: the tiled product rotates and stores itself where its K is not split; where it is, it
+    # leaves the splits apart and the rotation kernel adds them (at 7B sizes and 512 rows the product
+    # with K split in two takes 45 us and the rotation kernel 13, the whole product in one kernel 82)
+    if M > SKINNY_MAX_ROWS and K % 8 == 0:
         x, scale = _rows_for(x, w, rt)
-        gemm_tiled_rope(x, w.packed, w.rows, store, row_scale=scale)
+        N = w.rows
+        splits = gemm_tiled_splits(M, N, K)
+        if splits == 1:
+            gemm_tiled_rope(x, w.packed, N, store, row_scale=scale)
+        else:
+            parts = gemm_tiled_partials(x, w.packed, _split_workspace(rt, splits * M * N, x.device), N, row_scale=scale)
+            ops.rope_kv_write(parts, store.positions, store.tok_seq, store.block_table, store.q_out, store.cache, store.n_heads,
+                              store.rotated_dims, 0.0, write_cache=store.write_cache, table=store.angles, paired=True, parts=splits)
         return True
     if FUSED_NORM_MAX_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0:
         # 17 to 64 rows: the product leaves its K-splits apart and the rotation kernel adds them
@@ -343,6 +351,22 @@ def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale
     else:
         call("fl_gemm_tiled_scaled", *args, stream_handle())
     return out
+
+
+def gemm_tiled_partials(x, w_packed, workspace, n_features: int, row_scale: NormedRows | None = None):
+    """``gemm_mid_partials`` for many rows: the K-splits of ``x @ w.T`` as ``[gemm_tiled_splits(M, N, K),
+    M, N]`` float32 (a view of ``workspace``)."""
+    M, K = x.shape
+    N = n_features
+    if w_packed.numel() != _packed_size(N, K):
+        raise KernelError(f"gemm.w: packed matrix of {w_packed.numel()} values, a [{N}, {K}] matrix packs to {_packed_size(N, K)}")
+    splits = gemm_tiled_splits(M, N, K)
+    if workspace is None or workspace.numel() < splits * M * N:
+        raise KernelError(f"gemm_tiled_partials: needs a workspace of {splits * M * N} floats")
+    ssq, parts, eps = _row_scale_args(row_scale, M, K)
+    call("fl_gemm_tiled_partials", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
+         _check(workspace, "gemm.workspace", torch.float32), M, N, K, ssq, parts, eps, stream_handle())
+    return workspace[:splits * M * N].view(splits, M, N)
 
 
 def tiled_parts(M: int, n_features: int, K: int, variant: int = 0) -> int:

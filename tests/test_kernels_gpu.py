@@ -767,11 +767,13 @@ def test_gemm_mid_refuses_what_it_cannot_do():
                                                   (300, 6, 2, 64, 64, 16, 96), (2048, 32, 8, 128, 128, 16, 512),
                                                   (130, 3, 1, 48, 32, 32, 72), (70, 8, 8, 16, 16, 8, 40),
                                                   (64, 32, 8, 128, 128, 16, 4096), (17, 6, 2, 64, 32, 16, 96), (40, 5, 5, 32, 16, 8, 2048),
-                                                  (33, 4, 2, 16, 16, 8, 40)])
+                                                  (33, 4, 2, 16, 16, 8, 40),
+                                                  (512, 32, 8, 128, 128, 16, 4096), (200, 6, 2, 64, 32, 16, 4104), (96, 5, 1, 32, 16, 8, 8192)])
 def test_gemm_with_rotation_and_stores_in_its_kernel(M, nh, nkv, hd, rot, ps, H):
     """The joined q/k/v projection with rows in paired order, rotated and stored by the product's own
-    kernel (few rows: skinny; many rows: tiled) or, for 17 to 64 rows, by a rotation kernel that adds
-    the product's K-splits itself; against product + rotation kernel apart and float64."""
+    kernel (few rows: skinny; many rows: tiled) or, for 17 to 64 rows and for more rows whose product
+    splits K, by a rotation kernel that adds the product's K-splits itself; against product + rotation
+    kernel apart and float64."""
     from flambeau_amd.kernels.packing import rotary_paired_rows
     theta = 1e4
     N = (nh + 2 * nkv) * hd
@@ -809,15 +811,19 @@ def test_gemm_with_rotation_and_stores_in_its_kernel(M, nh, nkv, hd, rot, ps, H)
     cache_b = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
     q_b = torch.full((M, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     store = tuned().RopeStore(pos_d, seq_d, table, angles, q_b, cache_b, nh, rot, True)
-    if (16 < M <= 64 and H % 32) or (M > 64 and tuned().gemm_tiled_splits(M, N, H) > 1):
+    if 16 < M <= 64 and H % 32:
         assert not tuned().gemm_rope_store(x, W, store)
         return
+    split = M > 64 and tuned().gemm_tiled_splits(M, N, H) > 1
+    assert split == ((M, H) in ((512, 4096), (200, 4104), (96, 8192)))          # the cases meant to split do
     assert tuned().gemm_rope_store(x, W, store)
     top = q_a.float().abs().max()
     assert (q_a.float() - q_b.float()).abs().max() <= 2e-2 * top
     assert (cache_a.pool.float() - cache_b.pool.float()).abs().max() <= 2e-2 * cache_a.pool.float().abs().max()
     assert ((cache_a.pool != 0) == (cache_b.pool != 0)).all()          # the same places were written
-    if M > 64:
+    if split:
+        assert torch.equal(q_a, q_b) and torch.equal(cache_a.pool, cache_b.pool)      # the same sums in the same order
+    elif M > 64:
         # every block shape of the tiled product writes the same
         for variant in (3, 6, 7, 8, 10):
             cache_v = make_cache(n_pages, nkv, ps, hd, torch.bfloat16)
