@@ -165,6 +165,10 @@ int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int*
                     const int* positions, const int* block_table, int max_blocks, int nh, int nkv, int hd,
                     int page_size, int n_pages, float scale, int window, int qt_hint, float* part_o, float* part_ml,
                     int n_split, hipStream_t stream);
+// Block-table entries of a request that a block of fl_attn_prefill can keep at a head size, and whether
+// it takes a cache shape with tables max_blocks wide (with a window only the window's pages count).
+int fl_attn_prefill_max_pages(int hd);
+int fl_attn_prefill_takes(int hd, int page_size, int max_blocks, int window);
 int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int max_keys);
 int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats, long* ml_floats);

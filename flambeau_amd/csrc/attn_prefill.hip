@@ -390,14 +390,15 @@ static int pf_units() {                  // compute units of the device
 template <int HDP, int QT, int NS>
 static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                                const int* tiles, const int* positions, const int* block_table, int max_blocks,
-                               int nh, float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml) {
+                               int nh, float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml, int lds_pages) {
     // blocks that the chip holds at one time: one or two per compute unit
     const int units = pf_units();
     const int total = (int)(grid.x * grid.y * grid.z);
-    const int resident = units * (QT * HDP <= 256 ? 2 : 1);
-    // (whole rows of the grid: every tile of a head group is taken exactly once either way)
-    const int mirror_from = (QT * HDP <= 256 && grid.z == 1 && total <= resident && total > units) ? (int)((grid.y / 2) * grid.x) : (int)(grid.x * grid.y);
     constexpr int RING = NS * (4 * (HDP / 32) + 2 * (HDP / 16)) * 1024;
+    const int lds = RING + lds_pages * (int)sizeof(int);
+    const int resident = units * ((QT * HDP <= 256 && 2 * lds <= PF_LDS_BYTES) ? 2 : 1);
+    // (whole rows of the grid: every tile of a head group is taken exactly once either way)
+    const int mirror_from = (resident == 2 * units && grid.z == 1 && total <= resident && total > units) ? (int)((grid.y / 2) * grid.x) : (int)(grid.x * grid.y);
     static bool configured = false;
     auto kern = attn_prefill_kernel<HDP, QT, NS>;
     if (!configured) {
@@ -405,23 +406,23 @@ static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, b
                                   min(RING + PF_MAX_PAGES * (int)sizeof(int), PF_LDS_BYTES));
         configured = true;
     }
-    kern<<<grid, 256, RING + max_blocks * sizeof(int), stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from, part_o, part_ml);
+    kern<<<grid, 256, lds, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from, part_o, part_ml);
 }
 
 template <int HDP, int NS>
 static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                            const int* tiles, const int* positions, const int* block_table, int max_blocks, int nh,
-                           float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml) {
+                           float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml, int lds_pages) {
     if constexpr (HDP <= 64) {            // four heads per wave only where two blocks still fit a compute unit
         if (qt == 4) {
-            launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml);
+            launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml, lds_pages);
             return;
         }
     }
     if (qt >= 2)
-        launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml);
+        launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml, lds_pages);
     else
-        launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml);
+        launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml, lds_pages);
 }
 
 // query heads per wave: a divisor of the group size; as many as leave room for two blocks per
@@ -450,6 +451,27 @@ extern "C" int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int 
     const int want = (2 * pf_units()) / max(blocks, 1);
     const int by_keys = ceil_div(max(max_keys, 1), PF_STAGE) / 8;
     return max(1, min(min(want, by_keys), 16));
+}
+
+// Block-table entries per request that the kernel takes at a head size: the table of a request sits in
+// LDS beside the ring of two stages of 64 keys and values (256 bytes per padded head dim and stage).
+extern "C" int fl_attn_prefill_max_pages(int hd) {
+    if (hd <= 0 || hd > 256) return 0;
+    const int hdp = ceil_div(hd, 32) * 32;
+    return min(PF_MAX_PAGES, (PF_LDS_BYTES - 2 * hdp * 256) / (int)sizeof(int));
+}
+
+// Entries of a request's table that a block may need: all of them, or with a window the pages of the
+// window + 63 keys that its 64 queries see between them.
+static int pf_table_need(int max_blocks, int page_size, int window) {
+    if (window <= 0) return max_blocks;
+    return min(max_blocks, (window + PF_TOKENS - 2) / page_size + 2);
+}
+
+// Whether fl_attn_prefill takes a cache of this shape with block tables max_blocks wide.
+extern "C" int fl_attn_prefill_takes(int hd, int page_size, int max_blocks, int window) {
+    if (hd <= 0 || hd > 256 || hd % 8 || page_size < 8 || (page_size & (page_size - 1)) || max_blocks < 0 || window < 0) return 0;
+    return pf_table_need(max_blocks, page_size, window) <= fl_attn_prefill_max_pages(hd) ? 1 : 0;
 }
 
 // Workspace of the split form, in floats: part_o and part_ml for n_rows rows of tiles.
@@ -520,12 +542,10 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     FL_CHECK(page_size >= 8 && (page_size & (page_size - 1)) == 0,
              "attn_prefill: page size %d must be a power of two, at least 8", page_size);
     FL_CHECK((long long)2 * nkv * page_size * hd < (1ll << 31), "attn_prefill: a page of %d heads x %d keys x %d is too large (2^31 values)", nkv, page_size, hd);
-    {
-        // (the ring of two stages of 64 keys and values: 256 bytes per padded head dim and stage)
-        const int hdp = (hd + 31) / 32 * 32, most = min(PF_MAX_PAGES, (PF_LDS_BYTES - 2 * hdp * 256) / (int)sizeof(int));
-        FL_CHECK(max_blocks <= most, "attn_prefill: %d pages per request, at most %d with heads of %d", max_blocks, most, hd);
-    }
     FL_CHECK(window >= 0, "attn_prefill: negative window");
+    const int lds_pages = pf_table_need(max_blocks, page_size, window);
+    FL_CHECK(lds_pages <= fl_attn_prefill_max_pages(hd), "attn_prefill: %d pages per request in reach of a block, at most %d with heads of %d",
+             lds_pages, fl_attn_prefill_max_pages(hd), hd);
     FL_CHECK(scale > 0.f, "attn_prefill: the score scale must be positive");
     FL_CHECK(n_split >= 1 && n_split <= 16, "attn_prefill: %d splits (at most 16)", n_split);
     FL_CHECK(n_split == 1 || (part_o && part_ml && (uintptr_t)part_o % 16 == 0), "attn_prefill: splits need a 16-byte aligned workspace");
@@ -543,7 +563,7 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     // a ring of two stages: two blocks then fit a compute unit (three stages were no faster)
 #define FL_PF(HDP_)                                                                                            \
     launch_prefill<HDP_, 2>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                            max_blocks, nh, sl, window, log2_ps, part_o, part_ml)
+                            max_blocks, nh, sl, window, log2_ps, part_o, part_ml, lds_pages)
     switch (hdp) {
         case 32: FL_PF(32); break;
         case 64: FL_PF(64); break;

@@ -40,6 +40,8 @@ register_signatures({
     "fl_gemm_tiled_shape": [I, I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, P, I, P],
     "fl_attn_prefill_splits": [I, I, I, I, I],
+    "fl_attn_prefill_max_pages": [I],
+    "fl_attn_prefill_takes": [I, I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
     "fl_attn_decode_items": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P, I, P],
 })
@@ -663,12 +665,18 @@ def decode_supported(cache) -> bool:
         and cache.page_size % 8 == 0
 
 
-PREFILL_MAX_PAGES = 4096     # block-table entries per request the tiled kernel keeps in LDS
+def prefill_max_pages(head_dim: int) -> int:
+    """Block-table entries per request that the tiled kernel takes (it keeps a request's table in LDS
+    beside its ring of keys and values); the library is the one place that knows."""
+    from .library import load
+    return load().fl_attn_prefill_max_pages(int(head_dim))
 
 
-def prefill_supported(cache, table) -> bool:
-    ps = cache.page_size
-    return decode_supported(cache) and ps >= 8 and ps & (ps - 1) == 0 and table.shape[1] <= PREFILL_MAX_PAGES
+def prefill_supported(cache, table, window: int = 0) -> bool:
+    """Whether the tiled kernel takes this cache with block tables this wide (the library decides)."""
+    from .library import load
+    return cache.pool.dtype == torch.bfloat16 and bool(
+        load().fl_attn_prefill_takes(cache.head_dim, cache.page_size, table.shape[1], int(window or 0)))
 
 
 def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int, with_items: bool = True):
@@ -697,7 +705,7 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
     sends the whole batch to the plain kernel."""
     rows, tiles = step.extra.get("attn_rows"), step.extra.get("attn_tiles")
     batch = step.host
-    if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table)):
+    if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table, window)):
         return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
     items = step.extra.get(f"attn_items/{decode_blocks_per_row(n_heads, cache.n_kv_heads)}/{window or 0}")
     key = ("attention_splits", n_heads, cache.n_kv_heads, cache.head_dim, window)

@@ -131,10 +131,12 @@ def rope_neox(x, positions, theta, rotated_dims=None):
     return x
 
 
-def attention(q, k, v, positions, scale, window=0):
+def attention(q, k, v, positions, scale, window=0, key_positions=None):
     """Causal grouped-query attention over one whole sequence.
 
-    q[n, nh, hd], k/v[n, nkv, hd]; token j sits at absolute position positions[j].
+    q[m, nh, hd] are queries at absolute positions ``positions``; k/v[n, nkv, hd] are the keys
+    and values of the whole sequence at ``key_positions`` (the same places as the queries unless
+    given: a caller that wants the output at a few rows only passes those rows' queries).
     kv_head = q_head // (nh // nkv); query at p sees keys t in
     [max(0, p-W+1), p] (W = 0: [0, p]); s_t = (q.k_t)*scale, scale applied after
     the dot; o = sum softmax(s)_t v_t over the visible keys only.
@@ -142,26 +144,34 @@ def attention(q, k, v, positions, scale, window=0):
     :58-71 (limit and window start), :89-133 (scores, softmax, PV);
     window counts keys including the query's own: crates/ops/tests/swa_softcap_parity.rs:243;
     default scale 1/sqrt(hd): crates/forward/src/core/composites/standard_attn.rs:418-420.
+
+    Queries are taken 256 at a time, each batch against the keys that any of its queries sees, so that
+    no score matrix is larger than 256 x n (the arithmetic per query is the same).
     """
     q = np.asarray(q, dtype=F64)
     k = np.asarray(k, dtype=F64)
     v = np.asarray(v, dtype=F64)
     positions = np.asarray(positions, dtype=np.int64)
-    n, nh, hd = q.shape
+    key_positions = positions if key_positions is None else np.asarray(key_positions, dtype=np.int64)
+    m, nh, hd = q.shape
     nkv = k.shape[1]
     group = nh // nkv
-    # visible[i, t]: key t lies in [max(0, p_i - W + 1), p_i]
     lo = np.maximum(0, positions - window + 1) if window > 0 else np.zeros_like(positions)
-    visible = (positions[None, :] >= lo[:, None]) & (positions[None, :] <= positions[:, None])
-    out = np.zeros((n, nh, v.shape[2]), dtype=F64)
-    for h in range(nh):
-        g = h // group
-        s = (q[:, h, :] @ k[:, g, :].T) * scale
-        s = np.where(visible, s, -np.inf)              # keys outside the range take no part
-        s = s - s.max(axis=1, keepdims=True)
-        w = np.exp(s)
-        w = w / w.sum(axis=1, keepdims=True)
-        out[:, h, :] = w @ v[:, g, :]
+    out = np.zeros((m, nh, v.shape[2]), dtype=F64)
+    for a in range(0, m, 256):
+        b = min(m, a + 256)
+        near = np.nonzero((key_positions >= lo[a:b].min()) & (key_positions <= positions[a:b].max()))[0]
+        kp = key_positions[near]
+        # visible[i, t]: key t lies in [max(0, p_i - W + 1), p_i]
+        visible = (kp[None, :] >= lo[a:b, None]) & (kp[None, :] <= positions[a:b, None])
+        for h in range(nh):
+            g = h // group
+            s = (q[a:b, h, :] @ k[near, g, :].T) * scale
+            s = np.where(visible, s, -np.inf)              # keys outside the range take no part
+            s = s - s.max(axis=1, keepdims=True)
+            w = np.exp(s)
+            w = w / w.sum(axis=1, keepdims=True)
+            out[a:b, h, :] = w @ v[near, g, :]
     return out
 
 
@@ -186,20 +196,23 @@ def default_scale(hd: int) -> float:
     return 1.0 / math.sqrt(hd)
 
 
-def attention_mixer(x, w, prefix, positions, nh, nkv, hd, theta, window):
+def attention_mixer(x, w, prefix, positions, nh, nkv, hd, theta, window, rows=None):
     """Q/K/V projections, rotation of Q and K (not V), attention, output projection.
 
     crates/forward/src/core/composites/standard_attn.rs:198-286 (projections),
     :356-397 (rotation of Q and K), :1289-1301 (output projection).
+    ``rows``: the output at these rows only (their queries against everyone's keys and values).
     """
     n = x.shape[0]
-    q = linear(x, w[prefix + "q_proj.weight"]).reshape(n, nh, hd)
+    positions = np.asarray(positions, dtype=np.int64)
+    at = np.arange(n) if rows is None else np.asarray(rows, dtype=np.int64)
+    q = linear(x[at], w[prefix + "q_proj.weight"]).reshape(len(at), nh, hd)
     k = linear(x, w[prefix + "k_proj.weight"]).reshape(n, nkv, hd)
     v = linear(x, w[prefix + "v_proj.weight"]).reshape(n, nkv, hd)
-    q = rope_neox(q, positions, theta)
+    q = rope_neox(q, positions[at], theta)
     k = rope_neox(k, positions, theta)
-    o = attention(q, k, v, positions, default_scale(hd), window)
-    return linear(o.reshape(n, nh * hd), w[prefix + "o_proj.weight"])
+    o = attention(q, k, v, positions[at], default_scale(hd), window, key_positions=positions)
+    return linear(o.reshape(len(at), nh * hd), w[prefix + "o_proj.weight"])
 
 
 def config_numbers(cfg: dict) -> dict:
@@ -240,17 +253,23 @@ def forward(cfg: dict, w: dict, tokens, positions=None, keep_layers=None, rows=N
     if positions is None:
         positions = np.arange(n)
     x = embedding(tokens, w["model.embed_tokens.weight"])
-    layers = range(c["L"]) if keep_layers is None else keep_layers
-    for l in layers:
+    layers = list(range(c["L"]) if keep_layers is None else keep_layers)
+    picked = None if rows is None else np.asarray(rows, dtype=np.int64)
+    for i, l in enumerate(layers):
         p = f"model.layers.{l}."
         a = rmsnorm(x, w[p + "input_layernorm.weight"], c["eps"])
-        x = x + attention_mixer(a, w, p + "self_attn.", positions, c["nh"], c["nkv"], c["hd"],
-                                c["theta"], layer_window(c, l))
+        # the last layer's output is needed at the wanted rows only: their queries against all keys
+        only = picked if i == len(layers) - 1 else None
+        mixed = attention_mixer(a, w, p + "self_attn.", positions, c["nh"], c["nkv"], c["hd"],
+                                c["theta"], layer_window(c, l), rows=only)
+        if only is not None:
+            x, picked = x[only], None
+        x = x + mixed
         b = rmsnorm(x, w[p + "post_attention_layernorm.weight"], c["eps"])
         x = x + swiglu_mlp(b, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                            w[p + "mlp.down_proj.weight"])
-    if rows is not None:
-        x = x[np.asarray(rows, dtype=np.int64)]
+    if picked is not None:
+        x = x[picked]
     f = rmsnorm(x, w["model.norm.weight"], c["eps"])
     head = w["model.embed_tokens.weight"] if c["tied"] else w["lm_head.weight"]
     return linear(f, head)

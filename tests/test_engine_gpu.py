@@ -591,41 +591,65 @@ def test_short_portions_behind_a_long_context(tmp_path_factory, dtype):
     rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, "long context")
 
 
-def test_context_beyond_65536_tokens(tmp_path):
-    """70,000 tokens of context (4,375 pages of 16: a block table 8,192 wide): the prompt in portions of
-    4,096, the last tokens one by one; the bfloat16 kernels against the 32-bit path of the same engine on
-    the same (bfloat16-valued) weights.  The plain implementation cannot hold a score matrix this large."""
+def test_context_beyond_65536_tokens(tmp_path, monkeypatch):
+    """70,000 tokens of context (4,375 pages of 16: block tables 8,192 wide from token 65,537 on): the
+    prompt in portions of 4,096, the last tokens one by one, against the plain implementation at rows of
+    the last two portions and at every decoded token.  The first layer has a window of 700 (so the plain
+    implementation needs no score matrix of 70,000 squared there), the second sees everything and is
+    computed at the wanted rows only.  In bfloat16 the tiled and the split-K attention kernels must take
+    tables this wide themselves: the plain attention kernel is not allowed to run."""
     import torch
     from flambeau_amd.engine import ModelRunner, load_model
+    from flambeau_amd.kernels import ops, tuned
     from flambeau_amd.weights import write_random_model
     config = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "hidden_act": "silu",
               "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2,
-              "intermediate_size": 96, "vocab_size": 150, "rope_theta": 1e6, "sliding_window": None,
+              "intermediate_size": 96, "vocab_size": 150, "rope_theta": 1e6, "sliding_window": 700,
+              "layer_types": ["sliding_attention", "full_attention"],
               "rms_norm_eps": 1e-5, "max_position_embeddings": 131072, "tie_word_embeddings": False}
     d = write_random_model(config, tmp_path / "model", seed=14, std=0.08, gain_std=0.02, store_dtype=torch.bfloat16)
     n, tail = 70000, 6
     toks = rh.make_requests(150, [n], seed=10)["r0"]
-    steps, at = [], 0
+    steps, wanted, at = [], [], 0
     while at < n - tail:
         cnt = min(4096, n - tail - at)
-        steps.append(dict(step=len(steps), entries=[dict(id="r0", tokens=toks[at:at + cnt], want=[cnt - 1] if at + cnt == n - tail else [])], end=[]))
+        # rows of the portions that lie beyond 65,536 tokens: tile edges, and the portion's last rows
+        want = sorted({0, 63, 64, 1000, 2047, cnt - 2, cnt - 1} & set(range(cnt))) if at + cnt > 65536 else []
+        steps.append(dict(step=len(steps), entries=[dict(id="r0", tokens=toks[at:at + cnt], want=want)], end=[]))
+        wanted += [at + r for r in want]
         at += cnt
     for i in range(n - tail, n):
         steps.append(dict(step=len(steps), entries=[dict(id="r0", tokens=toks[i:i + 1], want=[0])], end=["r0"] if i == n - 1 else []))
-    results = {}
+        wanted.append(i)
+    assert len(wanted) == 12 + tail and min(wanted) == 65536
+    cfg, w = pm.read_model_dir(d)
+    ref = dict(zip(wanted, pm.forward(cfg, w, toks, rows=wanted)))
+    scale = max(float(np.abs(v).max()) for v in ref.values())
     for dtype in ("float32", "bfloat16"):
+        widths = []
+        if dtype == "bfloat16":
+            def no_plain(*a, **k):
+                raise AssertionError("the plain attention kernel ran on the bfloat16 path")
+            monkeypatch.setattr(ops, "attn_plain", no_plain)
+            tiled = tuned.attn_prefill
+
+            def counted(q, out, cache, tiles, positions, table, *a, **k):
+                widths.append(table.shape[1])
+                return tiled(q, out, cache, tiles, positions, table, *a, **k)
+            monkeypatch.setattr(tuned, "attn_prefill", counted)
         model, _ = load_model(d, dtype=dtype, max_batch_tokens=4096)
         runner = ModelRunner(model, n_pages=4400, page_size=16, max_slots=2, max_logit_rows=8)
         runner.storage.fill(float("nan"))
-        results[dtype] = rh.run_in_process(runner, steps)
-        assert not runner.manager.live and runner.manager.free_pages() == [4400]
+        got = rh.run_in_process(runner, steps)
+        assert not runner.manager.live and runner.manager.free_pages() == [4400, 4400]
         del runner, model
         torch.cuda.empty_cache()
-    want, got = results["float32"], results["bfloat16"]
-    assert sorted(want) == sorted(got) and len(want) == tail + 1
-    scale = max(float(np.abs(v).max()) for v in want.values())
-    for k in want:
-        assert np.isfinite(got[k]).all() and np.abs(got[k] - want[k]).max() <= 2e-2 * scale, k
+        assert sorted(p for _, p in got) == wanted
+        tol = 1e-4 if dtype == "float32" else 2e-2 * scale
+        for (_, p), row in got.items():
+            assert np.isfinite(row).all() and np.abs(row - ref[p]).max() <= tol, (dtype, p, np.abs(row - ref[p]).max())
+        if dtype == "bfloat16":
+            assert 8192 in widths, widths          # both layers of the two widest portions
 
 
 def test_serving_loop_under_random_pressure(model_dirs):

@@ -939,6 +939,119 @@ def test_attn_prefill_peaked_scores_find_single_keys():
     assert hits > 0.9 * n
 
 
+def build_long_attention_case(nh, nkv, hd, ps, seqs, width, seed=0):
+    """``build_attention_case`` for contexts of tens of thousands of keys (bfloat16): the cache is filled
+    with a few indexed copies instead of key by key, the pool starts as NaN (a key read from a page that
+    was never written shows), and the block tables are ``width`` wide."""
+    g = torch.Generator().manual_seed(seed)
+    dtype = torch.bfloat16
+    n_pages = sum(-(-c // ps) for c, _ in seqs) + 5
+    from flambeau_amd.kernels.ops import PagedLayerCache
+    cache = PagedLayerCache(torch.full((n_pages, 2, nkv, ps, hd), float("nan"), dtype=dtype, device=DEV))
+    perm = torch.randperm(n_pages, generator=g)
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    used, K, V = 0, [], []
+    for s, (c, _) in enumerate(seqs):
+        nb = -(-c // ps)
+        table[s, :nb] = perm[used:used + nb].int()
+        used += nb
+        k = (torch.randn(c, nkv, hd, generator=g) * 0.8).to(dtype).to(DEV)
+        v = torch.randn(c, nkv, hd, generator=g).to(dtype).to(DEV)
+        K.append(k.double())
+        V.append(v.double())
+        t = torch.arange(c, device=DEV)
+        page, r = table[s].to(DEV)[t // ps].long(), t % ps
+        keys = cache.pool[:, 0].reshape(n_pages, nkv, ps, hd)
+        vals = cache.pool[:, 1].reshape(n_pages, nkv, hd, ps)
+        keys[page, :, r] = k                      # [c, nkv, hd]
+        vals[page, :, :, r] = v                   # values lie transposed inside a page
+    pos, tok_seq = [], []
+    for s, (c, ql) in enumerate(seqs):
+        pos += list(range(c - ql, c))
+        tok_seq += [s] * ql
+    n = len(pos)
+    q = (torch.randn(n, nh, hd, generator=g) * 0.8).to(dtype).to(DEV)
+    return dict(cache=cache, table=table.to(DEV), K=K, V=V, pos=pos, tok_seq=tok_seq, q=q, n=n,
+                pos_d=torch.tensor(pos, dtype=torch.int32, device=DEV),
+                seq_d=torch.tensor(tok_seq, dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 64, 0), (2, 1, 128, 0), (4, 2, 64, 5000), (2, 2, 256, 0)])
+def test_attn_prefill_with_block_tables_beyond_4096_pages(nh, nkv, hd, window):
+    """Portions behind 66,000 to 70,000 keys in pages of 16: block tables 8,192 wide, which a block keeps
+    in LDS beside its ring (one block per compute unit then, where two fit with narrower tables).  Random
+    queries against the float64 formula and the plain kernel; then queries that each single out one key
+    (the first of the context, keys either side of page 4,096, the window's first key, a near one)."""
+    ps, width = 16, 8192
+    assert tuned().prefill_max_pages(hd) >= width
+    seqs = [(70000, 136), (66000, 64), (300, 300), (65552, 70)]
+    case = build_long_attention_case(nh, nkv, hd, ps, seqs, width, seed=8)
+    assert tuned().prefill_supported(case["cache"], case["table"], window)
+    n = case["n"]
+    scale = 1 / math.sqrt(hd)
+    tiles = tiles_for(seqs)
+    q2 = case["q"].reshape(n, nh * hd)
+    ref = attention_case_ref(case, scale, window)
+    top = ref.abs().max()
+    plain = torch.empty_like(q2)
+    ops().attn_plain(q2, plain, case["cache"], case["pos_d"], case["seq_d"], case["table"], nh, scale, window)
+    assert (plain.double().reshape(n, nh, hd) - ref).abs().max() < 1e-2 * top
+    for n_split in (1, 5, tuned().attn_prefill_splits(tiles.shape[0], nh, nkv, hd, 70000)):
+        out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        part_o, part_ml = split_workspace(n, nh, hd, n_split) if n_split > 1 else (None, None)
+        tuned().attn_prefill(q2, out, case["cache"], tiles, case["pos_d"], case["table"], nh, scale, window,
+                             n_split=n_split, part_o=part_o, part_ml=part_ml)
+        err = (out.double().reshape(n, nh, hd) - ref).abs()
+        assert not torch.isnan(out).any(), n_split
+        assert err.max() < 1e-2 * top, f"{n_split} splits: worst at {np.unravel_index(int(err.argmax()), err.shape)}"
+        assert (out.double() - plain.double()).abs().max() < 1.5e-2 * top
+    # peaked: every query of the long requests picks one key, all heads of a kv head alike
+    q = case["q"].clone()
+    targets = {}
+    for i in range(n):
+        s, p = case["tok_seq"][i], case["pos"][i]
+        if seqs[s][0] < 60000:
+            continue
+        lo = max(0, p - window + 1) if window else 0
+        t = [lo, 65535, 65536, p - 3, lo + 17, 65519][i % 6]
+        t = min(max(t, lo), p)
+        targets[i] = t
+        for h in range(nh):
+            k = case["K"][s][t, h // (nh // nkv)]
+            q[i, h] = (k / k.norm() * 60.0 / scale / k.norm()).to(torch.bfloat16)       # the score of key t is 60
+    case["q"] = q
+    ref = attention_case_ref(case, scale, window)
+    hits = sum(float((ref[i, 0] - case["V"][case["tok_seq"][i]][t, 0]).abs().max()) < 0.05 for i, t in targets.items())
+    assert hits > 0.9 * len(targets)                    # the reference indeed picks single keys
+    for n_split in (1, 3):
+        out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        part_o, part_ml = split_workspace(n, nh, hd, n_split) if n_split > 1 else (None, None)
+        tuned().attn_prefill(q.reshape(n, nh * hd), out, case["cache"], tiles, case["pos_d"], case["table"], nh, scale, window,
+                             n_split=n_split, part_o=part_o, part_ml=part_ml)
+        assert (out.double().reshape(n, nh, hd) - ref).abs().max() < 2e-2 * ref.abs().max(), n_split
+
+
+def test_attn_prefill_table_limits_come_from_the_library():
+    """Tables wider than a block can keep are refused by the kernel, and the wrapper that chooses the
+    kernel asks the same function; with a window only the window's pages count."""
+    from flambeau_amd.kernels import KernelError
+    t = tuned()
+    assert t.prefill_max_pages(128) == 16384 and t.prefill_max_pages(64) == 16384 and 4096 < t.prefill_max_pages(256) < 16384
+    case = build_attention_case(torch.bfloat16, 2, 1, 16, 16, [(40, 40)], seed=1)
+    wide = torch.full((1, 20000), -1, dtype=torch.int32, device=DEV)
+    wide[:, :case["table"].shape[1]] = case["table"]
+    assert not t.prefill_supported(case["cache"], wide, 0)
+    assert t.prefill_supported(case["cache"], wide, 1000)
+    assert t.prefill_supported(case["cache"], wide[:, :16384].contiguous(), 0)
+    q2 = case["q"].reshape(40, 32)
+    with pytest.raises(KernelError, match="pages per request"):
+        t.attn_prefill(q2, torch.empty_like(q2), case["cache"], tiles_for([(40, 40)]), case["pos_d"], wide, 2, 0.25, 0)
+    out = torch.full_like(q2, float("nan"))
+    t.attn_prefill(q2, out, case["cache"], tiles_for([(40, 40)]), case["pos_d"], wide, 2, 0.25, 24)      # a window: taken
+    ref = attention_case_ref(case, 0.25, 24)
+    assert (out.double().reshape(40, 2, 16) - ref).abs().max() < 1e-2 * ref.abs().max()
+
+
 # ---------------------------------------------------------------- gated feed-forward in the product's epilogue
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,I,K", [(1, 14336, 4096), (8, 224, 96), (64, 136, 80), (5, 13, 40), (200, 14336, 512),

@@ -206,6 +206,23 @@ def test_attention_special_cases():
     np.testing.assert_allclose(a, b, atol=1e-12)
 
 
+def test_attention_in_batches_of_queries_is_the_whole_matrix():
+    """More queries than one batch of the implementation's loop (256), with and without a window,
+    against the library form over the whole score matrix; and queries at a few rows only."""
+    rng = np.random.default_rng(6)
+    n, nh, nkv, hd = 700, 4, 2, 8
+    q = rng.normal(size=(n, nh, hd))
+    k, v = (rng.normal(size=(n, nkv, hd)) for _ in range(2))
+    kr, vr = np.repeat(k, 2, axis=1), np.repeat(v, 2, axis=1)
+    pos = np.arange(n) + 11
+    for window in (0, 1, 90, 300):
+        want = _library_attention(q, kr, vr, 0.3, _causal_mask(n, window))
+        np.testing.assert_allclose(pm.attention(q, k, v, pos, 0.3, window), want, atol=1e-12)
+        rows = np.array([0, 255, 256, 511, 699, 3])
+        got = pm.attention(q[rows], k, v, pos[rows], 0.3, window, key_positions=pos)
+        np.testing.assert_allclose(got, want[rows], atol=1e-12)
+
+
 # ---------------------------------------------------------------- feed-forward
 def test_swiglu():
     """silu(g) = g * sigmoid(g); the gate, not the up projection, goes through it
@@ -282,6 +299,17 @@ def test_forward_layer_types_switch_the_window_per_layer():
     assert np.abs(mixed - base).max() > 1e-6 and np.abs(mixed - free).max() > 1e-6
     # only the second layer has the window: the same as a model whose other layers see everything
     np.testing.assert_array_equal(mixed[:4], free[:4])            # (no difference before the window bites)
+
+
+def test_forward_at_some_rows_is_the_whole_forward_at_those_rows():
+    rng = np.random.default_rng(10)
+    for L, window in ((1, None), (3, 6), (2, None)):
+        cfg, w = _random_model(rng, L=L, window=window)
+        toks = list(rng.integers(0, 30, 40))
+        full = pm.forward(cfg, w, toks)
+        rows = [39, 0, 17, 18]
+        np.testing.assert_allclose(pm.forward(cfg, w, toks, rows=rows), full[rows], atol=1e-11)
+        np.testing.assert_allclose(pm.forward(cfg, w, toks, rows=rows, keep_layers=[]), pm.forward(cfg, w, toks, keep_layers=[])[rows], atol=1e-12)
 
 
 def test_forward_tied_head_uses_the_embedding_table():
