@@ -32,6 +32,7 @@ int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
                   const int* positions, const int* tok_seq, const int* block_table,
                   int max_blocks, int n, int nh, int nkv, int hd, int page_size, int n_pages,
                   float scale, int window, hipStream_t stream);
+int fl_attn_max_head_dim(void);             // the largest head size the attention kernels take
 int fl_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n, int I,
                 hipStream_t stream);
 int fl_feed_tokens(int* tokens, const int* ids, const int* src, int n, hipStream_t stream);
@@ -45,6 +46,7 @@ int fl_sample_filtered(const float* logits, const float* inv_temp, const float* 
                        const float* top_p, const float* min_p, int* out, int rows, int V, unsigned* stash,
                        hipStream_t stream);
 int fl_sample_filtered_max_k(void);
+int fl_sample_filtered_max_vocab(void);      // the largest vocabulary fl_sample_filtered takes
 // Penalties over the tokens a request has generated (counts[slot][V], 16-bit, one row per state slot) and
 // logit bias, in place on the step's logits before the draw; slot[r] < 0 (as a float): the row has none.
 int fl_sample_penalise(float* logits, int rows, int V, const unsigned short* counts, const float* slot,

@@ -471,6 +471,9 @@ __global__ __launch_bounds__(256) void attn_plain_kernel(
     }
 }
 
+// The largest head size any attention kernel of the library takes (the plain kernel keeps a head in LDS).
+extern "C" int fl_attn_max_head_dim(void) { return FL_PLAIN_MAX_HD; }
+
 extern "C" int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
                              const int* positions, const int* tok_seq, const int* block_table,
                              int max_blocks, int n, int nh, int nkv, int hd, int page_size,
@@ -573,7 +576,6 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
                                                      const float* __restrict__ inv_temp,
                                                      const float* __restrict__ uniform,
                                                      int* __restrict__ out, int V) {
-    __shared__ float red[4];
     __shared__ float chunk_sum[256];
     __shared__ float sv[4];
     __shared__ int si[4];
@@ -617,8 +619,12 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
         for (; i < hi; ++i) part += expf((row[i] - mx) * it);
     }
     chunk_sum[threadIdx.x] = part;
-    const float total = block_sum<4>(part, red);
+    __syncthreads();
     if (threadIdx.x == 0) {
+        // the total is the chunks' sums added in index order, as the walk below takes them away again:
+        // the target can never outlast the last chunk by rounding, and nothing depends on a tree's shape
+        float total = 0.f;
+        for (int c = 0; c < 256; ++c) total += chunk_sum[c];
         float target = uniform[r] * total;
         int chosen = -1;
         int c = 0;

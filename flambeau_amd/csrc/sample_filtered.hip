@@ -315,3 +315,4 @@ extern "C" int fl_sample_filtered(const float* logits, const float* inv_temp, co
 }
 
 extern "C" int fl_sample_filtered_max_k(void) { return SF_MAX_K; }
+extern "C" int fl_sample_filtered_max_vocab(void) { return 255 * SF_THREADS; }

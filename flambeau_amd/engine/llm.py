@@ -120,7 +120,7 @@ class LLMEngine:
             else:
                 entries.append(StepEntry(r.request_id, s.tokens, want))
         rows = [s for s in sched if s.sample]
-        on_device = self.options.gpu_sampler and all(s.request.params.device_ok for s in rows)
+        on_device = self.options.gpu_sampler and all(s.request.params.device_takes(self.model.spec.vocab_size) for s in rows)
         logits = self.runner.step(entries)
         if on_device:
             if any(PENDING in r.output and r.params.has_penalties and self._slot(r) is not None
@@ -145,7 +145,7 @@ class LLMEngine:
         finished += self.flush()
         sampled = {}
         live = [i for i, s in enumerate(rows) if s.request.status != "finished"]   # (a stop token of the step before may just have ended one)
-        on_dev = [i for i in live if self.options.gpu_sampler and rows[i].request.params.device_ok]
+        on_dev = [i for i in live if self.options.gpu_sampler and rows[i].request.params.device_takes(self.model.spec.vocab_size)]
         if on_dev:
             params = [rows[i].request.params for i in on_dev]
             inv_t = [0.0 if p.is_greedy else 1.0 / p.temperature for p in params]

@@ -183,6 +183,12 @@ def attn_plain(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, 
     return out
 
 
+def attention_max_head_dim() -> int:
+    """The largest head size the attention kernels take (a host function: no GPU needed)."""
+    from .library import load
+    return load().fl_attn_max_head_dim()
+
+
 def silu_mul(gu, out):
     n, two_i = gu.shape
     I = two_i // 2

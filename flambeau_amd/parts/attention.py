@@ -16,6 +16,7 @@ import math
 
 import torch
 
+from ..config.base import ConfigError
 from ..kernels import ops
 from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, Product, TensorSpec
 
@@ -30,6 +31,10 @@ class PagedGQAAttention(Mixer):
                  position: PartSpec, window: int = 0, scale: float | None = None):
         if n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} query heads are not a multiple of {n_kv_heads} key/value heads")
+        if head_dim > ops.attention_max_head_dim():
+            # refused when the model is built, not at its first step
+            raise ConfigError(f"paged_gqa_attention: 'head_dim' {head_dim} is beyond what the attention kernels take "
+                              f"(head sizes up to {ops.attention_max_head_dim()})")
         self.hidden_size = hidden_size
         self.n_heads = n_heads
         self.n_kv_heads = n_kv_heads

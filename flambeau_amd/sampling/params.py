@@ -6,6 +6,7 @@ from dataclasses import dataclass, field
 
 DEVICE_TOP_K_MAX = 2048       # candidates the device sampler keeps (fl_sample_filtered_max_k)
 DEVICE_BIAS_MAX = 256         # logit-bias entries of one request that the device sampler takes
+DEVICE_FILTER_VOCAB_MAX = 261120     # the largest vocabulary the filtered draw takes (fl_sample_filtered_max_vocab)
 
 
 @dataclass
@@ -50,6 +51,13 @@ class SamplingParams:
         (top-k up to 2048, top-p, min-p) run on the device; what is beyond goes to the host sampler."""
         return not ((self.logit_bias is not None and len(self.logit_bias) > DEVICE_BIAS_MAX)
                     or (self.top_k is not None and self.top_k > DEVICE_TOP_K_MAX))
+
+    def device_takes(self, vocab_size: int) -> bool:
+        """``device_ok`` for a model's vocabulary: the filtered draw keeps a count per 1,024 tokens in a
+        byte, so filters over a vocabulary beyond 261,120 go to the host sampler too."""
+        if self.has_filters and not self.is_greedy and vocab_size > DEVICE_FILTER_VOCAB_MAX:
+            return False
+        return self.device_ok
 
     @property
     def penalties(self) -> tuple:

@@ -129,3 +129,21 @@ def test_config_from_dir(tmp_path):
         config_from_dir(tmp_path)
     with pytest.raises(ConfigError, match="no such file"):
         config_from_dir(tmp_path / "nowhere")
+
+
+def test_sizes_no_kernel_takes_are_refused_when_the_model_is_built():
+    """A head size beyond the attention kernels' limit passes the configuration (it is a kernel's limit,
+    not the architecture's) and is refused when the model's parts are made, before any weight is read
+    or any step runs, with an error that names the key."""
+    from flambeau_amd.kernels import ops
+    from flambeau_amd.models.mistral import mistral_spec
+    from flambeau_amd.parts import BLOCKS
+    limit = ops.attention_max_head_dim()
+    assert limit >= 256
+    raw = dict(architectures=["MistralForCausalLM"], hidden_size=64, num_hidden_layers=1, num_attention_heads=2,
+               num_key_value_heads=1, intermediate_size=96, vocab_size=50, rms_norm_eps=1e-5, max_position_embeddings=64)
+    ok = mistral_spec(MistralConfig.from_dict(dict(raw, head_dim=limit), "config"))
+    BLOCKS.create(ok.layers[0].block)
+    spec = mistral_spec(MistralConfig.from_dict(dict(raw, head_dim=limit + 16), "config"))
+    with pytest.raises(ConfigError, match="'head_dim'"):
+        BLOCKS.create(spec.layers[0].block)

@@ -688,3 +688,76 @@ def test_serving_loop_under_random_pressure(model_dirs):
             n_pre += eng.scheduler.n_preemptions
             n_stopped += sum(len(g) < new for g in got)
     assert n_pre > 0 and n_stopped > 0          # the cases did pre-empt, and did stop requests early
+
+
+def test_arrivals_and_aborts_while_a_step_is_in_flight(model_dirs):
+    """Requests that arrive while others decode, and aborts at random steps (of waiting requests, of
+    requests in the middle of their prompt, of requests whose last token the host has not seen yet),
+    through the serving loop with tight pools: a surviving request's tokens are those it gets alone, an
+    aborted request's tokens so far are a prefix of those, and every page and slot comes back.  (The
+    reference checks the same of its sessions: crates/forward/tests/multi_session_leak.rs:180-193;
+    requests join its running batch in crates/server/src/routes.rs:631-733.)"""
+    from flambeau_amd import EngineOptions, LLMEngine, SamplingParams
+    from flambeau_amd.engine import load_model
+    from flambeau_amd.engine.scheduler import PENDING
+    seen = dict(pending=0, waiting=0, prompt=0, joined=0, preempted=0, survivors=0)
+    for name, ps in (("A", 8), ("D", 8)):
+        d = model_dirs[(name, "float32")]
+        vocab = TINY[name]["config"]["vocab_size"]
+        ctx = min(TINY[name]["config"]["max_position_embeddings"], 200)
+        model, _ = load_model(d, dtype="float32", max_batch_tokens=ctx + 8)
+        alone = LLMEngine(model, EngineOptions(dtype="float32", inflight_slots=1, prefill_chunk_tokens=ctx, page_size=ps, ctx_cap=ctx))
+        for case in range(25):
+            rng = np.random.default_rng(7000 + 100 * ps + case + (500 if name == "D" else 0))
+            n_req = int(rng.integers(4, 9))
+            new = int(rng.integers(6, 30))
+            prompts = [[int(t) for t in rng.integers(0, vocab, int(rng.integers(1, ctx - new - 1)))] for _ in range(n_req)]
+            stops = tuple(int(t) for t in rng.integers(0, vocab, int(rng.integers(0, 6))))
+            params = [SamplingParams(max_tokens=new, temperature=float(rng.choice([0.0, 0.8])), seed=300 + i,
+                                     top_k=int(rng.integers(2, 40)) if rng.random() < 0.3 else None,
+                                     repetition_penalty=1.3 if rng.random() < 0.2 else 1.0, stop_token_ids=stops)
+                      for i in range(n_req)]
+            want = [alone.generate([p], sp)[0] for p, sp in zip(prompts, params)]
+            longest = -(-(max(len(p) for p in prompts) + new) // ps)
+            slots = int(rng.integers(2, 5))
+            pages = longest + int(rng.integers(1, 2 * longest))
+            chunk = int(rng.choice([16, 64, ctx]))
+            eng = LLMEngine(model, EngineOptions(dtype="float32", inflight_slots=slots, prefill_chunk_tokens=chunk, page_size=ps,
+                                                 paged_kv=pages, ctx_cap=ctx, max_batch_tokens=ctx + 8))
+            arrive = sorted(int(a) for a in rng.integers(0, 25, n_req))
+            arrive[0] = 0
+            kill = {i: int(rng.integers(a, a + 30)) for i, a in enumerate(arrive) if rng.random() < 0.4}
+            reqs, aborted, step_no = {}, set(), 0
+            what = f"{name} case {case}: slots {slots}, pages {pages}, portions {chunk}"
+            while len(reqs) < n_req or eng.has_work():
+                for i, a in enumerate(arrive):
+                    if a == step_no:
+                        seen["joined"] += any(r.status == "running" and r.output for r in reqs.values())
+                        reqs[i] = eng.add_request(prompts[i], params[i], request_id=f"r{i}")
+                for i, k in kill.items():
+                    if k == step_no and i in reqs and reqs[i].status != "finished":
+                        r = reqs[i]
+                        seen["pending"] += PENDING in r.output
+                        seen["waiting"] += r.status == "waiting"
+                        seen["prompt"] += r.status == "running" and not r.output
+                        assert eng.abort(f"r{i}"), what
+                        assert r.status == "finished" and r.finish_reason == "abort"
+                        aborted.add(i)
+                if eng.has_work():
+                    eng.step()
+                step_no += 1
+                assert step_no < 3000, what
+            eng.flush()
+            eng.runner.manager.check_invariants()
+            assert not eng.runner.manager.live and all(f == pages for f in eng.runner.manager.free_pages()), what
+            assert eng.runner.manager.n_free_slots == slots, what
+            seen["preempted"] += eng.scheduler.n_preemptions
+            for i in range(n_req):
+                out = [t for t in reqs[i].output if t != PENDING]
+                if i in aborted:
+                    assert out == want[i][:len(out)], f"{what}: the tokens of aborted request {i} differ"
+                else:
+                    seen["survivors"] += 1
+                    assert list(reqs[i].output) == want[i], f"{what}: request {i} differs (aborted: {sorted(aborted)})"
+            assert not eng.abort("r0") and not eng.abort("nobody")          # finished or unknown: nothing to drop
+    assert all(v > 0 for v in seen.values()), seen

@@ -984,7 +984,7 @@ def test_attn_prefill_with_block_tables_beyond_4096_pages(nh, nkv, hd, window):
     (the first of the context, keys either side of page 4,096, the window's first key, a near one)."""
     ps, width = 16, 8192
     assert tuned().prefill_max_pages(hd) >= width
-    seqs = [(70000, 136), (66000, 64), (300, 300), (65552, 70)]
+    seqs = [(70000, 72), (300, 200), (65552, 66)]
     case = build_long_attention_case(nh, nkv, hd, ps, seqs, width, seed=8)
     assert tuned().prefill_supported(case["cache"], case["table"], window)
     n = case["n"]

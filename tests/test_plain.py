@@ -378,6 +378,36 @@ def test_xoshiro_matches_hand_computed_values():
     assert [pm.Xoshiro(42).next_u64() for _ in range(2)] == [pm.Xoshiro(42).next_u64()] * 2
 
 
+def test_seeding_vector_for_seed_zero():
+    """The four state words for seed 0, written out.  The first is SplitMix64's published first output
+    from state 0 (0xE220A8397B1DCDAF: its increment added once, then its mixer).  The reference's
+    loop (crates/runtime/src/sampling.rs:116-131) then differs from SplitMix64 proper: it does not add
+    the increment again but mixes the running value in place (the value before the last xor-shift is
+    carried on), so the second word is NOT SplitMix64's second output 0x6E789E6AA1B965F4.  The words are
+    recomputed here with wrapping 64-bit machine arithmetic, step by step, not with masked big integers."""
+    want = [0xE220A8397B1DCDAF, 0x622CF263EEB1289A, 0xC17A83783EC77EE4, 0xCCF1FA6DFE5D7959]
+    assert pm.Xoshiro(0).s == want
+    assert pm.Xoshiro(0).s[1] != 0x6E789E6AA1B965F4
+    u = np.uint64
+    with np.errstate(over="ignore"):
+        x = u(0) + u(0x9E3779B97F4A7C15)
+        words = []
+        for _ in range(4):
+            x = x ^ (x >> u(30))
+            x = x * u(0xBF58476D1CE4E5B9)
+            x = x ^ (x >> u(27))
+            x = x * u(0x94D049BB133111EB)
+            words.append(int(x ^ (x >> u(31))))
+    assert words == want
+    # and the first numbers drawn from that state: (1 + 2^-24 steps in [0, 1))
+    g = pm.Xoshiro(0)
+    first = g.next_u64()
+    s1 = want[1]
+    by_hand = (((s1 * 5) % 2 ** 64 << 7 | (s1 * 5) % 2 ** 64 >> 57) % 2 ** 64 * 9) % 2 ** 64
+    assert first == by_hand
+    assert pm.Xoshiro(0).next_f32() == (by_hand >> 40) / 2 ** 24
+
+
 def test_sampler_rules():
     """The cases of crates/runtime/src/sampling.rs:752-939."""
     logits = np.array([0.1, 2.0, -1.0, 1.9, 0.5], dtype=np.float32)

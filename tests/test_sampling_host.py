@@ -43,6 +43,15 @@ def test_parameter_checks():
     assert not SamplingParams(temperature=1.0, top_k=2049).device_ok
     assert SamplingParams(repetition_penalty=1.1).device_ok and SamplingParams(logit_bias={3: 1.0}).device_ok
     assert not SamplingParams(logit_bias={t: 1.0 for t in range(257)}).device_ok
+    # a vocabulary beyond what the filtered draw takes sends filters (and only them) to the host sampler
+    from flambeau_amd.kernels.library import load
+    from flambeau_amd.sampling.params import DEVICE_FILTER_VOCAB_MAX, DEVICE_TOP_K_MAX
+    lib = load()
+    assert lib.fl_sample_filtered_max_vocab() == DEVICE_FILTER_VOCAB_MAX and lib.fl_sample_filtered_max_k() == DEVICE_TOP_K_MAX
+    assert SamplingParams(temperature=1.0, top_p=0.9).device_takes(DEVICE_FILTER_VOCAB_MAX)
+    assert not SamplingParams(temperature=1.0, top_p=0.9).device_takes(DEVICE_FILTER_VOCAB_MAX + 1)
+    assert SamplingParams(temperature=1.0).device_takes(300000) and SamplingParams(top_k=5).device_takes(300000)   # no filter; greedy
+    assert not SamplingParams(temperature=1.0, top_k=3000).device_takes(1000)
     assert SamplingParams(presence_penalty=0.5, frequency_penalty=0.25).penalties == (1.0, 0.5, 0.25)
     assert SamplingParams(temperature=1.0, top_p=0.9).device_filters == (2048, 0.9, 0.0)
     assert SamplingParams(temperature=1.0, top_k=7, min_p=0.1).device_filters == (7, 0.0, 0.1)
