@@ -180,10 +180,17 @@ typedef union FlArg { void* p; long l; int i; float f; } FlArg;
 void* fl_program_new(void);
 void fl_program_free(void* program);
 int fl_program_size(const void* program);
-// name: one of the launch functions above (those that take a stream); args: its arguments in order,
-// the stream's value is ignored
+// name: a launch function the recorder knows (every function above that takes a stream); args: its
+// arguments in order, the stream's value is ignored
 int fl_program_append(void* program, const char* name, const FlArg* args, int n_args);
 int fl_program_run(const void* program, hipStream_t stream, int* failed_at);
+// What the recorder knows: launch functions register themselves (FL_RECORDABLE in recordable.h puts a
+// registrar beside a definition); a launch function of another library is added with
+// fl_program_register, `call` being a function that unpacks the recorded arguments and calls it with
+// the stream given.  fl_program_knows: the number of arguments (stream included) or -1.
+typedef int (*FlTrampoline)(const FlArg* args, hipStream_t stream);
+int fl_program_register(const char* name, FlTrampoline call, int n_args);
+int fl_program_knows(const char* name);
 
 #ifdef __cplusplus
 }

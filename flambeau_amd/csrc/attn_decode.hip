@@ -31,6 +31,7 @@
 // attention_decode_f16_splitk.cu:31-256 (partials and merge).
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 #include "attn_merge.h"
 #include <mutex>
 
@@ -371,6 +372,7 @@ extern "C" int fl_attn_decode(const void* q, void* out, float* part_o, float* pa
     return attn_decode_launch("attn_decode", q, out, part_o, part_ml, cache_base, items, n_items, block_table, max_blocks,
                               nh, nkv, hd, page_size, n_pages, scale, window, n_split, stream);
 }
+FL_RECORDABLE(fl_attn_decode)
 
 // Items with splits of their own: items[i] = (row, position, request, split + 256 * splits), the splits of
 // a row one after the other from split 0 on (up to 255), row < 0 for a place that is not used.  part_o
@@ -385,6 +387,7 @@ extern "C" int fl_attn_decode_items(const void* q, void* out, float* part_o, flo
     return attn_decode_launch("attn_decode_items", q, out, part_o, part_ml, cache_base, items, n_items, block_table, max_blocks,
                               nh, nkv, hd, page_size, n_pages, scale, window, 1, stream, true, firsts, n_rows);
 }
+FL_RECORDABLE(fl_attn_decode_items)
 
 // ---- the same without any allocation: the splits' partial results go to an array that is part of
 // the library's image on every GPU.  `scratch` is a host-side stand-in for that array, not a device
@@ -438,3 +441,4 @@ extern "C" int fl_attn_decode_static(const void* q, void* out, const void* cache
     return attn_decode_launch("attn_decode_static", q, out, part_o, part_ml, cache_base, items, n_items, block_table,
                               max_blocks, nh, nkv, hd, page_size, n_pages, scale, window, n_split, stream);
 }
+FL_RECORDABLE(fl_attn_decode_static)

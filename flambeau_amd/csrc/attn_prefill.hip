@@ -24,6 +24,7 @@
 // prefill, 4 query rows per tile), attention_prefill_f16_paged.cu:50-150 (paged addressing).
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 #include "attn_merge.h"
 
 #define PF_TOKENS 64          // query tokens per block
@@ -584,3 +585,4 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     }
     return 0;
 }
+FL_RECORDABLE(fl_attn_prefill)

@@ -29,6 +29,7 @@
 // (crates/kernels-hip/src/kernels/dense_gemv_f16_f16_batched.cu:17-63).
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 
 
 template <typename TOut>
@@ -392,17 +393,20 @@ extern "C" int fl_gemm_mid_ex(const void* x, const void* w_packed, void* out, fl
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_mid_ex)
 
 extern "C" int fl_gemm_mid_scaled(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                                   int M, int N, int K, int epilogue, int out_cols, const float* in_ssq, int in_parts,
                                   float eps, hipStream_t stream) {
     return fl_gemm_mid_ex(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, in_ssq, in_parts, eps, 0, 0, stream);
 }
+FL_RECORDABLE(fl_gemm_mid_scaled)
 
 extern "C" int fl_gemm_mid(const void* x, const void* w_packed, void* out, float* workspace, int out_dtype,
                            int M, int N, int K, int epilogue, int out_cols, hipStream_t stream) {
     return fl_gemm_mid_scaled(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, stream);
 }
+FL_RECORDABLE(fl_gemm_mid)
 
 // The K-splits of x w^T left apart: workspace[s][M][N] for s < fl_gemm_mid_splits(M, N, K) (one "split"
 // if K is not split), for a kernel that adds them itself (fl_rope_kv_write).  in_ssq as in
@@ -420,6 +424,7 @@ extern "C" int fl_gemm_mid_partials(const void* x, const void* w_packed, float* 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_mid_partials)
 
 // resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_mid_parts(N)] =
 // sums of resid^2 over 4096 columns each: the factors of the norm that follows.  The workspace holds
@@ -441,6 +446,7 @@ extern "C" int fl_gemm_mid_residual(const void* x, const void* w_packed, float* 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_mid_residual)
 
 extern "C" int fl_gemm_mid_parts(int N) { return ceil_div(N, GM_RED_COLS); }
 
@@ -459,3 +465,4 @@ extern "C" int fl_reduce_residual(const float* part, float* resid, const float* 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_reduce_residual)

@@ -33,6 +33,7 @@
 // (crates/kernels-hip/src/kernels/dense_gemv_f16_f16.cu:27-71, ..._batched.cu:17-63).
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 #include "rope_store.h"
 
 __device__ __forceinline__ void store4(float* p, f32x4 v) { *(f32x4*)p = v; }
@@ -484,6 +485,7 @@ extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, in
     const SkinnyFusion none = {nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr};
     return skinny_entry(x, w_packed, out, out_dtype, M, N, K, nw_hint, epilogue, out_cols, none, RopeStore{}, stream);
 }
+FL_RECORDABLE(fl_gemm_skinny)
 
 // The same product fused with the norms around it.  in_ssq (or null): [M, in_parts] partial sums of
 // squares of the rows that x was made from; every token's results are multiplied by
@@ -500,6 +502,7 @@ extern "C" int fl_gemm_skinny_fused(const void* x, const void* w_packed, void* o
     return skinny_entry(x, w_packed, out, epilogue == EPI_RESIDUAL ? FL_F32 : out_dtype, M, N, K, 0, epilogue,
                         out_cols, fu, RopeStore{}, stream);
 }
+FL_RECORDABLE(fl_gemm_skinny_fused)
 
 // The joined q/k/v projection of at most 16 rows with its rows in paired order: q is rotated and
 // written to q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens'
@@ -514,5 +517,6 @@ extern "C" int fl_gemm_skinny_rope(const void* x, const void* w_packed, int M, i
                           PagedCache{cache_base, nkv, page_size, hd, n_pages}, nh, rot, write_cache};
     return skinny_entry(x, w_packed, q_out, FL_BF16, M, N, K, 0, EPI_ROPE, N, fu, rs, stream);
 }
+FL_RECORDABLE(fl_gemm_skinny_rope)
 
 extern "C" int fl_gemm_skinny_blocks(int N) { return ceil_div(N, 16); }

@@ -32,6 +32,7 @@
 #include <type_traits>
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 #include "rope_store.h"
 
 #define TG_PLAIN 0                       // epilogues
@@ -547,18 +548,21 @@ extern "C" int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_tiled_ex)
 
 extern "C" int fl_gemm_tiled_scaled(const void* x, const void* w_packed, void* out, float* workspace,
                                     int out_dtype, int M, int N, int K, int epilogue, int out_cols,
                                     const float* in_ssq, int in_parts, float eps, hipStream_t stream) {
     return fl_gemm_tiled_ex(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, in_ssq, in_parts, eps, 0, 0, stream);
 }
+FL_RECORDABLE(fl_gemm_tiled_scaled)
 
 extern "C" int fl_gemm_tiled(const void* x, const void* w_packed, void* out, float* workspace,
                              int out_dtype, int M, int N, int K, int epilogue, int out_cols,
                              hipStream_t stream) {
     return fl_gemm_tiled_ex(x, w_packed, out, workspace, out_dtype, M, N, K, epilogue, out_cols, nullptr, 0, 0.f, 0, 0, stream);
 }
+FL_RECORDABLE(fl_gemm_tiled)
 
 // resid[M, N] += x w^T (float, in place), xg[M, N] = bf16(resid * g), out_ssq[M, fl_gemm_tiled_residual_parts(M, N, K)]
 // = the sums of resid^2 in parts: the factors of the norm that follows.  Where K is not split the
@@ -592,11 +596,13 @@ extern "C" int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, fl
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_tiled_residual_ex)
 
 extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
                                       float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream) {
     return fl_gemm_tiled_residual_ex(x, w_packed, workspace, M, N, K, resid, g, xg, out_ssq, 0, stream);
 }
+FL_RECORDABLE(fl_gemm_tiled_residual)
 
 // Parts in which fl_gemm_tiled_residual leaves a token's sum of squares.
 extern "C" int fl_gemm_tiled_residual_parts(int M, int N, int K) {
@@ -622,6 +628,7 @@ extern "C" int fl_gemm_tiled_partials(const void* x, const void* w_packed, float
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_tiled_partials)
 
 // The joined q/k/v projection of many rows with its rows in paired order: q is rotated and written to
 // q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens' positions; cs[M,
@@ -652,6 +659,7 @@ extern "C" int fl_gemm_tiled_rope_ex(const void* x, const void* w_packed, int M,
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_tiled_rope_ex)
 
 extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, int N, int K, const float* in_ssq,
                                   int in_parts, float eps, const int* positions, const int* tok_seq,
@@ -661,3 +669,4 @@ extern "C" int fl_gemm_tiled_rope(const void* x, const void* w_packed, int M, in
     return fl_gemm_tiled_rope_ex(x, w_packed, M, N, K, in_ssq, in_parts, eps, positions, tok_seq, block_table, max_blocks, cs,
                                  q_out, cache_base, nh, nkv, hd, page_size, n_pages, rot, write_cache, 0, stream);
 }
+FL_RECORDABLE(fl_gemm_tiled_rope)

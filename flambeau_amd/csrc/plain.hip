@@ -12,6 +12,7 @@
 //   SiLU gate crates/kernels-hip/src/kernels/swiglu_f32_to_f16.cu:21-23
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 
 // ------------------------------------------------------------------ embedding
 template <typename T>
@@ -48,6 +49,7 @@ extern "C" int fl_embed(const void* table, int dtype, const int* tokens, float* 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_embed)
 
 // ------------------------------------------------------------------ RMSNorm
 // out[r,:] = v * w * rsqrt(mean(v^2) + eps), v = x[src,:] (+ delta[src,:]); src = rows ? rows[r] : r.
@@ -164,6 +166,7 @@ extern "C" int fl_rmsnorm(const float* x, const float* delta, float* resid_out, 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_rmsnorm)
 
 // ------------------------------------------------------------------ residual add
 __global__ __launch_bounds__(256) void add_kernel(float* __restrict__ x, const float* __restrict__ d, size_t n) {
@@ -178,6 +181,7 @@ extern "C" int fl_add_inplace(float* x, const float* delta, long n, hipStream_t 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_add_inplace)
 
 // ------------------------------------------------------------------ plain GEMM
 // out[m, n] = sum_k x[m,k] * w[n,k]; 64x64 tile per block, 4x4 per thread, k in steps of 16.
@@ -265,6 +269,7 @@ extern "C" int fl_gemm_plain(const void* x, const void* w, void* out, int in_dty
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_gemm_plain)
 
 // ------------------------------------------------------------------ rotation + cache write
 // cos and sin of every (token, pair) of a step: cs[token][i] = (cos, sin)(position * theta^(-2 i / rot)).
@@ -291,6 +296,7 @@ extern "C" int fl_rope_table(const int* positions, int n, int rot, float theta, 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_rope_table)
 
 // One block per (token, head) over the fused projection row [q heads | k heads | v heads].
 // Q heads: rotated, written to q_out.  K heads: rotated, written to the cache at the token's
@@ -386,6 +392,7 @@ extern "C" int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_rope_kv_write)
 
 // ------------------------------------------------------------------ plain attention over the cache
 // One block per (token, query head).  The query at position p sees the keys
@@ -493,6 +500,7 @@ extern "C" int fl_attn_plain(const void* q, void* out, const void* cache_base, i
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_attn_plain)
 
 // ------------------------------------------------------------------ SiLU gate
 // out[r, i] = silu(gu[r, i]) * gu[r, I + i], silu(g) = g / (1 + exp(-g)), all in float.
@@ -523,6 +531,7 @@ extern "C" int fl_silu_mul(const void* gu, int in_dtype, void* out, int out_dtyp
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_silu_mul)
 
 // ------------------------------------------------------------------ sampling
 // The better of two (value, index) candidates: the larger value, the smaller index among equals.
@@ -661,6 +670,7 @@ extern "C" int fl_feed_tokens(int* tokens, const int* ids, const int* src, int n
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_feed_tokens)
 
 extern "C" int fl_argmax(const float* logits, int* out, int rows, int V, hipStream_t stream) {
     FL_CHECK(rows >= 0 && V > 0, "argmax: bad sizes");
@@ -669,6 +679,7 @@ extern "C" int fl_argmax(const float* logits, int* out, int rows, int V, hipStre
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_argmax)
 
 extern "C" int fl_sample(const float* logits, const float* inv_temp, const float* uniform, int* out,
                          int rows, int V, hipStream_t stream) {
@@ -678,3 +689,4 @@ extern "C" int fl_sample(const float* logits, const float* inv_temp, const float
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_sample)

@@ -23,6 +23,7 @@
 // Rows without a filter (and greedy rows) are left alone: fl_sample draws them.
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 
 #define SF_MAX_K 2048
 #define SF_THREADS 1024
@@ -313,6 +314,7 @@ extern "C" int fl_sample_filtered(const float* logits, const float* inv_temp, co
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_sample_filtered)
 
 extern "C" int fl_sample_filtered_max_k(void) { return SF_MAX_K; }
 extern "C" int fl_sample_filtered_max_vocab(void) { return 255 * SF_THREADS; }

@@ -10,6 +10,7 @@
 // by the token drawn in every step.
 #include "common.h"
 #include "api.h"
+#include "recordable.h"
 
 // grid (blocks over the vocabulary, rows); rows whose slot is negative or whose penalties are neutral are skipped
 __global__ __launch_bounds__(256) void sample_penalise_kernel(float* __restrict__ logits, int V,
@@ -85,6 +86,7 @@ extern "C" int fl_sample_penalise(float* logits, int rows, int V, const unsigned
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_sample_penalise)
 
 extern "C" int fl_sample_bias(float* logits, int V, int n, const float* row, const float* token, const float* value,
                               hipStream_t stream) {
@@ -94,6 +96,7 @@ extern "C" int fl_sample_bias(float* logits, int V, int n, const float* row, con
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_sample_bias)
 
 // The drawn tokens join their requests' histories.
 extern "C" int fl_sample_count(unsigned short* counts, int V, int rows, const float* slot, const int* ids, hipStream_t stream) {
@@ -103,6 +106,7 @@ extern "C" int fl_sample_count(unsigned short* counts, int V, int rows, const fl
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_sample_count)
 
 // A request takes a slot: its row is zeroed and the n tokens it has generated so far are counted.
 extern "C" int fl_sample_history(unsigned short* counts, int V, int slot, const int* tokens, int n, hipStream_t stream) {
@@ -111,3 +115,4 @@ extern "C" int fl_sample_history(unsigned short* counts, int V, int slot, const 
     FL_LAUNCH_CHECK();
     return 0;
 }
+FL_RECORDABLE(fl_sample_history)

@@ -63,7 +63,9 @@ class ModelRunner:
         self._meta_copied = None     # event: the last metadata copy has left the pinned buffer
         # steps of single tokens replay a captured graph per batch-size bucket, if every mixer
         # of the model says that running a step twice leaves the same cache (graph_safe) and every part
-        # of it can be captured (a part that is not replayable may call what a capture does not allow)
+        # of it can be captured (a part that is not replayable may call what a capture does not allow); a
+        # model that cannot have its steps of single tokens recorded instead, and the recorded stretches
+        # around the blocks in question become graphs of their own
         self.decode_graphs = (bool(decode_graphs) and all(getattr(c, "graph_safe", False) for c in self._mixer_classes)
                               and getattr(model, "capturable", lambda: True)())
         self.max_graph_batch = min(max_graph_batch, max_slots)
@@ -305,24 +307,28 @@ class ModelRunner:
         if hit is not None and hit.valid == valid:
             self._programs.move_to_end(key)
             hit.hits += 1
-            whole = len(hit.stretches) == 1 and isinstance(hit.stretches[0], Program)
-            if whole and hit.graph is None and hit.hits >= self.graph_after_hits:
-                # a shape that keeps coming back: its launches become a graph (they are this
-                # library's kernels only, with fixed arguments), which costs one launch to replay
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
-                    hit.stretches[0].run(torch.cuda.current_stream().cuda_stream)
-                hit.graph = graph
-            if hit.graph is not None:
-                hit.graph.replay()
-            elif whole:
-                hit.stretches[0].run(stream)
+            if hit.hits >= self.graph_after_hits and not hit.graphs:
+                # a shape that keeps coming back: the launches of every recorded stretch become a graph
+                # (they are this library's kernels only, with fixed arguments), which costs one launch to
+                # replay; blocks that cannot be recorded still run as they are between the graphs
+                for i, s in enumerate(hit.stretches):
+                    if isinstance(s, Program):
+                        graph = torch.cuda.CUDAGraph()
+                        with torch.cuda.graph(graph):
+                            s.run(torch.cuda.current_stream().cuda_stream)
+                        hit.graphs[i] = graph
+            if len(hit.stretches) == 1 and isinstance(hit.stretches[0], Program):
+                if hit.graphs:
+                    hit.graphs[0].replay()
+                else:
+                    hit.stretches[0].run(stream)
             else:
-                # recorded stretches, and between them the blocks that cannot be replayed, run as they are
                 now = self._state_from(batch, parts, dev)
                 with ops.pinned_stream():
-                    for s in hit.stretches:
-                        if isinstance(s, Program):
+                    for i, s in enumerate(hit.stretches):
+                        if i in hit.graphs:
+                            hit.graphs[i].replay()
+                        elif isinstance(s, Program):
                             s.run(stream)
                         else:
                             s(now)
@@ -427,7 +433,7 @@ class _RecordedStep:
         self.logits = logits
         self.valid = valid          # (buffer generation, address of the metadata) the arguments belong to
         self.hits = 0
-        self.graph = None
+        self.graphs = {}            # index of a stretch -> the device graph of its launches
 
 
 class _GraphedStep:

@@ -35,6 +35,9 @@ _SIGNATURES = {
 }
 
 
+_functions: dict = {}     # name -> foreign function (of this library, or of a part's own)
+
+
 class KernelError(RuntimeError):
     """A kernel refused its arguments or its launch failed."""
 
@@ -59,17 +62,45 @@ def load():
     return lib
 
 
-def register_signatures(extra: dict) -> None:
-    """Further entry points (tuned kernels register theirs next to their wrappers)."""
+def register_signatures(extra: dict, library=None) -> None:
+    """Further entry points (tuned kernels register theirs next to their wrappers).  ``library``: a
+    ``ctypes.CDLL`` of the caller's own that holds them (a part that brings kernels of its own); such
+    launch functions return 0 or an error code and take the stream last, like this library's, and
+    become recordable with ``make_recordable``."""
     _SIGNATURES.update(extra)
-    if _lib is not None:
+    if library is not None:
+        for name, args in extra.items():
+            fn = getattr(library, name)
+            fn.argtypes = args
+            fn.restype = c_int
+            _functions[name] = fn
+    elif _lib is not None:
         for name, args in extra.items():
             fn = getattr(_lib, name)
             fn.argtypes = args
             fn.restype = c_int
 
 
-_functions: dict = {}
+def recordable(name: str) -> bool:
+    """Whether the recorder of step programs knows the launch function ``name``."""
+    lib = load()
+    lib.fl_program_knows.argtypes = [c_char_p]
+    return lib.fl_program_knows(name.encode()) >= 0
+
+
+def make_recordable(name: str, trampoline) -> None:
+    """Make a launch function of another library known to the recorder.  ``trampoline``: a C function
+    of that library, ``int (const FlArg* args, hipStream_t stream)``, that calls the launch function
+    with the recorded arguments and the stream given (a ctypes function pointer or an address); the
+    number of arguments comes from the signature registered under ``name``."""
+    lib = load()
+    lib.fl_program_register.argtypes = [c_char_p, c_void_p, c_int]
+    lib.fl_program_register.restype = c_int
+    address = ctypes.cast(trampoline, c_void_p).value if not isinstance(trampoline, int) else trampoline
+    if lib.fl_program_register(name.encode(), address, len(_SIGNATURES[name])) != 0:
+        raise KernelError(f"make_recordable {name}: {lib.fl_last_error().decode(errors='replace')}")
+
+
 _recording = None        # the Program that launches are being appended to, or None
 
 

@@ -533,6 +533,17 @@ def test_a_block_that_cannot_be_recorded_runs_between_recorded_stretches(model_d
     assert kinds and all(k == [True, False, True] for k in kinds)          # launches, the block, launches
     rh.compare(got, reqs, ref, dtype, "one unrecorded block: portions")
     rh.compare(got2, reqs, ref, dtype, "one unrecorded block: mixed")
+    # A stretch that keeps coming back becomes a device graph of its own, the block still runs between
+    # the graphs: steps of single tokens of this model, which cannot be captured whole, replay two graphs
+    # around one block run from Python.
+    runner = ModelRunner(model, n_pages=40, page_size=8, max_slots=4, max_logit_rows=256)
+    assert not runner.decode_graphs and runner.step_programs
+    runner.storage.fill(float("nan"))
+    got3 = rh.run_in_process(runner, rh.trace_tail(reqs, tail=32))
+    graphed = [r for r in runner._programs.values() if r.graphs]
+    assert graphed and all(sorted(r.graphs) == [0, 2] for r in graphed)
+    assert max(r.hits for r in graphed) > 10
+    rh.compare(got3, reqs, ref, dtype, "one unrecorded block: single tokens through graphs of stretches")
 
 
 @pytest.fixture(scope="module")

@@ -1,0 +1,89 @@
+"""The kernel library's interface as far as it can be checked without a GPU: its header, the argument
+lists the Python side holds, and what the recorder of step programs knows."""
+import ctypes
+import re
+from pathlib import Path
+
+from flambeau_amd.kernels import library
+from flambeau_amd.kernels import tuned  # noqa: F401  (registers the tuned kernels' argument lists)
+from flambeau_amd.sampling import device  # noqa: F401
+
+CSRC = Path(library.__file__).resolve().parent.parent / "csrc"
+
+
+def _declarations():
+    """``{name: [argument type texts]}`` of every ``int fl_*(...)`` declared in api.h."""
+    text = re.sub(r"//[^\n]*", "", (CSRC / "api.h").read_text())
+    out = {}
+    for m in re.finditer(r"\bint\s+(fl_\w+)\s*\(([^;]*?)\)\s*;", text, re.S):
+        args = [a.strip() for a in m.group(2).replace("\n", " ").split(",")]
+        out[m.group(1)] = [] if args == ["void"] else args
+    return out
+
+
+def _ctype_of(arg: str):
+    if "*" in arg or arg.startswith("hipStream_t"):
+        return library.P
+    if arg.startswith("float"):
+        return library.F
+    if arg.startswith("long"):
+        return library.L
+    assert arg.startswith("int") or arg.startswith("unsigned"), arg
+    return library.I
+
+
+def test_argument_lists_follow_the_header():
+    """Every argument list held on the Python side names a declared function and has its arguments' types
+    (a list one argument short or long corrupts the call without any error)."""
+    decl = _declarations()
+    assert len(decl) > 50
+    for name, types in library._SIGNATURES.items():
+        assert name in decl, f"{name} is not declared in api.h"
+        assert [_ctype_of(a) for a in decl[name]] == list(types), name
+
+
+def test_every_launch_function_is_recordable():
+    """A launch function (one whose last argument is the stream) registers itself with the recorder
+    beside its definition; the recorder's own file names no kernel."""
+    lib = library.load()
+    decl = _declarations()
+    launch = [n for n, a in decl.items() if a and a[-1].startswith("hipStream_t")]
+    assert len(launch) >= 37
+    lib.fl_program_knows.argtypes = [ctypes.c_char_p]
+    for name in launch:
+        assert lib.fl_program_knows(name.encode()) == len(decl[name]), name
+        assert library.recordable(name)
+    assert not library.recordable("fl_no_such_kernel") and not library.recordable("fl_attn_prefill_splits")
+    program = (CSRC / "program.hip").read_text()
+    body = program[program.index("namespace {"):]
+    assert not re.search(r"\bfl_(?!program_|set_error|last_error)\w+", body), "program.hip names a kernel"
+
+
+def test_a_launch_function_from_elsewhere_can_be_registered():
+    """``fl_program_register`` takes a trampoline for a function the library has never seen; a program
+    then records it by name (here the trampoline is a Python callback that notes what it was given)."""
+    lib = library.load()
+    seen = []
+    proto = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.POINTER(library.FlArg), ctypes.c_void_p)
+
+    def tramp(args, stream):
+        seen.append((args[0].i, round(args[1].f, 3), stream))
+        return 0 if args[0].i >= 0 else -7
+    cb = proto(tramp)
+    library._SIGNATURES["toy_launch"] = [library.I, library.F, library.P]
+    try:
+        library.make_recordable("toy_launch", cb)
+        assert library.recordable("toy_launch")
+        prog = library.Program()
+        prog.append("toy_launch", (5, 0.25, None))
+        prog.append("toy_launch", (-1, 1.5, None))
+        prog.append("toy_launch", (9, 2.0, None))
+        assert len(prog) == 3
+        try:
+            prog.run(1234)
+            raise AssertionError("the failing call did not stop the replay")
+        except library.KernelError as e:
+            assert "call 1" in str(e)
+        assert seen == [(5, 0.25, 1234), (-1, 1.5, 1234)]
+    finally:
+        del library._SIGNATURES["toy_launch"]
