@@ -28,6 +28,9 @@ int fl_rope_kv_write(const void* qkv, int in_dtype, int ld, const int* positions
                      int n_parts, long part_stride, hipStream_t stream);
 // cs[n][rot / 2][2]: cosine and sine of every (token, rotation pair) of a step
 int fl_rope_table(const int* positions, int n, int rot, float theta, float* cs, hipStream_t stream);
+// the same from frequencies of the caller's own: cs = magnitude * (cos, sin)(position * inv_freq[i]), inv_freq[rot / 2] double
+int fl_rope_table_ladder(const int* positions, int n, int rot, const double* inv_freq, float magnitude,
+                         float* cs, hipStream_t stream);
 int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
                   const int* positions, const int* tok_seq, const int* block_table,
                   int max_blocks, int n, int nh, int nkv, int hd, int page_size, int n_pages,

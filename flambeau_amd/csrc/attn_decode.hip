@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* part_o,
     float* part_ml, PagedCache cache, const int4* __restrict__ items,
     const int* __restrict__ block_table, int max_blocks, int nh, float scale, int window,
-    int n_split, int q_tiles, int ps_shift) {
+    int n_split, int q_tiles, int ps_shift, int item_base) {
     constexpr int QS = HDP / 32;     // k-steps of the score product
     constexpr int DT = HDP / 16;     // 16-wide tiles of head dims in the output
     constexpr bool PIPELINED = HDP <= 128;       // two chunks of keys and values fit the registers
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
     __shared__ f32x4 s_o[DEC_WAVES - 1][DT][64];     // wave 0 keeps its own in registers
 
     // (the items are the slow index of the grid: the places of a list that no row uses come last)
-    const int item = blockIdx.y;
+    const int item = item_base + blockIdx.y;
     const int kvh = blockIdx.x / q_tiles, qt = blockIdx.x % q_tiles;
     const int4 it = items[item];
     if (it.x < 0) return;                              // a place in the list that no row uses
@@ -329,25 +329,27 @@ static int attn_decode_launch(const char* who, const void* q, void* out, float* 
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
     const int G = nh / nkv;
     const int q_tiles = ceil_div(G, 16);
-    FL_CHECK(n_items <= 65535, "%s: %d items, at most 65535", who, n_items);
-    dim3 grid(nkv * q_tiles, n_items, own_splits ? 1 : n_split);
     const int hdp = ceil_div(hd, 32) * 32;
+    // a grid's slow index holds 65,535 places: longer lists of items take several launches
+    for (int item_base = 0; item_base < n_items; item_base += 65535) {
+        dim3 grid(nkv * q_tiles, min(n_items - item_base, 65535), own_splits ? 1 : n_split);
 #define FL_DEC(HDP_)                                                                                  \
     attn_decode_kernel<HDP_><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, part_ml, c,       \
                                                        (const int4*)items, block_table, max_blocks, nh, scale,   \
-                                                       window, n_split, q_tiles, ps_shift)
-    switch (hdp) {
-        case 32: FL_DEC(32); break;
-        case 64: FL_DEC(64); break;
-        case 96: FL_DEC(96); break;
-        case 128: FL_DEC(128); break;
-        case 160: FL_DEC(160); break;
-        case 192: FL_DEC(192); break;
-        case 224: FL_DEC(224); break;
-        default: FL_DEC(256); break;
-    }
+                                                       window, n_split, q_tiles, ps_shift, item_base)
+        switch (hdp) {
+            case 32: FL_DEC(32); break;
+            case 64: FL_DEC(64); break;
+            case 96: FL_DEC(96); break;
+            case 128: FL_DEC(128); break;
+            case 160: FL_DEC(160); break;
+            case 192: FL_DEC(192); break;
+            case 224: FL_DEC(224); break;
+            default: FL_DEC(256); break;
+        }
 #undef FL_DEC
-    FL_LAUNCH_CHECK();
+        FL_LAUNCH_CHECK();
+    }
     if (own_splits) {
         if (firsts && n_rows > 0) {              // (without: the caller knows that no row has more than one split)
             FL_CHECK((uintptr_t)firsts % 16 == 0, "%s: the rows' first items must be 16-byte aligned", who);

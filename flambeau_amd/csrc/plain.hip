@@ -288,6 +288,30 @@ __global__ __launch_bounds__(64) void rope_table_kernel(const int* __restrict__ 
     }
 }
 
+// The same from a ladder of frequencies of the caller's own (inv_freq[rot / 2], double): cs[token][i] =
+// magnitude * (cos, sin)(position * inv_freq[i]).  Scaled and interpolated ladders are such tables.
+__global__ __launch_bounds__(64) void rope_table_ladder_kernel(const int* __restrict__ positions, int rot,
+                                                               const double* __restrict__ inv_freq, float magnitude,
+                                                               float2* __restrict__ cs) {
+    const int token = blockIdx.x, half = rot >> 1;
+    const double pos = (double)positions[token];
+    for (int i = threadIdx.x; i < half; i += 64) {
+        const double angle = pos * inv_freq[i];
+        cs[(size_t)token * half + i] = make_float2((float)(magnitude * cos(angle)), (float)(magnitude * sin(angle)));
+    }
+}
+
+extern "C" int fl_rope_table_ladder(const int* positions, int n, int rot, const double* inv_freq, float magnitude,
+                                    float* cs, hipStream_t stream) {
+    FL_CHECK(n >= 0 && rot > 0 && rot % 2 == 0 && inv_freq, "rope_table_ladder: %d rotated dims", rot);
+    FL_CHECK((uintptr_t)cs % 8 == 0 && (uintptr_t)inv_freq % 8 == 0, "rope_table_ladder: the tables must be 8-byte aligned");
+    if (n == 0) return 0;
+    rope_table_ladder_kernel<<<n, 64, 0, stream>>>(positions, rot, inv_freq, magnitude, (float2*)cs);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_rope_table_ladder)
+
 extern "C" int fl_rope_table(const int* positions, int n, int rot, float theta, float* cs, hipStream_t stream) {
     FL_CHECK(n >= 0 && rot > 0 && rot % 2 == 0, "rope_table: %d rotated dims", rot);
     FL_CHECK((uintptr_t)cs % 8 == 0, "rope_table: the table must be 8-byte aligned");

@@ -36,6 +36,16 @@ class Runtime:
         self._views: dict = {}
         self._scope = ""
         self.generation = 0          # counts allocations of buffers: recorded launches name buffers by address
+        self._kernel_sets: dict = {}
+
+    def kernels(self, name: str):
+        """The kernel set ``name`` in the form this runtime runs (``kernels/sets.py``): what a kind of
+        part needs beyond matrix products.  The runtime knows no set by name; parts register theirs."""
+        ks = self._kernel_sets.get(name)
+        if ks is None:
+            from ..kernels.sets import make_kernel_set
+            ks = self._kernel_sets[name] = make_kernel_set(name, self)
+        return ks
 
     # ------------------------------------------------------------ buffers
     def buffer(self, name: str, rows: int, cols: int, dtype=None, max_rows: int | None = None):
@@ -109,17 +119,6 @@ class Runtime:
             return tuned.gemm(x, w, out, rt=self)
         return ops.gemm_plain(x, w.rowmajor, out)
 
-    def gemm_rope_store(self, x, w, step, table, angles, q_out, kv, n_heads: int, rotated_dims: int, writes: bool) -> bool:
-        """The joined q/k/v projection fused with rotation and the stores of q (into ``q_out``) and of
-        the cache rows (into ``kv`` where ``writes``); the rows of ``w`` lie in ``rotary_row_order``,
-        ``angles`` are the step's cosines and sines.  ``False`` if no kernel takes the shape: the
-        caller then runs product and rotation apart."""
-        if not self.tuned:
-            return False
-        from ..kernels import tuned
-        store = tuned.RopeStore(step.positions, step.tok_seq, table, angles, q_out, kv, n_heads, rotated_dims, writes)
-        return tuned.gemm_rope_store(x, w, store, rt=self)
-
     def gemm_add_norm(self, x, w, resid, norm_weight, eps: float):
         """``resid += x @ w.T`` with the norm that follows left in factors, where a kernel does both
         (``kernels.tuned.gemm_add_norm``); ``None`` if none does: the caller adds and norms itself."""
@@ -127,39 +126,6 @@ class Runtime:
             return None
         from ..kernels import tuned
         return tuned.gemm_add_norm(self, x, w, resid, norm_weight, eps)
-
-    def rotary_row_order(self, n_heads: int, n_kv_heads: int, head_dim: int, rotated_dims: int):
-        """The order in which the rows of a joined q/k/v matrix have to lie for ``gemm_rope_store``
-        (a permutation), or ``None`` where the kernels of this runtime read them as they are."""
-        if not self.tuned or not rotated_dims:
-            return None
-        from ..kernels.packing import rotary_paired_rows
-        return rotary_paired_rows(n_heads, n_kv_heads, head_dim, rotated_dims)
-
-    def attention(self, q, out, kv, step, table, n_heads: int, scale: float, window: int):
-        """Grouped-query attention of the step's rows over the paged cache."""
-        if self.tuned:
-            from ..kernels import tuned
-            return tuned.attention(self, q, out, kv, step, table, n_heads, scale, window)
-        return ops.attn_plain(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window)
-
-    def attention_metadata(self, batch, mixers):
-        """The attention kernels' work lists for a batch (integer arrays for the step's upload): the
-        rows and tiles, and for the tuned single-row kernel the rows with splits of their own, one
-        list per shape (blocks per row, window) among ``mixers``."""
-        from ..kernels import tuned
-        shapes = ()
-        if self.tuned:
-            shapes = sorted({(tuned.decode_blocks_per_row(m.n_heads, m.n_kv_heads), m.window or 0) for m in mixers})
-        return tuned.attention_metadata(batch, shapes)
-
-    def attention_splits(self, batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int):
-        """What the attention kernels of this runtime decide from the contexts' lengths (part of a
-        recorded step's key); nothing for the plain kernels."""
-        if not self.tuned:
-            return ()
-        from ..kernels import tuned
-        return tuned.attention_splits(batch, n_heads, n_kv_heads, head_dim, window)
 
     def gemm_swiglu(self, x, w, out):
         """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``.  The tuned

@@ -22,6 +22,7 @@ _SIGNATURES = {
     "fl_gemm_plain": [P, P, P, I, I, I, I, I, P],
     "fl_rope_kv_write": [P, I, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, P, I, I, L, P],
     "fl_rope_table": [P, I, I, F, P, P],
+    "fl_rope_table_ladder": [P, I, I, P, F, P, P],
     "fl_attn_plain": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
     "fl_silu_mul": [P, I, P, I, I, I, P],
     "fl_feed_tokens": [P, P, P, I, P],

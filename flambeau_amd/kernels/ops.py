@@ -140,6 +140,16 @@ def rope_table(positions, rotated_dims, theta, out):
     return out
 
 
+def rope_table_ladder(positions, rotated_dims, inv_freq, out, magnitude: float = 1.0):
+    """``rope_table`` from frequencies of the caller's own: ``out[n, rotated_dims / 2, 2]`` = ``magnitude`` *
+    (cos, sin)(position * inv_freq[i]); ``inv_freq``: float64 ``[rotated_dims / 2]`` on the device."""
+    n = positions.shape[0]
+    call("fl_rope_table_ladder", _check(positions, "rope.positions", torch.int32, (n,)), n, int(rotated_dims),
+         _check(inv_freq, "rope.inv_freq", torch.float64, (rotated_dims // 2,)), float(magnitude),
+         _check(out, "rope.table", torch.float32, (n, rotated_dims // 2, 2)), stream_handle())
+    return out
+
+
 def rope_kv_write(qkv, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads,
                   rotated_dims, theta, write_cache=True, table=None, paired=False, parts: int = 1):
     """Rotate q and k, store q and the cache rows.  ``table``: the step's ``rope_table`` (else the

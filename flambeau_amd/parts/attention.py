@@ -18,6 +18,7 @@ import torch
 
 from ..config.base import ConfigError
 from ..kernels import ops
+from ..kernels import paged_attention  # noqa: F401  (registers this mixer's kernel set)
 from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, Product, TensorSpec
 
 
@@ -55,7 +56,7 @@ class PagedGQAAttention(Mixer):
     def step_signature(self, batch):
         """Into how many parts the kernels split the keys: all that this mixer decides from the
         contexts' lengths."""
-        return self.rt.attention_splits(batch, self.n_heads, self.n_kv_heads, self.head_dim, self.window)
+        return self.kernels.signature(batch, self.n_heads, self.n_kv_heads, self.head_dim, self.window)
 
     def tensors(self):
         H, qw, kvw = self.hidden_size, self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
@@ -63,22 +64,19 @@ class PagedGQAAttention(Mixer):
                 "v.weight": TensorSpec((kvw, H)), "o.weight": TensorSpec((H, qw))}
 
     @classmethod
-    def step_metadata(cls, batch):
-        from ..kernels import tuned
-        return tuned.attention_metadata(batch)
-
-    @classmethod
     def step_metadata_for(cls, batch, mixers):
-        return mixers[0].rt.attention_metadata(batch, mixers) if mixers else cls.step_metadata(batch)
+        """The work lists the attention kernels of the mixers' runtime want for the batch."""
+        return mixers[0].kernels.metadata(batch, mixers) if mixers else {}
 
     def bind(self, weights, rt):
         self.rt = rt
+        self.kernels = rt.kernels("paged_attention")
         w_qkv = torch.cat([weights["q.weight"], weights["k.weight"], weights["v.weight"]], dim=0)
         # Where the runtime's kernels want it, the rows of a rotated projection are put in an order in which the
         # product's own kernel can rotate (8 dims, their 8 partners, ...); the rotation kernel reads
         # that order too.
         rotary = self.position.rotary_parameters()
-        order = rt.rotary_row_order(self.n_heads, self.n_kv_heads, self.head_dim, rotary[0]) if rotary is not None else None
+        order = self.kernels.row_order(self.n_heads, self.n_kv_heads, self.head_dim, rotary[0]) if rotary is not None else None
         self.paired = order is not None
         if self.paired:
             w_qkv = w_qkv[order.to(w_qkv.device)]
@@ -95,7 +93,7 @@ class PagedGQAAttention(Mixer):
         q = rt.buffer("attn_q", n, nh * hd)
         fused = False
         if self.paired and angles is not None:
-            fused = rt.gemm_rope_store(x, self.w_qkv, step, table, angles, q, cache.kv, nh, rotary[0], cache.writes)
+            fused = self.kernels.project_rotate_store(x, self.w_qkv, step, table, angles, q, cache.kv, nh, rotary[0], cache.writes)
         if not fused:
             qkv = rt.buffer("attn_qkv", n, (nh + 2 * nkv) * hd, torch.float32)
             rt.gemm(x, self.w_qkv, qkv)
@@ -105,5 +103,5 @@ class PagedGQAAttention(Mixer):
             ops.rope_kv_write(qkv, step.positions, step.tok_seq, table, q, cache.kv, nh, rotary[0], rotary[1],
                               write_cache=cache.writes, table=angles, paired=self.paired)
         out = rt.buffer("attn_out", n, nh * hd)
-        rt.attention(q, out, cache.kv, step, table, nh, self.scale, self.window)
+        self.kernels.attention(q, out, cache.kv, step, table, nh, self.scale, self.window)
         return Product(out, self.w_o)

@@ -33,9 +33,14 @@ class PartSpec:
 @dataclass(frozen=True)
 class TensorSpec:
     """A tensor a part needs.  ``role``: ``matrix``/``table`` are stored in the compute
-    dtype; ``vector32`` (norm gains) is always held in float32; ``int32`` integer tables."""
+    dtype; ``vector32`` (norm gains, biases, decay rates) is always held in float32; ``int32`` integer
+    tables.  ``init`` says what random weights give it: ``None`` = by role (matrices and tables
+    N(0, std^2), vectors a gain 1 + N(0, gain_std^2)); ``"normal"``, ``"gain"``, ``"zeros"``,
+    ``"ones"``; or a function ``(generator, shape, device) -> float32 tensor`` (a part whose vector is
+    a bias or the logarithm of a decay says so here)."""
     shape: tuple
     role: str = "matrix"
+    init: object = None
 
 
 class CacheSpec:

@@ -27,16 +27,40 @@ class RotaryNeoX(PositionEncoding):
     def rotary_parameters(self):
         return self.rotated_dims, self.theta
 
+    def inverse_frequencies(self):
+        """``None``: the ladder ``theta^(-2 i / rotated_dims)``.  A subclass with another ladder (scaled,
+        interpolated, cut) returns its ``rotated_dims / 2`` frequencies (floats, made in double) and
+        may set ``magnitude``, a factor on every cosine and sine; everything else stays: the table is
+        made from them, and the kernels that rotate read the table."""
+        return None
+
+    magnitude = 1.0
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        freqs = self.inverse_frequencies()
+        self._ladder = None
+        if freqs is not None:
+            if len(freqs) != self.rotated_dims // 2:
+                raise ValueError(f"{len(freqs)} frequencies for {self.rotated_dims} rotated dims")
+            self._ladder = torch.tensor([float(f) for f in freqs], dtype=torch.float64, device=rt.device)
+            self._ladder_key = tuple(float(f) for f in freqs)
+
     def rotary_table(self, rt, step):
         """The angles depend on the positions only: their cosines and sines are made once per
         forward pass and shared by all layers with the same constants."""
-        key = ("rope_neox", self.rotated_dims, self.theta)
+        ladder = getattr(self, "_ladder", None)
+        key = ("rope_neox", self.rotated_dims, self.theta if ladder is None else self._ladder_key, self.magnitude)
         table = step.scratch.get(key)
         if table is None:
             half = self.rotated_dims // 2
-            table = rt.buffer(f"rope_table_{self.rotated_dims}_{self.theta}", step.n_tokens, 2 * half, torch.float32)
+            name = f"rope_table_{self.rotated_dims}_{self.theta}" if ladder is None else f"rope_table_{hash(key)}"
+            table = rt.buffer(name, step.n_tokens, 2 * half, torch.float32)
             table = table.view(step.n_tokens, half, 2)
-            ops.rope_table(step.positions, self.rotated_dims, self.theta, table)
+            if ladder is None:
+                ops.rope_table(step.positions, self.rotated_dims, self.theta, table)
+            else:
+                ops.rope_table_ladder(step.positions, self.rotated_dims, ladder, table, self.magnitude)
             step.scratch[key] = table
         return table
 

@@ -1,6 +1,8 @@
 """Seeded random weights: as a tensor source, and written out as a model folder.
 
-Matrices and tables are i.i.d. N(0, std^2); norm gains are 1 + N(0, gain_std^2).  Each tensor
+Matrices and tables are i.i.d. N(0, std^2); norm gains are 1 + N(0, gain_std^2); a part may say
+otherwise for a tensor of its own (``TensorSpec.init``: zeros, ones, a bias drawn like a matrix, a
+function).  Each tensor
 has a generator of its own, seeded from (seed, tensor name), so a tensor's values do not
 depend on which others are made.  The reference has no random weights; its tests use a
 deterministic signal instead (crates/forward/tests/common/mod.rs:80-86).
@@ -39,19 +41,33 @@ class RandomSource:
         return list(self.manifest)
 
     def info(self, name):
-        return tuple(self.manifest[name][2].shape), _TAGS[self.store_dtype]
+        tspec = self.manifest[name][2]
+        return tuple(tspec.shape), ("I32" if tspec.role == "int32" else _TAGS[self.store_dtype])
 
     def read(self, name):
         tspec = self.manifest[name][2]
         g = torch.Generator(device=self.device)
         g.manual_seed(_tensor_seed(self.seed, name))
+        init = getattr(tspec, "init", None)
+        shape = tuple(tspec.shape)
+        if callable(init):
+            x = init(g, shape, self.device)
+            if tuple(x.shape) != shape:
+                raise ValueError(f"random weights: the rule of '{name}' made {tuple(x.shape)}, the tensor is {shape}")
+            return x.to(torch.int32 if tspec.role == "int32" else self.store_dtype)
         if tspec.role == "int32":
-            raise ValueError(f"random weights: no rule for the integer table '{name}'")
-        x = torch.randn(tuple(tspec.shape), generator=g, device=self.device, dtype=torch.float32)
-        if tspec.role == "vector32":
-            x = 1.0 + x * self.gain_std
+            raise ValueError(f"random weights: no rule for the integer table '{name}' (give its TensorSpec an init function)")
+        if init is None:
+            init = "gain" if tspec.role == "vector32" else "normal"
+        if init == "zeros":
+            x = torch.zeros(shape, device=self.device, dtype=torch.float32)
+        elif init == "ones":
+            x = torch.ones(shape, device=self.device, dtype=torch.float32)
+        elif init in ("normal", "gain"):
+            x = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32)
+            x = 1.0 + x * self.gain_std if init == "gain" else x * self.std
         else:
-            x = x * self.std
+            raise ValueError(f"random weights: unknown init '{init}' for '{name}'")
         return x.to(self.store_dtype)
 
 
@@ -71,7 +87,8 @@ def write_random_model(config: dict, out_dir, seed: int, std: float = 0.02, gain
     cfg_out["torch_dtype"] = {torch.float32: "float32", torch.bfloat16: "bfloat16",
                               torch.float16: "float16"}[store_dtype]
     (out / "config.json").write_text(json.dumps(cfg_out, indent=2) + "\n")
-    items = [(name, tuple(spec[2].shape), store_dtype, (lambda n=name: src.read(n))) for name, spec in manifest.items()]
+    items = [(name, tuple(spec[2].shape), torch.int32 if spec[2].role == "int32" else store_dtype, (lambda n=name: src.read(n)))
+             for name, spec in manifest.items()]
     write_safetensors(out / "model.safetensors", items,
                       metadata={"format": "pt", "seed": seed, "std": std, "gain_std": gain_std})
     return out

@@ -646,6 +646,37 @@ def test_attn_decode_subset_of_rows_leaves_the_others_alone():
     assert (out[[1, 4]].double().reshape(2, nh, hd) - ref[[1, 4]]).abs().max() < 1e-2 * ref.abs().max()
 
 
+def test_attn_decode_takes_more_items_than_a_grid_has_places():
+    """70,000 single rows in one call (the grid's slow index holds 65,535): all of them are computed,
+    in the uniform form with two splits and with a list of items."""
+    nh, nkv, hd, ps, n = 2, 1, 16, 8, 70000
+    case = build_attention_case(torch.bfloat16, nh, nkv, hd, ps, [(40, 1), (23, 1)], seed=2)
+    q = (torch.randn(n, nh, hd, generator=torch.Generator().manual_seed(3)) * 0.8).to(torch.bfloat16).to(DEV)
+    req = torch.arange(n, device=DEV) % 2
+    pos = torch.where(req == 0, torch.arange(n, device=DEV) % 40, torch.arange(n, device=DEV) % 23)
+    rows = torch.stack([torch.arange(n, device=DEV), pos, req, torch.zeros_like(req)], 1).int().contiguous()
+    # the reference, all rows at once: scores against every key of the row's request, masked beyond its position
+    ref = torch.zeros(n, nh, hd, dtype=torch.float64, device=DEV)
+    for r in range(2):
+        sel = (req == r).nonzero().squeeze(1)
+        K, V = case["K"][r][:, 0], case["V"][r][:, 0]
+        s = torch.einsum("nhd,td->nht", q[sel].double(), K) * 0.25
+        s = s.masked_fill(torch.arange(K.shape[0], device=DEV)[None, None, :] > pos[sel][:, None, None], float("-inf"))
+        ref[sel] = torch.einsum("nht,td->nhd", torch.softmax(s, -1), V)
+    hdp = 32
+    for n_split in (2, 0):
+        out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        items = rows.clone()
+        k = max(n_split, 1)
+        if n_split == 0:
+            items[:, 3] = 256
+        part_o = torch.empty(n * nh * k * hdp, dtype=torch.float32, device=DEV)
+        part_ml = torch.empty(n * nh * k * 2, dtype=torch.float32, device=DEV)
+        tuned().attn_decode(q.reshape(n, nh * hd), out, case["cache"], items, case["table"], nh, 0.25, 0, n_split, part_o, part_ml)
+        err = (out.double().reshape(n, nh, hd) - ref).abs().amax((1, 2))
+        assert not torch.isnan(out).any() and err.max() < 1e-2 * ref.abs().max(), int(err.argmax())
+
+
 # ---------------------------------------------------------------- tiled matrix product
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (65, 100, 72), (300, 250, 40), (2048, 512, 256), (129, 37, 264),

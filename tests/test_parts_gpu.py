@@ -158,6 +158,58 @@ def test_attention_mixer_part(dtype, tuned, nh, nkv, hd, window, theta, ps):
         assert np.abs(got - want).max() < tol(dtype) * np.abs(want).max(), cuts
 
 
+@pytest.mark.parametrize("tuned", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_rotation_with_a_ladder_of_its_own(dtype, tuned):
+    """A toy position encoding defined here: the built-in split-half rotation with other frequencies
+    (every rung slowed down by a factor of its own) and a magnitude on cosines and sines.  It only
+    overrides ``inverse_frequencies``; the table, the fused rotate-and-store kernels and the rotation
+    kernel serve it as they serve the built-in ladder, in every cutting."""
+    from flambeau_amd.cache.storage import CacheStorage
+    from flambeau_amd.parts import MIXERS, POSITION_ENCODINGS, PartSpec
+    from flambeau_amd.parts.rope import RotaryNeoX
+    if "toy_slowed_ladder" not in POSITION_ENCODINGS.known():
+        @POSITION_ENCODINGS.register("toy_slowed_ladder")
+        class Slowed(RotaryNeoX):
+            magnitude = 1.25
+
+            def inverse_frequencies(self):
+                half = self.rotated_dims // 2
+                return [self.theta ** (-2.0 * i / self.rotated_dims) / (1.0 + 0.5 * i) for i in range(half)]
+    rt = make_rt(dtype, tuned)
+    H, n, nh, nkv, hd, theta, ps, window = 56, 75, 4, 2, 32, 1e4, 8, 50
+    mixer = MIXERS.create(PartSpec("paged_gqa_attention", dict(hidden_size=H, n_heads=nh, n_kv_heads=nkv, head_dim=hd, window=window,
+                                                            position=PartSpec("toy_slowed_ladder", dict(head_dim=hd, theta=theta)))))
+    w = _mixer_weights(mixer, dtype)
+    mixer.bind({k: put(rt, v) for k, v in w.items()}, rt)
+    x = rnd(n, H, seed=7).to(dtype)
+    W = {k: v.double().numpy() for k, v in w.items()}
+    xs = x.double().numpy()
+
+    def rotate(t):                                   # t [n, heads, hd]: the toy's formula, written out
+        half = hd // 2
+        freqs = np.array([theta ** (-2.0 * i / hd) / (1.0 + 0.5 * i) for i in range(half)])
+        ang = np.arange(n)[:, None] * freqs[None, :]
+        c, s_ = 1.25 * np.cos(ang)[:, None, :], 1.25 * np.sin(ang)[:, None, :]
+        lo, hi = t[:, :, :half], t[:, :, half:]
+        return np.concatenate([lo * c - hi * s_, lo * s_ + hi * c], axis=2)
+    q = rotate(pm.linear(xs, W["q.weight"]).reshape(n, nh, hd))
+    k = rotate(pm.linear(xs, W["k.weight"]).reshape(n, nkv, hd))
+    v = pm.linear(xs, W["v.weight"]).reshape(n, nkv, hd)
+    want = pm.linear(pm.attention(q, k, v, np.arange(n), pm.default_scale(hd), window).reshape(n, nh * hd), W["o.weight"])
+    plain_ladder = pm.attention_mixer(xs, {"a." + k_.replace(".weight", "_proj.weight"): v_ for k_, v_ in W.items()}, "a.",
+                                      np.arange(n), nh, nkv, hd, theta, window)
+    assert np.abs(want - plain_ladder).max() > 0.05 * np.abs(want).max()          # the toy is not the built-in ladder
+    for cuts in ([n], [40, 5, 1, 1, 20, 2, 6]):
+        store = CacheStorage([mixer.cache_spec()], [None], rt.device, dtype, n_pages=32, page_size=ps, max_slots=2)
+        got, at = [], 0
+        for c in cuts:
+            step = step_for(rt, [(at, c)], ps, 32, shuffle_seed=1)
+            got.append(delta_of(rt, mixer.forward(x[at:at + c].to(DEV).contiguous(), step, store.entries[0])).double().cpu().numpy())
+            at += c
+        assert np.abs(np.concatenate(got) - want).max() < tol(dtype) * np.abs(want).max(), cuts
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_prenorm_block_part(dtype):
     from flambeau_amd.cache.storage import CacheStorage

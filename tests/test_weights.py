@@ -156,3 +156,35 @@ def test_sharded_folder(tmp_path):
     check_against_manifest(_manifest("A"), src)
     for n in names:
         assert torch.equal(src.read(n), whole[n])
+
+
+def test_random_weights_follow_what_a_tensor_says_of_itself():
+    """By role a vector is a gain (1 + noise) and a matrix noise; a part whose vector is a bias, a
+    decay rate or an integer table says so in its TensorSpec, and the defaults' values stay what they were."""
+    import torch
+    from flambeau_amd.parts import TensorSpec
+    from flambeau_amd.weights.random_init import RandomSource
+
+    def decay(generator, shape, device):
+        return -torch.rand(shape, generator=generator, device=device) - 0.5
+
+    def table(generator, shape, device):
+        return torch.randint(0, 7, shape, generator=generator, device=device)
+    manifest = {"gain": (0, "g", TensorSpec((64,), "vector32")), "matrix": (0, "m", TensorSpec((8, 16))),
+                "bias": (0, "b", TensorSpec((64,), "vector32", init="normal")), "zero": (0, "z", TensorSpec((5,), "vector32", init="zeros")),
+                "one": (0, "o", TensorSpec((5, 2), init="ones")), "decay": (0, "d", TensorSpec((32,), "vector32", init=decay)),
+                "ids": (0, "i", TensorSpec((9,), "int32", init=table)), "bad": (0, "x", TensorSpec((3,), "int32"))}
+    src = RandomSource(manifest, seed=4, std=0.05, gain_std=0.01, store_dtype=torch.float32)
+    gain, bias = src.read("gain"), src.read("bias")
+    assert abs(float(gain.mean()) - 1) < 0.01 and float(gain.std()) < 0.03
+    assert abs(float(bias.mean())) < 0.03 and 0.02 < float(bias.std()) < 0.08
+    assert float(src.read("zero").abs().max()) == 0 and torch.equal(src.read("one"), torch.ones(5, 2))
+    d = src.read("decay")
+    assert float(d.max()) <= -0.5 and float(d.min()) >= -1.5
+    ids = src.read("ids")
+    assert ids.dtype == torch.int32 and src.info("ids") == ((9,), "I32") and 0 <= int(ids.min()) and int(ids.max()) < 7
+    with pytest.raises(ValueError, match="no rule for the integer table"):
+        src.read("bad")
+    # a tensor's values depend on the seed and its name alone
+    again = RandomSource({"matrix": manifest["matrix"]}, seed=4, std=0.05, gain_std=0.5, store_dtype=torch.float32)
+    assert torch.equal(again.read("matrix"), src.read("matrix"))
