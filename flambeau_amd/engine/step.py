@@ -362,11 +362,14 @@ class ModelRunner:
         is captured, and replayed; a step leaves the same cache however often it runs."""
         bk = self._bucket(len(entries))
         batch, parts = self._assemble(entries, pad_to=bk)
-        gs = self._graphs.get(bk)
+        # one graph per bucket and per thing the mixers decide from the contexts (whether a kernel that
+        # merges splits of the keys runs at all, for one); the graphs of a bucket share their buffers
+        key = (bk, self.model.step_signature(batch))
+        gs = self._graphs.get(key)
         if gs is None:
             _, total = self._layout(parts)
             gs = _GraphedStep(torch.empty(max(total, 1), dtype=torch.int32, device=self.rt.device))
-            self._graphs[bk] = gs
+            self._graphs[key] = gs
         dev = self._upload(parts, gs.meta)
         feedback = self.token_feedback is not None
         if gs.graph is None:

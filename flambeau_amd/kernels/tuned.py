@@ -521,7 +521,10 @@ def attention_metadata(batch, shapes=()) -> dict:
     rows = np.asarray(rows, dtype=np.int32).reshape(-1, 4)
     out = {"attn_rows": rows, "attn_tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 4)}
     for per_row, window in shapes:
-        out[f"attn_items/{per_row}/{window}"], out[f"attn_item_rows/{per_row}/{window}"] = balanced_items(rows, per_row, window)
+        items, firsts = balanced_items(rows, per_row, window)
+        out[f"attn_items/{per_row}/{window}"], out[f"attn_item_rows/{per_row}/{window}"] = items, firsts
+        # whether any row is split at all decides if the kernel that merges runs: a part of the step's signature
+        batch.notes[("attn_rows_split", per_row, window)] = bool(firsts.shape[0] and int(firsts[:, 2].max()) > 1)
     return out
 
 
@@ -556,31 +559,47 @@ def balanced_items(rows, blocks_per_row: int, window: int = 0, budget: int | Non
     if window:
         keys = np.minimum(keys, window)
     most = np.minimum(-(-keys // DECODE_MIN_KEYS_PER_SPLIT), DECODE_MAX_SPLITS)
-    # How many places to use.  Rows of about one length: a block per unit is enough (measured at 16 to 64
-    # rows of 2,100 keys: 256 blocks, or one per row and kv head if that is more, beat 512 and 1,024; up
-    # to 8 rows, two per unit were 1 % of a 7B decode step faster).  A ragged batch: all places, since
-    # many short blocks spread over the units as they finish (55 rows of 128 to 4,600 keys: 136 us with
-    # a place per row, 100 with two, 94 with four per row).
-    ragged = int(keys.max()) * n > 1.5 * int(keys.sum())
-    even_blocks = DECODE_TARGET_BLOCKS if n * blocks_per_row <= DECODE_TARGET_BLOCKS // 8 else DECODE_EVEN_BLOCKS
-    use = budget if ragged else min(budget, max(n, even_blocks // max(1, blocks_per_row)))
-    splits = np.clip(keys * use // max(int(keys.sum()), 1), 1, most)
-    # what rounding down and the caps left over goes to the rows whose splits are longest; what the
-    # least of one split per row took too much comes from the rows whose splits are shortest
-    left = use - int(splits.sum())
-    while left > 0:
-        room = splits < most
-        if not room.any():
-            break
-        take = np.argsort(-np.where(room, keys / splits, 0.0), kind="stable")[:left]
-        take = take[room[take]]
-        splits[take] += 1
-        left -= take.size
-    while left < 0:
-        give = np.argsort(np.where(splits > 1, keys / splits, np.inf), kind="stable")[:-left]
-        give = give[splits[give] > 1]
-        splits[give] -= 1
-        left += give.size
+    # Rows that cannot be split anyway (a split holds 128 keys at least: the rows that pad a batch of
+    # fixed shape, requests that have just begun) take a place each and have no say in what follows.
+    big = most > 1
+    n_big, n_small = int(big.sum()), int(n - big.sum())
+    splits = np.ones(n, dtype=np.int64)
+    if n_big:
+        kb, mb = keys[big], most[big]
+        # How many places to use.  Rows of about one length: a block per unit is enough (measured at 16 to 64
+        # rows of 2,100 keys: 256 blocks, or one per row and kv head if that is more, beat 512 and 1,024; up
+        # to 8 rows, two per unit were 1 % of a 7B decode step faster), and every row gets the same number of
+        # splits (a row with one split beside rows with two ends the kernel alone).  A ragged batch: all
+        # places, since many short blocks spread over the units as they finish (55 rows of 128 to 4,600
+        # keys: 136 us with a place per row, 100 with two, 94 with four per row).
+        room = budget - n_small
+        ragged = int(kb.max()) * n_big > 1.5 * int(kb.sum())
+        if ragged:
+            use = room
+        else:
+            even_blocks = DECODE_TARGET_BLOCKS if n_big * blocks_per_row <= DECODE_TARGET_BLOCKS // 8 else DECODE_EVEN_BLOCKS
+            each = max(1, -(-even_blocks // (n_big * max(1, blocks_per_row))))
+            while each > 1 and n_big * each > room:
+                each -= 1
+            use = n_big * each
+        sb = np.clip(kb * use // max(int(kb.sum()), 1), 1, mb)
+        # what rounding down and the caps left over goes to the rows whose splits are longest; what the
+        # least of one split per row took too much comes from the rows whose splits are shortest
+        left = use - int(sb.sum())
+        while left > 0:
+            free = sb < mb
+            if not free.any():
+                break
+            take = np.argsort(-np.where(free, kb / sb, 0.0), kind="stable")[:left]
+            take = take[free[take]]
+            sb[take] += 1
+            left -= take.size
+        while left < 0:
+            give = np.argsort(np.where(sb > 1, kb / sb, np.inf), kind="stable")[:-left]
+            give = give[sb[give] > 1]
+            sb[give] -= 1
+            left += give.size
+        splits[big] = sb
     first = np.concatenate(([0], np.cumsum(splits)[:-1]))
     which = np.repeat(np.arange(n), splits)
     total = int(splits.sum())
@@ -683,7 +702,8 @@ def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window
     """``(parts of the keys for the tiled kernel, for the single-row kernel)`` for a batch: everything
     that ``attention`` decides from the contexts' lengths (the rest follows from the batch's shape).
     ``with_items``: the single rows come with splits of their own (``balanced_items``), which are
-    data of the step and decide nothing here (0 stands for that)."""
+    data of the step; all they decide here is whether any row is split at all (0 if so: the kernel
+    that merges runs; -1 if not: it is left out)."""
     n_tiles = sum(-(-ql // PREFILL_TILE) for ql in batch.q_lens if ql > SHORT_PORTION)
     n_items = sum(ql for ql in batch.q_lens if ql <= SHORT_PORTION)
     p_split = n_split = 1
@@ -696,7 +716,10 @@ def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window
         if window:
             max_ctx = min(max_ctx, window + 32)
         n_split = decode_splits(n_items, n_kv_heads, n_heads // n_kv_heads, max_ctx)
-    return p_split, (0 if n_items and with_items else n_split)
+    if n_items and with_items:
+        split = batch.notes.get(("attn_rows_split", decode_blocks_per_row(n_heads, n_kv_heads), window or 0), True)
+        return p_split, (0 if split else -1)
+    return p_split, n_split
 
 
 def attention(rt, q, out, cache, step, table, n_heads, scale, window):
@@ -726,8 +749,8 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
         # rows with splits of their own; the list's length follows from the number of rows alone
         # (a list with a place per row and no more: no row is ever split, nothing to merge)
         firsts = step.extra.get(f"attn_item_rows/{decode_blocks_per_row(n_heads, cache.n_kv_heads)}/{window or 0}")
-        if items.shape[0] <= rows.shape[0]:
-            firsts = None
+        if items.shape[0] <= rows.shape[0] or n_split < 0:
+            firsts = None                    # no row is split: every block writes its row itself
         part_o = part_ml = None
         if firsts is not None:
             hdp = -(-cache.head_dim // 32) * 32

@@ -158,6 +158,7 @@ class HostBatch:
     n_logit_rows: int
     ctx_bound: int | None = None   # set for a fixed-shape batch (graph replay): longest context it may ever hold
     every_row: bool = False        # the wanted rows are exactly rows 0 .. n_tokens - 1, in that order
+    notes: dict = field(default_factory=dict)   # what parts found out about the batch while they laid out its metadata (``step_metadata``) and want to find again in ``step_signature`` or ``forward``
 
     @property
     def n_seqs(self): return len(self.q_lens)

@@ -435,12 +435,45 @@ def test_captured_decode_steps_equal_eager_ones(model_dirs, dtype):
         steps.append(dict(entries=[dict(id="r1", tokens=[reqs["r1"][41]], want=[0])], end=["r1", "r2"]))
         results.append(rh.run_in_process(runner, steps))
         if graphs:
-            assert sorted(runner._graphs) == [1, 2, 4]
+            assert sorted({bucket for bucket, _ in runner._graphs}) == [1, 2, 4]
     eager, graphed = results
     assert eager.keys() == graphed.keys() and len(eager) > 30
     for k in eager:
         assert np.array_equal(eager[k], graphed[k]), k
     rh.compare(graphed, reqs, rh.plain_logits(d, reqs), dtype, "captured steps")
+
+
+def test_a_bucket_has_a_graph_for_each_thing_the_mixers_decide(model_dirs):
+    """While no row's keys are split the kernel that merges splits is left out of the step; when a
+    context grows beyond what one split holds the same bucket gets a second graph with it.  Both give
+    the eager step's logits, before and after the change, and the plain implementation's."""
+    d = model_dirs[("B", "bfloat16")]
+    reqs = rh.make_requests(384, [230, 60], seed=23)
+    from flambeau_amd.engine import ModelRunner, load_model
+    model, _ = load_model(d, dtype="bfloat16", max_batch_tokens=256)
+    steps = [dict(entries=[dict(id="r0", tokens=reqs["r0"][:90], want=[89]), dict(id="r1", tokens=reqs["r1"][:20], want=[])], end=[])]
+    for i in range(90, 230):                       # r0 passes 128 keys on the way; r1 decodes beside it for a while
+        e = [dict(id="r0", tokens=[reqs["r0"][i]], want=[0])]
+        if i - 70 < 60:
+            e.append(dict(id="r1", tokens=[reqs["r1"][i - 70]], want=[0]))
+        steps.append(dict(entries=e, end=["r1"] if i - 70 == 59 else []))
+    steps[-1]["end"] = ["r0"]
+    results = []
+    for graphs in (False, True):
+        runner = ModelRunner(model, n_pages=24, page_size=16, max_slots=2, max_logit_rows=256, decode_graphs=graphs,
+                             step_programs=False)
+        runner.storage.fill(float("nan"))
+        results.append(rh.run_in_process(runner, steps))
+        if graphs:
+            by_bucket = {}
+            for bucket, decided in runner._graphs:
+                by_bucket.setdefault(bucket, set()).add(decided)
+            assert set(by_bucket) == {1, 2} and len(by_bucket[2]) == 2, by_bucket          # (r0 is alone only once it is split)
+    eager, graphed = results
+    assert eager.keys() == graphed.keys() and len(eager) > 170
+    for k in eager:
+        assert np.array_equal(eager[k], graphed[k]), k
+    rh.compare(graphed, reqs, rh.plain_logits(d, reqs), "bfloat16", "graphs with and without the kernel that merges")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
