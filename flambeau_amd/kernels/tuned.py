@@ -540,6 +540,37 @@ def decode_item_budget(n_rows: int, blocks_per_row: int) -> int:
     return max(n_rows, min(max(DECODE_TARGET_BLOCKS // max(1, blocks_per_row), 4 * n_rows), n_rows * DECODE_MAX_SPLITS))
 
 
+# What the single-row kernel costs on this chip, measured with 8 to 64 rows of 2,100 keys at 7B head sizes:
+# a compute unit streams keys and values at about 30 GB/s whether one block or two share it, so a step
+# takes as long as the unit with the most bytes (blocks go to the 256 units in turn), a block costs 1.5 us
+# beside its bytes, the kernel that merges splits 4.7 us, and the chip as a whole gives 6.4 TB/s.
+DECODE_UNITS = 256
+DECODE_UNIT_RATE = 30e9
+DECODE_CHIP_RATE = 6.4e12
+DECODE_BLOCK_US = 1.5
+DECODE_MERGE_US = 4.7
+DECODE_KEY_BYTES = 512             # keys and values of one kv head of 128 dims in bfloat16 (the constants' reference)
+
+
+def even_splits(n_rows: int, blocks_per_row: int, keys: float, most: int) -> int:
+    """Splits per row (1 .. ``most``) for ``n_rows`` rows of about ``keys`` keys each: the number that makes
+    the unit with the most blocks finish first by the measured costs above.  17 to 32 rows of 2,100 keys:
+    one (a block per row and kv head, nothing to merge: 35 us where two splits take 42); 16 rows: two; 40: three."""
+    units = n_rows * max(1, blocks_per_row)
+    if units <= DECODE_TARGET_BLOCKS // 8:
+        # few rows: two blocks per unit (measured up to 8 rows: 1 % of a 7B decode step faster than one)
+        return max(1, min(most, DECODE_TARGET_BLOCKS // units))
+    row_us = keys * DECODE_KEY_BYTES / DECODE_UNIT_RATE * 1e6
+    chip_us = units * keys * DECODE_KEY_BYTES / DECODE_CHIP_RATE * 1e6
+    best, best_us = 1, None
+    for s in range(1, max(1, min(most, DECODE_MAX_SPLITS)) + 1):
+        per_unit = -(-units * s // DECODE_UNITS)
+        us = max(per_unit * (row_us / s + DECODE_BLOCK_US), chip_us) + (DECODE_MERGE_US if s > 1 else 0.0)
+        if best_us is None or us < best_us * 0.97:              # (more splits only where they pay)
+            best, best_us = s, us
+    return best
+
+
 def balanced_items(rows, blocks_per_row: int, window: int = 0, budget: int | None = None):
     """``rows`` (row, position, request, 0) with splits of their own: every row gets splits in
     proportion to the keys it sees (a split of 128 keys at least, 64 splits at most), so that the blocks
@@ -566,21 +597,16 @@ def balanced_items(rows, blocks_per_row: int, window: int = 0, budget: int | Non
     splits = np.ones(n, dtype=np.int64)
     if n_big:
         kb, mb = keys[big], most[big]
-        # How many places to use.  Rows of about one length: a block per unit is enough (measured at 16 to 64
-        # rows of 2,100 keys: 256 blocks, or one per row and kv head if that is more, beat 512 and 1,024; up
-        # to 8 rows, two per unit were 1 % of a 7B decode step faster), and every row gets the same number of
-        # splits (a row with one split beside rows with two ends the kernel alone).  A ragged batch: all
-        # places, since many short blocks spread over the units as they finish (55 rows of 128 to 4,600
-        # keys: 136 us with a place per row, 100 with two, 94 with four per row).
+        # How many places to use.  Rows of about one length: the same number of splits for every row (a row
+        # with one split beside rows with two ends the kernel alone), chosen by what the blocks then cost
+        # (``even_splits``).  A ragged batch: all places, since many short blocks spread over the units as
+        # they finish (55 rows of 128 to 4,600 keys: 136 us with a place per row, 100 with two, 94 with four).
         room = budget - n_small
         ragged = int(kb.max()) * n_big > 1.5 * int(kb.sum())
         if ragged:
             use = room
         else:
-            even_blocks = DECODE_TARGET_BLOCKS if n_big * blocks_per_row <= DECODE_TARGET_BLOCKS // 8 else DECODE_EVEN_BLOCKS
-            each = max(1, -(-even_blocks // (n_big * max(1, blocks_per_row))))
-            while each > 1 and n_big * each > room:
-                each -= 1
+            each = even_splits(n_big, blocks_per_row, float(kb.mean()), min(int(mb.min()), max(1, room // n_big)))
             use = n_big * each
         sb = np.clip(kb * use // max(int(kb.sum()), 1), 1, mb)
         # what rounding down and the caps left over goes to the rows whose splits are longest; what the
