@@ -174,6 +174,41 @@ def run_portion(model, dtype_name, portion, ctx_before, reps=REPS, seed=3):
     return statistics.median(times)
 
 
+def run_decode_filled(model, batch, ctx, steps=24, warmup=6, seed=4):
+    """Decode steps of ``batch`` requests that each hold ``ctx`` tokens, without running their prompts:
+    the pages are handed out and filled with random values (what attention reads costs the same), then
+    single tokens are stepped through ``ModelRunner.step`` (graph replay, no sampling).  Returns
+    (seconds per step, mean context)."""
+    import numpy as np
+    import torch
+    from flambeau_amd.engine import ModelRunner, StepEntry
+    rng = np.random.default_rng(seed)
+    V = model.spec.vocab_size
+    total = ctx + steps + warmup + 2
+    runner = ModelRunner(model, n_pages=batch * (-(-total // PAGE)) + 2, page_size=PAGE, max_slots=batch, max_seq_len=total,
+                         max_logit_rows=batch)
+    for pool in runner.storage.pools:
+        pool.normal_(0.0, 0.5)
+    for i in range(batch):
+        runner.begin(i)
+        runner.manager.ensure(i, ctx)
+        runner.manager.advance(i, ctx)
+    step = lambda: runner.step([StepEntry(i, [int(rng.integers(0, V))], [0]) for i in range(batch)])
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    for i in range(batch):
+        runner.end(i)
+    del runner
+    torch.cuda.empty_cache()
+    return dt, ctx + warmup + steps / 2.0
+
+
 def run_enqueue(model, dtype_name, rows=64, decoders=16, seed=2):
     """Host time to enqueue one mixed step of ``rows`` rows (a prompt portion beside ``decoders``
     decoding requests): the time ``ModelRunner.step`` takes to return, the device idle before and
@@ -265,6 +300,14 @@ def bench_serving(a, name, label, cfg, dtype_name, el):
     runs = [run_serving(model, cfg, dtype_name, prompts, n_new, batch, chunk, ctx) for _ in range(a.reps)]
     r = sorted(runs, key=lambda x: x["t_decode"])[len(runs) // 2]
     window = cfg["sliding_window"] or 0
+    extra_points = {}
+    if name == "24b":
+        # decode at batch 1 and 8 behind 2,048 tokens each (the cache filled with random values)
+        for b in (1, 8):
+            dtl, ctxl = run_decode_filled(model, b, PROMPT_LEN, steps=32, warmup=8)
+            extra_points[f"decode_b{b}"] = round(b / dtl, 1)
+            extra_points[f"decode_b{b}_ms"] = round(dtl * 1e3, 3)
+            extra_points[f"decode_b{b}_frac"] = round(decode_bytes(sz, b, ctxl, el) / dtl / PEAK_HBM, 4)
     # the pure decode phase: all requests that are left decode; its bytes from the mean live context
     ms = r["t_decode"] / max(r["steps_decode"], 1) * 1e3
     tok_s = r["made_decode"] / r["t_decode"]
@@ -294,7 +337,7 @@ def bench_serving(a, name, label, cfg, dtype_name, el):
                      "frac": round(achieved / PEAK_HBM, 4)},
         "prefill": {"value": round(n_prompt / r["t_prompt"], 1), "tokens": n_prompt, "ms": round(r["t_prompt"] * 1e3, 2),
                     "frac": round(flops / r["t_prompt"] / PEAK_FLOPS[a.dtype], 4)},
-        "points": {"total_s": round(r["t_prompt"] + r["t_decode"], 3),
+        "points": {**extra_points, "total_s": round(r["t_prompt"] + r["t_decode"], 3),
                    "overall_generated_tok_s": round(batch * n_new / (r["t_prompt"] + r["t_decode"]), 1),
                    "tokens_decoded_beside_prompts": r["made_prompt"], "mean_live_requests": round(live, 2),
                    "preemptions": r["preemptions"], "reps": a.reps},
@@ -390,6 +433,12 @@ def main():
             key = f"prefill512_ctx{label}"
             points[key] = round(512 / t, 1)
             points[key + "_frac"] = round(prefill_flops(sz, 512, mid) / t / PEAK_FLOPS[a.dtype], 4)
+        # decode behind long contexts (the cache filled with random values, not by running prompts)
+        for b, ctx, name in ((8, 16384, "b8_ctx16k"), (8, 32768 - 64, "b8_ctx32k"), (64, 16384, "b64_ctx16k")):
+            dtl, ctxl = run_decode_filled(model, b, ctx)
+            points[f"decode_{name}"] = round(b / dtl, 1)
+            points[f"decode_{name}_ms"] = round(dtl * 1e3, 3)
+            points[f"decode_{name}_frac"] = round(decode_bytes(sz, b, ctxl, el) / dtl / PEAK_HBM, 4)
         out["points"] = points
     print(json.dumps(out), flush=True)
     return 0
