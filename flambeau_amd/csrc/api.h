@@ -11,6 +11,7 @@ extern "C" {
 
 const char* fl_last_error(void);
 int fl_abi_version(void);
+int fl_compute_units(void);        // compute units of the current device: what the kernels' plans count blocks against
 
 // ---- plain kernels (plain.hip) ----
 int fl_embed(const void* table, int dtype, const int* tokens, float* out, int n, int H, int V,

@@ -378,22 +378,12 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     }
 }
 
-static int pf_units() {                  // compute units of the device
-    static int units = 0;
-    if (!units) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || units <= 0)
-            units = 256;
-    }
-    return units;
-}
-
 template <int HDP, int QT, int NS>
 static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                                const int* tiles, const int* positions, const int* block_table, int max_blocks,
                                int nh, float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml, int lds_pages) {
     // blocks that the chip holds at one time: one or two per compute unit
-    const int units = pf_units();
+    const int units = fl_units();
     const int total = (int)(grid.x * grid.y * grid.z);
     constexpr int RING = NS * (4 * (HDP / 32) + 2 * (HDP / 16)) * 1024;
     const int lds = RING + lds_pages * (int)sizeof(int);
@@ -437,7 +427,7 @@ static int pf_heads_per_wave(int n_tiles, int nh, int nkv, int hd, int qt_hint) 
     int qt = (G % 4 == 0) ? 4 : (G % 2 == 0 ? 2 : 1);
     const int qt_max = hdp <= 64 ? 4 : 2;
     while (qt > qt_max) qt /= 2;
-    while (qt > 1 && n_tiles * nkv * (G / qt) <= pf_units()) qt /= 2;
+    while (qt > 1 && n_tiles * nkv * (G / qt) <= fl_units()) qt /= 2;
     if (qt_hint == 1 || qt_hint == 2 || qt_hint == 4)
         while (qt > qt_hint) qt /= 2;
     return qt;
@@ -449,7 +439,7 @@ extern "C" int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int 
     if (n_tiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv) return 1;
     const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, 0);
     const int blocks = n_tiles * nkv * ((nh / nkv) / qt);
-    const int want = (2 * pf_units()) / max(blocks, 1);
+    const int want = (2 * fl_units()) / max(blocks, 1);
     const int by_keys = ceil_div(max(max_keys, 1), PF_STAGE) / 8;
     return max(1, min(min(want, by_keys), 16));
 }

@@ -88,6 +88,7 @@ __device__ __forceinline__ size_t cache_v_offset(const PagedCache& c, int page, 
 
 // ---- host side -----------------------------------------------------------
 void fl_set_error(const char* fmt, ...);
+int fl_units(void);              // compute units of the current device (runtime.hip)
 
 #define FL_CHECK(cond, ...)                \
     do {                                   \

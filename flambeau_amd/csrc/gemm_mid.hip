@@ -283,7 +283,7 @@ __global__ __launch_bounds__(1024) void gemm_mid_reduce_residual_kernel(const fl
 // chip with such blocks, four otherwise.
 static int mid_waves(int N, int forced = 0) {
     if (forced == 4 || forced == 8) return forced;
-    return ceil_div(N, 16) >= 1024 ? 8 : 4;
+    return ceil_div(N, 16) >= 4 * fl_units() ? 8 : 4;
 }
 
 // How many ways K is split.  These products are short (tens of microseconds) and run best with
@@ -297,10 +297,11 @@ extern "C" int fl_gemm_mid_splits_ex(int M, int N, int K, int waves, int forced)
     const int n_chunks = ceil_div(ceil_div(K, 32), GM_STEPS);
     if (forced > 0) return min(forced, n_chunks);
     int splits = 1;
-    while (blocks * splits * 2 < 320 && n_chunks / (splits * 2) >= 4 && splits < 32) splits *= 2;
+    const int units = fl_units();               // (the numbers below were measured with 256 of them)
+    while (blocks * splits * 2 < units * 5 / 4 && n_chunks / (splits * 2) >= 4 && splits < 32) splits *= 2;
     // a long K (the down projection of a wide feed-forward) is split further while every part keeps 16
     // chunks: measured at 5120 x 32768 and 64 rows, 88 us with 8 splits against 103 with 4
-    while (blocks < 160 && blocks * splits * 2 <= 640 && n_chunks / (splits * 2) >= 16 && splits < 32) splits *= 2;
+    while (blocks < units * 5 / 8 && blocks * splits * 2 <= units * 5 / 2 && n_chunks / (splits * 2) >= 16 && splits < 32) splits *= 2;
     return splits;
 }
 extern "C" int fl_gemm_mid_splits(int M, int N, int K) { return fl_gemm_mid_splits_ex(M, N, K, 0, 0); }

@@ -350,15 +350,15 @@ static int skinny_tiles(int M, int N, int tiles_hint) {
     if (M > 16) return 1;
     if (tiles_hint > 0) return tiles_hint;
     const int groups = ceil_div(N, 16);
-    return groups > 256 && groups <= 512 ? 2 : 1;
+    return groups > fl_units() && groups <= 2 * fl_units() ? 2 : 1;      // (between one and two row groups per compute unit)
 }
 
 static int skinny_waves(int N, int K, int nw_hint, int T) {
     const int blocks = ceil_div(ceil_div(N, 16), T);
     const int n_steps = ceil_div(K, 32);
-    // enough waves in flight to cover the memory latency: about 2048 and more over the chip
+    // enough waves in flight to cover the memory latency: about eight per compute unit and more
     int nw = 4;
-    while (nw < 16 && blocks * nw < 2048) nw *= 2;
+    while (nw < 16 && blocks * nw < 8 * fl_units()) nw *= 2;
     if (nw_hint > 0) nw = nw_hint;
     if (T > 1 && nw > 8) nw = 8;              // two sets of w registers: blocks of 512 threads at most
     while (nw > 1 && n_steps < nw * 2) nw /= 2;

@@ -427,7 +427,7 @@ static const TileShape& tile_shape(int variant) {
 static bool tiled_known(int variant) { return variant == 0 || tile_shape(variant).variant == variant; }
 
 static float tiled_cost(const TileShape& t, int splits, int M, int N, int K) {
-    const int units = 256;
+    const int units = fl_units();
     const int steps = ceil_div(ceil_div(K, 32), splits);
     const long blocks = (long)ceil_div(N, t.features) * ceil_div(M, t.tokens) * splits;
     const long most = (blocks + units - 1) / units;                    // blocks of the unit with the most

@@ -59,19 +59,34 @@ __global__ __launch_bounds__(256) void sample_count_kernel(unsigned short* __res
     *p = (unsigned short)min(65535u, (unsigned)*p + 1u);
 }
 
-// one slot's row: zeroed, then the `n` tokens counted by one thread (16-bit counts have no atomics; the
-// list is short, and a request takes a slot rarely)
-__global__ __launch_bounds__(256) void sample_history_kernel(unsigned short* __restrict__ counts, int V, int slot,
-                                                             const int* __restrict__ tokens, int n) {
+// One slot's row is counted anew in two kernels: the row is zeroed by a grid over the vocabulary, then
+// every token adds one to its count.  16-bit counts have no atomics of their own: a thread adds 1 or
+// 65536 to the aligned 32-bit word that holds the count (rows start at even counts only if V is even, so
+// the word is found from the count's own address).  Fewer than 65,536 tokens cannot carry from one count
+// into its neighbour; longer lists are counted by one thread, saturating.
+__global__ __launch_bounds__(256) void sample_history_zero_kernel(unsigned short* __restrict__ counts, int V, int slot) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < V) counts[(size_t)slot * V + i] = 0;
+}
+
+__global__ __launch_bounds__(256) void sample_history_count_kernel(unsigned short* __restrict__ counts, int V, int slot,
+                                                                   const int* __restrict__ tokens, int n, int serial) {
     unsigned short* row = counts + (size_t)slot * V;
-    for (int i = threadIdx.x; i < V; i += 256) row[i] = 0;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int j = 0; j < n; ++j) {
-            const int t = tokens[j];
-            if (t >= 0 && t < V) row[t] = (unsigned short)min(65535u, (unsigned)row[t] + 1u);
+    if (serial) {
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            for (int j = 0; j < n; ++j) {
+                const int t = tokens[j];
+                if (t >= 0 && t < V) row[t] = (unsigned short)min(65535u, (unsigned)row[t] + 1u);
+            }
         }
+        return;
     }
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= n) return;
+    const int t = tokens[j];
+    if (t < 0 || t >= V) return;
+    const uintptr_t at = (uintptr_t)(row + t);
+    atomicAdd((unsigned*)(at & ~(uintptr_t)3), (at & 2) ? 65536u : 1u);
 }
 
 // Penalties of the rows that have a history slot (slot[r] >= 0, as a float), in place on logits [rows, V].
@@ -111,8 +126,14 @@ FL_RECORDABLE(fl_sample_count)
 // A request takes a slot: its row is zeroed and the n tokens it has generated so far are counted.
 extern "C" int fl_sample_history(unsigned short* counts, int V, int slot, const int* tokens, int n, hipStream_t stream) {
     FL_CHECK(V > 0 && slot >= 0 && n >= 0 && counts && (n == 0 || tokens), "sample_history: bad arguments");
-    sample_history_kernel<<<1, 256, 0, stream>>>(counts, V, slot, tokens, n);
+    FL_CHECK((uintptr_t)counts % 4 == 0, "sample_history: the counts must be 4-byte aligned");
+    sample_history_zero_kernel<<<ceil_div(V, 256), 256, 0, stream>>>(counts, V, slot);
     FL_LAUNCH_CHECK();
+    if (n > 0) {
+        const int serial = n >= 65536 ? 1 : 0;
+        sample_history_count_kernel<<<serial ? 1 : ceil_div(n, 256), 256, 0, stream>>>(counts, V, slot, tokens, n, serial);
+        FL_LAUNCH_CHECK();
+    }
     return 0;
 }
 FL_RECORDABLE(fl_sample_history)

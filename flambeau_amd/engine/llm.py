@@ -55,7 +55,7 @@ class LLMEngine:
                                    eos_token_id=getattr(spec, "eos_token_ids", ()) or spec.eos_token_id,
                                    default_seed=opt.seed,
                                    row_granule=opt.row_granule or model.rt.row_granule)
-        self.sampler = DeviceSampler(model.rt.device, max(opt.inflight_slots, 1))
+        self.sampler = DeviceSampler(model.rt.device, max(opt.inflight_slots, 1), vocab_size=spec.vocab_size)
         # tokens drawn on the device are fed to the next step on the device: the host enqueues
         # step i + 1 while step i runs and reads step i's tokens afterwards
         self.runner.token_feedback = self.sampler.ids

@@ -24,7 +24,10 @@ class Runtime:
         if not torch.cuda.is_available():
             raise RuntimeError("flambeau_amd: no GPU visible to this process")
         torch.cuda.set_device(self.device)
-        load()   # fails loudly when the kernel library cannot be built or loaded
+        lib = load()   # fails loudly when the kernel library cannot be built or loaded
+        if bool(tuned) and dtype == torch.bfloat16:
+            from ..kernels import tuned as tuned_kernels
+            tuned_kernels.set_units(lib.fl_compute_units())
         self.dtype = dtype
         # tuned kernels exist for bfloat16 only; the 32-bit path always runs the plain ones
         self.tuned = bool(tuned) and dtype == torch.bfloat16

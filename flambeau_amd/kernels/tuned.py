@@ -490,6 +490,7 @@ def prepare_gate_up(gate: torch.Tensor, up: torch.Tensor) -> Weight:
 # Rows of portions up to this length are treated as single query rows by the split-K kernel;
 # longer portions go to the tiled prefill kernel.
 SHORT_PORTION = 8
+DECODE_UNITS = 256                   # compute units of the device (``set_units``; an MI355X has 256)
 DECODE_TARGET_BLOCKS = 512           # two blocks per compute unit
 DECODE_EVEN_BLOCKS = 256             # one per unit: enough when all rows have about the same number of keys
 DECODE_MIN_KEYS_PER_SPLIT = 128
@@ -497,6 +498,13 @@ DECODE_MAX_SPLITS = 64
 
 
 PREFILL_TILE = 64        # query tokens per block of the tiled kernel
+
+
+def set_units(units: int) -> None:
+    """Plan the attention kernels' blocks for a device of ``units`` compute units (the runtime says so
+    when it starts; the library's own plans ask the device themselves)."""
+    global DECODE_UNITS, DECODE_TARGET_BLOCKS, DECODE_EVEN_BLOCKS
+    DECODE_UNITS, DECODE_TARGET_BLOCKS, DECODE_EVEN_BLOCKS = int(units), 2 * int(units), int(units)
 
 
 def attention_metadata(batch, shapes=()) -> dict:
@@ -544,7 +552,6 @@ def decode_item_budget(n_rows: int, blocks_per_row: int) -> int:
 # a compute unit streams keys and values at about 30 GB/s whether one block or two share it, so a step
 # takes as long as the unit with the most bytes (blocks go to the 256 units in turn), a block costs 1.5 us
 # beside its bytes, the kernel that merges splits 4.7 us, and the chip as a whole gives 6.4 TB/s.
-DECODE_UNITS = 256
 DECODE_UNIT_RATE = 30e9
 DECODE_CHIP_RATE = 6.4e12
 DECODE_BLOCK_US = 1.5

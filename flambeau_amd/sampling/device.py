@@ -17,7 +17,10 @@ from .params import DEVICE_BIAS_MAX as BIAS_MAX
 
 
 class DeviceSampler:
-    def __init__(self, device, max_rows: int):
+    def __init__(self, device, max_rows: int, vocab_size: int | None = None):
+        """``vocab_size``: if given, the counts for the penalties and the scratch of the filtered draw
+        are made now, beside everything else that is sized when an engine is built (64 + 128 MB at 256
+        rows and a vocabulary of 131,072); without it they are made when a request first needs them."""
         self.device = device
         self.max_rows = max_rows
         # per row: 1 / temperature, the uniform number, top-k (0: none), top-p (0: none), min-p (0: none),
@@ -34,6 +37,10 @@ class DeviceSampler:
         self._events = [torch.cuda.Event(), torch.cuda.Event()]
         self._turn = 0
         self._stash = None           # scratch of the filtered draw for vocabularies beyond 32,768
+        if vocab_size is not None:
+            self._counts = torch.zeros((max_rows, vocab_size), dtype=torch.int16, device=device)
+            if vocab_size > 32768:
+                self._stash = torch.empty(max_rows * vocab_size, dtype=torch.int32, device=device)
 
     def _histories(self, k, logits, histories):
         """Penalties of the rows that ask for them; returns the device array of their slots."""
