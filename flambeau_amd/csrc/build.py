@@ -149,5 +149,33 @@ def build(force: bool = False, verbose: bool = True) -> Path:
     return target
 
 
+def build_own_library(name: str, srcs: list, out_dir, force: bool = False) -> Path:
+    """Compile HIP sources of the caller's own (a part that brings kernels which this library does not
+    have) into ``out_dir/lib<name>-<hash>.so``, with this library's flags and with this folder on the
+    include path (``api.h`` for ``FlArg``, ``recordable.h`` for the trampoline a step program replays a
+    launch function through).  Compiles only if that file is missing, or when ``force``."""
+    srcs = [Path(s) for s in srcs]
+    h = hashlib.sha256()
+    for s in srcs + _headers():
+        h.update(s.name.encode())
+        h.update(s.read_bytes())
+    h.update(" ".join(FLAGS).encode())
+    out_dir = Path(out_dir)
+    out_dir.mkdir(parents=True, exist_ok=True)
+    target = out_dir / f"lib{name}-{h.hexdigest()[:16]}.so"
+    if target.exists() and not force:
+        return target
+    tmp = target.with_suffix(f".tmp{os.getpid()}.so")
+    _run([_hipcc(), *FLAGS, "-I", str(CSRC), "-shared", "-o", str(tmp), *map(str, srcs)], f"compiling {name}")
+    os.replace(tmp, target)
+    for old in out_dir.glob(f"lib{name}-*.so"):
+        if old != target:
+            try:
+                old.unlink()
+            except OSError:
+                pass
+    return target
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv))

@@ -55,6 +55,8 @@ def load():
     lib.fl_last_error.argtypes = []
     lib.fl_abi_version.restype = c_int
     for name, args in _SIGNATURES.items():
+        if name in _functions:          # a launch function of a part's own library
+            continue
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = c_int
@@ -172,6 +174,10 @@ class Program:
 
     def __len__(self):
         return len(self._names)
+
+    def names(self) -> list:
+        """The launch functions recorded, in order."""
+        return list(self._names)
 
     def append(self, name: str, args) -> None:
         types = _SIGNATURES[name]

@@ -87,3 +87,19 @@ def test_a_launch_function_from_elsewhere_can_be_registered():
         assert seen == [(5, 0.25, 1234), (-1, 1.5, 1234)]
     finally:
         del library._SIGNATURES["toy_launch"]
+
+
+def test_a_function_of_another_library_registered_before_the_first_load_stays_there():
+    """A part may give the argument list of its own launch function before anything has loaded the kernel
+    library; loading then looks up only its own functions."""
+    import subprocess
+    import sys
+    code = ("import ctypes\n"
+            "from flambeau_amd.kernels import library\n"
+            "assert library._lib is None\n"
+            "library.register_signatures({'getpid': []}, library=ctypes.CDLL(None))\n"
+            "library.load()\n"
+            "assert library._functions['getpid']() > 0\n"
+            "print('ok')\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=str(CSRC.parent.parent))
+    assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr
