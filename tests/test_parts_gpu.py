@@ -588,6 +588,154 @@ def test_a_part_that_cannot_be_captured_keeps_decode_steps_out_of_graphs(tmp_pat
     assert random_model(TINY["A"]["config"], 1, dtype="bfloat16")[0].capturable()
 
 
+def _register_parallel_toys():
+    """Another arrangement of a layer, another embedding and another head, known to this test only."""
+    from dataclasses import dataclass
+    from flambeau_amd.config.base import KeyReader
+    from flambeau_amd.models.decoder import LayerSpec, ModelSpec, RunEntry
+    from flambeau_amd.parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Block, OutputHead, PartSpec,
+                                    TokenEmbedding)
+    from flambeau_amd.registry import known_architectures, register_architecture
+    if "ToyParallelLM" in known_architectures():
+        return
+
+    @BLOCKS.register("toy_parallel")
+    class ParallelBlock(Block):
+        """x += Mixer(Norm(x)) + FeedForward(Norm(x)): one norm, both parts read the same normed rows."""
+        replayable = True
+
+        def __init__(self, mixer, feed_forward, norm):
+            self.norm, self.mixer, self.ffn = NORMS.create(norm), MIXERS.create(mixer), FEED_FORWARDS.create(feed_forward)
+            self._parts = {"norm": self.norm, "mixer": self.mixer, "ffn": self.ffn}
+
+        def cache_spec(self):
+            return self.mixer.cache_spec()
+
+        def mixers(self):
+            return [self.mixer]
+
+        def subparts(self):
+            return list(self._parts.values())
+
+        def tensors(self):
+            return {f"{p}.{name}": spec for p, part in self._parts.items() for name, spec in part.tensors().items()}
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            for p, part in self._parts.items():
+                part.bind({k[len(p) + 1:]: v for k, v in weights.items() if k.startswith(p + ".")}, rt)
+
+        def forward(self, stream, step, cache):
+            a = stream.normed(self.norm, name="toy_parallel_normed")
+            stream.push(self.mixer.forward(a, step, cache))
+            stream.push(self.ffn.forward(a, step))
+
+    @EMBEDDINGS.register("toy_scaled_embedding")
+    class ScaledEmbedding(TokenEmbedding):
+        """h0 = scale * E[token]."""
+        replayable = False
+
+        def __init__(self, vocab_size, hidden_size, scale):
+            super().__init__(vocab_size, hidden_size)
+            self.scale = scale
+
+        def forward(self, tokens, out):
+            super().forward(tokens, out)
+            return out.mul_(self.scale)
+
+    @HEADS.register("toy_capped_head")
+    class CappedHead(OutputHead):
+        """logits = cap * tanh(x W^T / cap)."""
+        replayable = False
+
+        def __init__(self, vocab_size, hidden_size, cap, tied=False):
+            super().__init__(vocab_size, hidden_size, tied)
+            self.cap = cap
+
+        def forward(self, x, max_rows):
+            logits = super().forward(x, max_rows)
+            return logits.copy_(self.cap * torch.tanh(logits / self.cap))
+
+    @dataclass(frozen=True)
+    class ParallelConfig:
+        hidden_size: int
+        vocab_size: int
+        n_layers: int
+        embedding_scale: float
+        logit_cap: float
+        window: int
+        max_position_embeddings: int
+
+        @classmethod
+        def from_dict(cls, raw, where="config.json"):
+            r = KeyReader(raw, where)
+            return cls(r.integer("hidden_size"), r.integer("vocab_size"), r.integer("n_layers"), r.number("embedding_scale"),
+                       r.number("logit_cap"), r.integer("window"), r.integer("max_position_embeddings"))
+
+    def spec(cfg):
+        H = cfg.hidden_size
+        norm = PartSpec("rmsnorm", dict(hidden_size=H, eps=1e-4))
+        mixer = PartSpec("paged_gqa_attention", dict(hidden_size=H, n_heads=4, n_kv_heads=2, head_dim=16, window=cfg.window,
+                                                     position=PartSpec("rope_neox", dict(head_dim=16, theta=500.0))))
+        ffn = PartSpec("swiglu", dict(hidden_size=H, intermediate_size=56))
+        layers = []
+        for l in range(cfg.n_layers):
+            names = {f"mixer.{t}.weight": f"p{l}.{t}_proj.weight" for t in "qkvo"}
+            names.update({"norm.weight": f"p{l}.norm", "ffn.gate.weight": f"p{l}.gate", "ffn.up.weight": f"p{l}.up",
+                          "ffn.down.weight": f"p{l}.down"})
+            layers.append(LayerSpec(PartSpec("toy_parallel", dict(mixer=mixer, feed_forward=ffn, norm=norm)), names))
+        sizes = dict(vocab_size=cfg.vocab_size, hidden_size=H)
+        return ModelSpec("ToyParallelLM", H, cfg.vocab_size, cfg.max_position_embeddings, layers,
+                         [RunEntry(l) for l in range(cfg.n_layers)], norm,
+                         {"embedding.weight": "table", "final_norm.weight": "norm"}, tied_head=True,
+                         embedding=PartSpec("toy_scaled_embedding", dict(sizes, scale=cfg.embedding_scale)),
+                         head=PartSpec("toy_capped_head", dict(sizes, cap=cfg.logit_cap, tied=True)))
+
+    register_architecture("ToyParallelLM", ParallelConfig, spec)
+
+
+def _parallel_plain(cfg, w, toks):
+    n, pos = len(toks), np.arange(len(toks))
+    x = cfg["embedding_scale"] * w["table"][toks]
+    for l in range(cfg["n_layers"]):
+        a = pm.rmsnorm(x, w[f"p{l}.norm"], 1e-4)
+        x = x + pm.attention_mixer(a, w, f"p{l}.", pos, 4, 2, 16, 500.0, cfg["window"]) \
+              + pm.swiglu_mlp(a, w[f"p{l}.gate"], w[f"p{l}.up"], w[f"p{l}.down"])
+    logits = pm.rmsnorm(x, w["norm"], 1e-4) @ w["table"].T
+    return cfg["logit_cap"] * np.tanh(logits / cfg["logit_cap"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_another_arrangement_embedding_and_head_from_a_test_file(tmp_path, dtype):
+    """A layer whose mixer and feed-forward read the same normed rows, an embedding with a scale, a tied
+    head with a soft cap on its logits: registered here, named by the model's description
+    (``ModelSpec.embedding``, ``.head``, a block kind), built from a config.json and stepped in every cutting."""
+    import replay_helpers as rh
+    from flambeau_amd.engine import ModelRunner, load_model
+    from flambeau_amd.weights import write_random_model
+    _register_parallel_toys()
+    cfg = dict(architectures=["ToyParallelLM"], hidden_size=40, vocab_size=77, n_layers=3, embedding_scale=6.3, logit_cap=4.0,
+               window=21, max_position_embeddings=128)
+    d = write_random_model(cfg, tmp_path / "par", seed=9, std=0.15, gain_std=0.05, store_dtype=torch.float32)
+    model, _ = load_model(d, dtype=dtype, max_batch_tokens=128)
+    assert [type(b).__name__ for b in model.blocks] == ["ParallelBlock"] * 3
+    assert type(model.embedding).__name__ == "ScaledEmbedding" and type(model.head).__name__ == "CappedHead"
+    assert not model.replayable()          # embedding and head call torch: such a model's steps are run, never replayed
+    runner = ModelRunner(model, n_pages=14, page_size=8, max_slots=3, max_logit_rows=128)
+    assert not runner.step_programs and not runner.decode_graphs
+    w = {k: v for k, v in pm.read_safetensors(d / "model.safetensors").items()}
+    if dtype == "bfloat16":
+        w = {k: pm.round_bf16(v) if v.ndim == 2 else v for k, v in w.items()}
+    reqs = rh.make_requests(77, [33, 11, 40, 26], seed=12)
+    ref = {rid: _parallel_plain(cfg, w, toks) for rid, toks in reqs.items()}
+    assert max(np.abs(r).max() for r in ref.values()) > 2.0          # the cap bends the logits
+    for mode, steps in [("whole", rh.trace_whole(reqs)), ("tail", rh.trace_tail(reqs, tail=10)),
+                        ("portions", rh.trace_portions(reqs, sizes=(2, 9, 3, 14))),
+                        ("mixed", rh.trace_mixed(reqs, seed=6, max_live=3, max_portion=9, decode_tail=5))]:
+        rh.compare(rh.run_in_process(runner, steps), reqs, ref, dtype, f"parallel toy {mode}")
+    assert not runner.manager.live and runner.manager.free_pages() == [14]
+
+
 def test_unknown_part_names_the_known_ones():
     from flambeau_amd.parts import MIXERS, PartSpec
     with pytest.raises(KeyError, match="paged_gqa_attention"):
