@@ -301,7 +301,7 @@ def bench_serving(a, name, label, cfg, dtype_name, el):
     r = sorted(runs, key=lambda x: x["t_decode"])[len(runs) // 2]
     window = cfg["sliding_window"] or 0
     extra_points = {}
-    if name == "24b":
+    if name == "24b" and not a.no_points:
         # decode at batch 1 and 8 behind 2,048 tokens each (the cache filled with random values)
         for b in (1, 8):
             dtl, ctxl = run_decode_filled(model, b, PROMPT_LEN, steps=32, warmup=8)
