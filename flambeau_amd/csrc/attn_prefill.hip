@@ -60,12 +60,16 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
     const int hd = cache.head_dim, ps = cache.page_size;
     const int G = nh / cache.n_kv_heads;
     const int hgroups = G / QT;
-    const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
     // Tiles late in a prompt have the most keys: they are started first.  When the whole grid is on
     // the chip at once (two blocks per compute unit, the second half of the grid beside the first),
     // the second half runs the other way round, so that a long tile shares its unit with a short one.
+    // A grid that comes in several rounds (mirror_from < 0) starts all head groups of the longest tile,
+    // then all of the next: no long tile is left for the end.
     const int lin = blockIdx.y * gridDim.x + blockIdx.x;
-    const int tile = lin < mirror_from ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+    const int by = mirror_from < 0 ? lin % gridDim.y : blockIdx.y;
+    const int tile = mirror_from < 0 ? gridDim.x - 1 - lin / gridDim.y
+                                     : (lin < mirror_from ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
+    const int kvh = by / hgroups, hg = by % hgroups;
     const int seq = tiles[4 * tile], row0 = tiles[4 * tile + 1], cnt = tiles[4 * tile + 2], item0 = tiles[4 * tile + 3];
     const int* table = block_table + (size_t)seq * max_blocks;
     const bf16_t* kv = (const bf16_t*)cache.base;
@@ -389,7 +393,8 @@ static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, b
     const int lds = RING + lds_pages * (int)sizeof(int);
     const int resident = units * ((QT * HDP <= 256 && 2 * lds <= PF_LDS_BYTES) ? 2 : 1);
     // (whole rows of the grid: every tile of a head group is taken exactly once either way)
-    const int mirror_from = (resident == 2 * units && grid.z == 1 && total <= resident && total > units) ? (int)((grid.y / 2) * grid.x) : (int)(grid.x * grid.y);
+    const int mirror_from = (resident == 2 * units && grid.z == 1 && total <= resident && total > units) ? (int)((grid.y / 2) * grid.x)
+                            : (grid.z == 1 && total > resident) ? -1 : (int)(grid.x * grid.y);
     static bool configured = false;
     auto kern = attn_prefill_kernel<HDP, QT, NS>;
     if (!configured) {

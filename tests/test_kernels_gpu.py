@@ -1062,6 +1062,34 @@ def test_attn_prefill_with_block_tables_beyond_4096_pages(nh, nkv, hd, window):
         assert (out.double().reshape(n, nh, hd) - ref).abs().max() < 2e-2 * ref.abs().max(), n_split
 
 
+@pytest.mark.parametrize("nh,nkv,hd,window", [(8, 8, 32, 0), (16, 8, 64, 700)])
+def test_attn_prefill_grid_that_comes_in_several_rounds(nh, nkv, hd, window):
+    """More blocks than the chip holds at once (over 70 tiles of 64 tokens x 8 kv heads): such a grid starts
+    the tiles with the most keys first, all head groups of a tile side by side; every (tile, head group)
+    must still be taken exactly once.  Three requests, so that the list of tiles is not in order of length."""
+    ps = 16
+    seqs = [(3000, 3000), (1500, 1300), (200, 150), (77, 77)]
+    tiles = tiles_for(seqs)
+    assert tiles.shape[0] * nkv > 2 * 256
+    case = build_long_attention_case(nh, nkv, hd, ps, seqs, 192, seed=3)
+    n = case["n"]
+    scale = 1 / math.sqrt(hd)
+    q2 = case["q"].reshape(n, nh * hd)
+    out = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    tuned().attn_prefill(q2, out, case["cache"], tiles, case["pos_d"], case["table"], nh, scale, window)
+    assert not torch.isnan(out).any()
+    plain = torch.empty_like(out)
+    ops().attn_plain(q2, plain, case["cache"], case["pos_d"], case["seq_d"], case["table"], nh, scale, window)
+    top = plain.double().abs().max()
+    assert (out.double() - plain.double()).abs().max() < 1.5e-2 * top
+    # the float64 formula at the rows of a few tiles: the longest, one in the middle, the last request's
+    rows = list(range(2936, 3000)) + list(range(3000 + 640, 3000 + 704)) + list(range(n - 77, n))
+    for i in rows[::3]:
+        s_, p_ = case["tok_seq"][i], case["pos"][i]
+        ref = attention_ref(case["q"][i].double(), case["K"][s_], case["V"][s_], p_, scale, window)
+        assert (out[i].double().reshape(nh, hd) - ref).abs().max() < 1e-2 * top, i
+
+
 def test_attn_prefill_table_limits_come_from_the_library():
     """Tables wider than a block can keep are refused by the kernel, and the wrapper that chooses the
     kernel asks the same function; with a window only the window's pages count."""
