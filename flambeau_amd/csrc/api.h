@@ -176,6 +176,7 @@ int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int*
 int fl_attn_prefill_max_pages(int hd);
 int fl_attn_prefill_takes(int hd, int page_size, int max_blocks, int window);
 int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int max_keys);
+int fl_attn_prefill_heads(int n_tiles, int nh, int nkv, int hd, int max_keys);      // query heads per wave: the qt_hint to pass
 int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 

@@ -421,32 +421,59 @@ static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* 
         launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml, lds_pages);
 }
 
-// query heads per wave: a divisor of the group size; as many as leave room for two blocks per
-// compute unit (two waves per SIMD hide each other's waits: measured 906 against 1314 us at 8192
-// tokens with 2 heads instead of 4 at head size 128), and few enough that the grid has more blocks
-// than the chip has units (a short portion: measured 176 against 217 us for 512 tokens behind 7,680
-// with 1 head instead of 2)
-static int pf_heads_per_wave(int n_tiles, int nh, int nkv, int hd, int qt_hint) {
+// Query heads per wave (QT, a divisor of the group size) and parts of the keys for a batch of n_tiles
+// tiles whose longest context has max_keys keys.
+//  * At most as many heads as leave room for two blocks per compute unit (two waves per SIMD hide each
+//    other's waits: 906 against 1314 us at 8192 tokens with 2 heads instead of 4 at head size 128).
+//  * A grid of fewer than two blocks per unit is filled by splitting the keys, as long as every part keeps
+//    12 stages of 64 keys or so, rather than by fewer heads per wave: a block of two heads reads its keys
+//    and values once for both (512 tokens behind 7,680 keys: 99 us with two heads and 4 parts against 125
+//    with one head and 2; behind 32,256: 314 against 422; 64 tokens behind 32,704: 83 against 115).
+//  * Where the keys are too few for that (a whole prompt of 1,024 tokens: 16 stages at most), fewer heads
+//    per wave give the blocks (29 us with one head, 35 with two).
+struct PrefillPlan { int qt, splits; };
+static PrefillPlan pf_plan(int n_tiles, int nh, int nkv, int hd, int max_keys) {
     const int G = nh / nkv;
     const int hdp = ceil_div(hd, 32) * 32;
     int qt = (G % 4 == 0) ? 4 : (G % 2 == 0 ? 2 : 1);
     const int qt_max = hdp <= 64 ? 4 : 2;
     while (qt > qt_max) qt /= 2;
-    while (qt > 1 && n_tiles * nkv * (G / qt) <= fl_units()) qt /= 2;
-    if (qt_hint == 1 || qt_hint == 2 || qt_hint == 4)
+    const int slots = 2 * fl_units();
+    const int by_keys = max(1, ceil_div(max(max_keys, 1), PF_STAGE) / 12);
+    for (;; qt /= 2) {
+        const int blocks = max(1, n_tiles * nkv * (G / qt));
+        if (blocks >= slots) return {qt, 1};
+        const int splits = max(1, min(min(slots / blocks, by_keys), 16));
+        // (at the most parts there are, fewer heads would only read the keys more often)
+        if (qt == 1 || splits == 16 || blocks * splits >= slots * 5 / 8) return {qt, splits};
+    }
+}
+
+// query heads per wave for fl_attn_prefill: qt_hint (1, 2 or 4) at most that many; else what goes with
+// the parts the caller has chosen
+static int pf_heads_per_wave(int n_tiles, int nh, int nkv, int hd, int qt_hint, int n_split) {
+    const int G = nh / nkv;
+    const int hdp = ceil_div(hd, 32) * 32;
+    int qt = (G % 4 == 0) ? 4 : (G % 2 == 0 ? 2 : 1);
+    const int qt_max = hdp <= 64 ? 4 : 2;
+    while (qt > qt_max) qt /= 2;
+    if (qt_hint == 1 || qt_hint == 2 || qt_hint == 4) {
         while (qt > qt_hint) qt /= 2;
+        return qt;
+    }
+    while (qt > 1 && n_tiles * nkv * (G / qt) * n_split < 3 * fl_units() / 2) qt /= 2;
     return qt;
 }
 
-// Into how many parts the keys are split: 1 unless the tiles are so few that the chip stays mostly
-// empty and the longest context (max_keys) gives every part at least 8 stages of 64 keys.
+// Query heads per wave for a batch of this shape (what fl_attn_prefill takes as its hint), and into how
+// many parts its keys are split (1: not at all).
+extern "C" int fl_attn_prefill_heads(int n_tiles, int nh, int nkv, int hd, int max_keys) {
+    if (n_tiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv) return 1;
+    return pf_plan(n_tiles, nh, nkv, hd, max_keys).qt;
+}
 extern "C" int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int max_keys) {
     if (n_tiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv) return 1;
-    const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, 0);
-    const int blocks = n_tiles * nkv * ((nh / nkv) / qt);
-    const int want = (2 * fl_units()) / max(blocks, 1);
-    const int by_keys = ceil_div(max(max_keys, 1), PF_STAGE) / 8;
-    return max(1, min(min(want, by_keys), 16));
+    return pf_plan(n_tiles, nh, nkv, hd, max_keys).splits;
 }
 
 // Block-table entries per request that the kernel takes at a head size: the table of a request sits in
@@ -553,7 +580,7 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     const int hdp = ceil_div(hd, 32) * 32;
     int log2_ps = 0;
     while ((1 << log2_ps) < page_size) ++log2_ps;
-    const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, qt_hint);
+    const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, qt_hint, n_split);
     dim3 grid(n_tiles, nkv * (G / qt), n_split);
     const float sl = scale * 1.4426950408889634f;
     // a ring of two stages: two blocks then fit a compute unit (three stages were no faster)

@@ -40,6 +40,7 @@ register_signatures({
     "fl_gemm_tiled_shape": [I, I, I, I],
     "fl_attn_prefill": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, P, I, P],
     "fl_attn_prefill_splits": [I, I, I, I, I],
+    "fl_attn_prefill_heads": [I, I, I, I, I],
     "fl_attn_prefill_max_pages": [I],
     "fl_attn_prefill_takes": [I, I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
@@ -685,6 +686,13 @@ def attn_prefill_splits(n_tiles: int, n_heads: int, n_kv_heads: int, head_dim: i
     return load().fl_attn_prefill_splits(n_tiles, n_heads, n_kv_heads, head_dim, max_keys)
 
 
+def attn_prefill_heads(n_tiles: int, n_heads: int, n_kv_heads: int, head_dim: int, max_keys: int) -> int:
+    """Query heads per wave that the tiled kernel wants for a batch of this shape (``heads_per_wave`` of
+    ``attn_prefill``; the splits of ``attn_prefill_splits`` go with it)."""
+    from .library import load
+    return load().fl_attn_prefill_heads(n_tiles, n_heads, n_kv_heads, head_dim, max_keys)
+
+
 def attn_prefill(q, out, cache, tiles, positions, table, n_heads, scale, window, heads_per_wave: int = 0,
                  n_split: int = 1, part_o=None, part_ml=None):
     """Attention of the longer portions; ``tiles[i] = (request's row in ``table``, first row, rows,
@@ -732,8 +740,9 @@ def prefill_supported(cache, table, window: int = 0) -> bool:
 
 
 def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int, with_items: bool = True):
-    """``(parts of the keys for the tiled kernel, for the single-row kernel)`` for a batch: everything
-    that ``attention`` decides from the contexts' lengths (the rest follows from the batch's shape).
+    """``(parts of the keys for the tiled kernel + 64 x its query heads per wave, parts for the single-row
+    kernel)`` for a batch: everything that ``attention`` decides from the contexts' lengths (the rest
+    follows from the batch's shape).
     ``with_items``: the single rows come with splits of their own (``balanced_items``), which are
     data of the step; all they decide here is whether any row is split at all (0 if so: the kernel
     that merges runs; -1 if not: it is left out)."""
@@ -743,7 +752,8 @@ def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window
     if n_tiles:
         # few tiles before a long context: the keys are split too, so that the chip has blocks enough
         longest = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + PREFILL_TILE)
-        p_split = attn_prefill_splits(n_tiles, n_heads, n_kv_heads, head_dim, longest)
+        p_split = attn_prefill_splits(n_tiles, n_heads, n_kv_heads, head_dim, longest) \
+            + 64 * attn_prefill_heads(n_tiles, n_heads, n_kv_heads, head_dim, longest)
     if n_items and not with_items:
         max_ctx = batch.ctx_bound or batch.max_ctx_len
         if window:
@@ -770,6 +780,7 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
         splits = step.scratch[key] = attention_splits(batch, n_heads, cache.n_kv_heads, cache.head_dim, window,
                                                        with_items=items is not None)
     p_split, n_split = splits
+    p_heads, p_split = p_split >> 6, p_split & 63
     if tiles.shape[0]:
         p_o = p_ml = None
         if p_split > 1:
@@ -777,7 +788,8 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
             hdp = -(-cache.head_dim // 32) * 32
             p_o = rt.buffer("attn_tile_part_o", n_rows * n_heads * p_split, hdp, torch.float32, max_rows=1 << 24)
             p_ml = rt.buffer("attn_tile_part_ml", n_rows * n_heads * p_split, 2, torch.float32, max_rows=1 << 24)
-        attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window, n_split=p_split, part_o=p_o, part_ml=p_ml)
+        attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window, heads_per_wave=p_heads,
+                     n_split=p_split, part_o=p_o, part_ml=p_ml)
     if rows.shape[0] and items is not None:
         # rows with splits of their own; the list's length follows from the number of rows alone
         # (a list with a place per row and no more: no row is ever split, nothing to merge)

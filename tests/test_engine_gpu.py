@@ -613,7 +613,7 @@ def test_cutting_at_real_layer_sizes(wide_model_dir, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_short_portions_behind_a_long_context(tmp_path_factory, dtype):
-    """A request of 1,500 tokens in portions that shrink: the late portions give the tiled attention
+    """A request of 2,000 tokens in portions that shrink: the late portions give the tiled attention
     few tiles with many keys, which it then splits over blocks and merges."""
     import torch
     from flambeau_amd.engine import ModelRunner, load_model
@@ -625,12 +625,12 @@ def test_short_portions_behind_a_long_context(tmp_path_factory, dtype):
               "rms_norm_eps": 1e-5, "max_position_embeddings": 2048, "tie_word_embeddings": False}
     d = write_random_model(config, tmp_path_factory.mktemp("long") / "model", seed=12, std=0.08, gain_std=0.02,
                            store_dtype=STORE_DTYPE[dtype])
-    assert tuned.attn_prefill_splits(2, 4, 2, 16, 1400) > 1
-    reqs = rh.make_requests(150, [1500], seed=9)
+    assert tuned.attn_prefill_splits(2, 4, 2, 16, 1900) > 1
+    reqs = rh.make_requests(150, [2000], seed=9)
     model, _ = load_model(d, dtype=dtype, max_batch_tokens=1024)
-    runner = ModelRunner(model, n_pages=100, page_size=16, max_slots=2, max_logit_rows=1024)
+    runner = ModelRunner(model, n_pages=140, page_size=16, max_slots=2, max_logit_rows=1024)
     runner.storage.fill(float("nan"))
-    steps = rh.trace_portions(reqs, sizes=(700, 500, 100, 64, 9, 70, 30, 27))
+    steps = rh.trace_portions(reqs, sizes=(1000, 700, 100, 64, 9, 70, 30, 27))
     got = rh.run_in_process(runner, steps)
     rh.compare(got, reqs, rh.plain_logits(d, reqs), dtype, "long context")
 

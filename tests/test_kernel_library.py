@@ -103,3 +103,23 @@ def test_a_function_of_another_library_registered_before_the_first_load_stays_th
             "print('ok')\n")
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=str(CSRC.parent.parent))
     assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr
+
+
+def test_the_tiled_attention_s_plan_for_few_tiles():
+    """Heads per wave and parts of the keys for a batch's shape (7B head counts, 256 units): a grid of too
+    few blocks is filled by parts of the keys while a part keeps a dozen stages, by fewer heads per wave
+    where the keys are too few for that; the two numbers come from one plan."""
+    def plan(tokens, keys):
+        n_tiles = -(-tokens // 64)
+        return tuned.attn_prefill_heads(n_tiles, 32, 8, 128, keys), tuned.attn_prefill_splits(n_tiles, 32, 8, 128, keys)
+    assert plan(2048, 2048) == (2, 1)               # 512 blocks as it is
+    assert plan(1024, 1024) == (1, 1)               # too few keys to split: one head per wave gives the blocks
+    assert plan(512, 512) == (1, 1)
+    assert plan(512, 8192) == (2, 4) and plan(512, 32768) == (2, 4)
+    assert plan(256, 32768) == (2, 8) and plan(64, 32768) == (2, 16)
+    assert plan(512, 1536) == (1, 2)
+    for tokens in (64, 200, 512, 1000, 3000):
+        for keys in (tokens, 2000, 9000, 70000, 262144):
+            h, s = plan(tokens, max(keys, tokens))
+            assert h in (1, 2) and 1 <= s <= 16
+            assert s == 1 or max(keys, tokens) // 64 // s >= 10        # a part keeps its stages
