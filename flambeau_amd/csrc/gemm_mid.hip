@@ -286,23 +286,42 @@ static int mid_waves(int N, int forced = 0) {
     return ceil_div(N, 16) >= 4 * fl_units() ? 8 : 4;
 }
 
-// How many ways K is split.  These products are short (tens of microseconds) and run best with
-// about one block per compute unit (measured on the 7B shapes at 32 and 64 rows); a part is at
-// least 4 chunks long.
+// Waves per block and parts of K for a product whose K may be split.  These products are short (tens of
+// microseconds) and a block has its compute unit to itself, so they run best as one round of blocks that
+// fills the chip as far as it goes: parts = units / blocks, rounded down, whatever number that is (a part is
+// at least 4 chunks long, 8 for blocks of eight waves).  Measured at 64 rows: 5120 x 4096 in 80 blocks x 3
+// parts 15.4 us, x 2 18.0, x 4 20.0; 5120 x 32768 in 40 blocks of eight waves x 6 parts 59 us, in 80 of four
+// x 3 74, x 8 (more than two rounds) 80.  Eight waves stream about 30 GB/s per unit against 22 for four
+// and are taken where that outweighs their longer blocks, by 15 % if a block streams less than a megabyte
+// (in effect for the long K of a wide feed-forward's down product); the chip as a whole gives 6.3 TB/s; parts cost a kernel that adds them and their way to memory
+// and back.
 // (The entry points whose names end in _ex take waves per block and K-splits from the caller, for
 // tests and measurements: 0 = chosen here.)
+struct MidPlan { int waves, splits; };
+static MidPlan mid_plan(int N, int K, int forced_waves, int forced_splits) {
+    const int groups = ceil_div(N, 16);
+    const int n_chunks = ceil_div(ceil_div(K, 32), GM_STEPS);
+    const int units = fl_units();
+    MidPlan best = {4, 1};
+    float best_us = 0.f;
+    for (int w = 4; w <= 8; w *= 2) {
+        if (forced_waves ? w != forced_waves : (w == 4 && groups >= 4 * units)) continue;      // (many row groups: eight share x)
+        const int blocks = ceil_div(groups, w);
+        const int s = forced_splits > 0 ? min(forced_splits, n_chunks)
+                                        : max(1, min(min(units / blocks, n_chunks / (w == 8 ? 8 : 4)), 32));
+        const long total = (long)blocks * s;
+        const float bytes = (float)groups * 32.f * K / total;                                   // of w per block
+        const float rate = fminf(w == 8 ? 30e3f : 22e3f, 6.3e6f / (float)min(total, (long)units));   // bytes per us
+        float us = (float)ceil_div((int)total, units) * bytes / rate + (s > 1 ? 4.5f + s * 64.f * N * 8.f / 5e6f : 0.f);
+        if (w == 8 && bytes < 1e6f) us *= 1.15f;      // (their higher rate shows in long streams only: no gain measured at 262 KB per block)
+        if (best_us == 0.f || us < best_us) { best = {w, s}; best_us = us; }
+    }
+    return best;
+}
+
 extern "C" int fl_gemm_mid_splits_ex(int M, int N, int K, int waves, int forced) {
     (void)M;
-    const int blocks = ceil_div(ceil_div(N, 16), mid_waves(N, waves));
-    const int n_chunks = ceil_div(ceil_div(K, 32), GM_STEPS);
-    if (forced > 0) return min(forced, n_chunks);
-    int splits = 1;
-    const int units = fl_units();               // (the numbers below were measured with 256 of them)
-    while (blocks * splits * 2 < units * 5 / 4 && n_chunks / (splits * 2) >= 4 && splits < 32) splits *= 2;
-    // a long K (the down projection of a wide feed-forward) is split further while every part keeps 16
-    // chunks: measured at 5120 x 32768 and 64 rows, 88 us with 8 splits against 103 with 4
-    while (blocks < units * 5 / 8 && blocks * splits * 2 <= units * 5 / 2 && n_chunks / (splits * 2) >= 16 && splits < 32) splits *= 2;
-    return splits;
+    return mid_plan(N, K, waves, forced).splits;
 }
 extern "C" int fl_gemm_mid_splits(int M, int N, int K) { return fl_gemm_mid_splits_ex(M, N, K, 0, 0); }
 
@@ -372,7 +391,9 @@ extern "C" int fl_gemm_mid_ex(const void* x, const void* w_packed, void* out, fl
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
     const MidScale sc = {in_ssq, in_parts, eps};
-    const int splits = epilogue ? 1 : fl_gemm_mid_splits_ex(M, N, K, waves, forced_splits);
+    const MidPlan plan = epilogue ? MidPlan{mid_waves(N, waves), 1} : mid_plan(N, K, waves, forced_splits);
+    const int splits = plan.splits;
+    waves = plan.waves;
     FL_CHECK(splits == 1 || workspace, "gemm_mid: this shape splits K %d ways and needs a workspace", splits);
     if (epilogue) {
         if (out_dtype == FL_F32) launch_mid_mt<float, true>(mt, xb, wb, (float*)out, M, N, K, 1, out_cols, sc, stream, waves);
@@ -420,8 +441,9 @@ extern "C" int fl_gemm_mid_partials(const void* x, const void* w_packed, float* 
              in_parts, GM_SCALE_PARTS);
     if (M == 0) return 0;
     const MidScale sc = {in_ssq, in_parts, eps};
+    const MidPlan plan = mid_plan(N, K, 0, 0);
     launch_mid_mt<float, false>(ceil_div(M, 16), (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K,
-                                fl_gemm_mid_splits(M, N, K), N, sc, stream);
+                                plan.splits, N, sc, stream, plan.waves);
     FL_LAUNCH_CHECK();
     return 0;
 }
@@ -437,10 +459,11 @@ extern "C" int fl_gemm_mid_residual(const void* x, const void* w_packed, float* 
     FL_CHECK(((uintptr_t)workspace % 16 == 0) && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)g % 16 == 0) &&
              ((uintptr_t)xg % 8 == 0), "gemm_mid_residual: workspace, resid and g must be 16-byte aligned, xg 8-byte");
     if (M == 0) return 0;
-    const int splits = fl_gemm_mid_splits(M, N, K);
+    const MidPlan plan = mid_plan(N, K, 0, 0);
+    const int splits = plan.splits;
     const MidScale none = {nullptr, 0, 0.f};
     launch_mid_mt<float, false>(ceil_div(M, 16), (const bf16_t*)x, (const bf16_t*)w_packed, workspace, M, N, K, splits, N,
-                                none, stream);
+                                none, stream, plan.waves);
     FL_LAUNCH_CHECK();
     dim3 grid(ceil_div(N, GM_RED_COLS), M);
     gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(workspace, resid, g, (bf16_t*)xg, out_ssq, M, N, splits);
