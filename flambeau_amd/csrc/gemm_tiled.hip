@@ -409,14 +409,14 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 // product is that of the units' load, taken half from the mean and half from the unit with the
 // most blocks; splitting K adds the parts' way to memory and back and the kernel that sums them.
 // A 256 x 256 block copies a third less per product and is bound by the matrix cores as much as by
-// the copies: 0.80 us per k-step, and 8 us per block that nothing overlaps (0.73 and 2 where K is
-// split and the grid gives no unit a second block).  It wins where its few blocks still load the units evenly (large
+// the copies: 0.80 us per k-step, and 8 us per block that nothing overlaps (0.73 and 2 where the grid
+// gives no unit a second block).  It wins where its few blocks still load the units evenly (large
 // products: 10 to 20 % at the 24B feed-forward, 12 to 15 % at 7B o/down and 4,096 rows, the 7B down
 // product at 300 to 2,048 rows with K in parts).
-// Against every shape and split measured (7B and 24B q/k/v, o, gate/up and down at 14 row counts
-// from 128 to 4,096, cold weights) the formula's pick is 2.2 % slower than the best on average and
-// 20 % at worst (o at 768 and 1,536 rows, where a split or a smaller block would do better than it
-// predicts); at 2,048 rows and more 0.7 % on average.
+// Against every shape and number of parts measured (7B and 24B q/k/v, o, gate/up and down at 14 row
+// counts from 128 to 4,096, cold weights, parts of K 1 to 6 and 8) the formula's picks take 1.0 % more time
+// than the best in total, 2.2 % per product on average and 38 % at worst (o at 384, 768 and 1,536 rows, where
+// a split or a smaller block would do better than it predicts).
 struct TileShape { int variant, features, tokens, per_unit; };
 static const TileShape g_shapes[] = {{3, 256, 128, 2}, {7, 192, 128, 2}, {8, 128, 128, 2}, {10, 256, 256, 1}, {6, 128, 256, 1}};
 static const TileShape& tile_shape(int variant) {
@@ -437,7 +437,7 @@ static float tiled_cost(const TileShape& t, int splits, int M, int N, int K) {
     float us;
     // eight waves, a unit to itself, one block after the other; a grid of parts of K that gives no
     // unit a second block measures shorter (the long K of a down product at 300 to 1,500 rows)
-    if (t.variant == 10) us = most == 1 && splits > 1 ? steps * 0.73f + 2.f + 3.f : most * (steps * 0.80f + 8.f) + 3.f;
+    if (t.variant == 10) us = most == 1 ? steps * 0.73f + 2.f + 3.f : most * (steps * 0.80f + 8.f) + 3.f;
     else us = steps * (0.10f * rounds + 0.0175f * kb * 0.5f * (mean + most)) + 3.f;
     if (splits > 1) us += 3.f + (float)M * N * 4.f * (2 * splits + 1) / 4.5e6f;
     return us;
@@ -455,7 +455,9 @@ static TilePlan tiled_plan(int M, int N, int K, bool may_split, int forced_varia
         float best_us = 0.f;
         for (const TileShape& t : g_shapes) {
             if (t.variant == 6) continue;                              // (128 x 256 only on request)
-            for (int s = 1; s <= 16 && (s == 1 || steps / s >= 8); s *= 2) {
+            // (any number of parts up to 6, or 8: three fill two rounds where four start a third; 7 and more
+            // than 8 measured worse than the formula says, their partial sums no longer stay in the caches)
+            for (int s = 1; s <= 8 && (s == 1 || steps / s >= 8); s += (s == 6 ? 2 : 1)) {
                 const float us = tiled_cost(t, s, M, N, K);
                 if (best_us == 0.f || us < best_us * 0.999f) { best_us = us; splits = s; }
             }
