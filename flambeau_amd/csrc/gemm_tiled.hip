@@ -409,13 +409,15 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 // product is that of the units' load, taken half from the mean and half from the unit with the
 // most blocks; splitting K adds the parts' way to memory and back and the kernel that sums them.
 // A 256 x 256 block copies a third less per product and is bound by the matrix cores as much as by
-// the copies: 0.80 us per k-step, and 8 us per block that nothing overlaps (0.73 and 2 where the grid
-// gives no unit a second block).  It wins where its few blocks still load the units evenly (large
+// the copies: 0.80 us per k-step, and 8 us per block that nothing overlaps (0.73 and 2 where K is
+// split and the grid gives no unit a second block: such blocks store plain partial sums; with K whole
+// the epilogue is a rotation, an addition to the residual stream or an activation, and the same
+// price for it made the joined q/k/v product of 2,048 rows 130 us instead of 118).  It wins where its few blocks still load the units evenly (large
 // products: 10 to 20 % at the 24B feed-forward, 12 to 15 % at 7B o/down and 4,096 rows, the 7B down
 // product at 300 to 2,048 rows with K in parts).
 // Against every shape and number of parts measured (7B and 24B q/k/v, o, gate/up and down at 14 row
-// counts from 128 to 4,096, cold weights, parts of K 1 to 6 and 8) the formula's picks take 1.0 % more time
-// than the best in total, 2.2 % per product on average and 38 % at worst (o at 384, 768 and 1,536 rows, where
+// counts from 128 to 4,096, cold weights, parts of K 1 to 6 and 8) the formula's picks take 1.1 % more time
+// than the best in total, 2.4 % per product on average and 38 % at worst (o at 384, 768 and 1,536 rows, where
 // a split or a smaller block would do better than it predicts).
 struct TileShape { int variant, features, tokens, per_unit; };
 static const TileShape g_shapes[] = {{3, 256, 128, 2}, {7, 192, 128, 2}, {8, 128, 128, 2}, {10, 256, 256, 1}, {6, 128, 256, 1}};
@@ -437,7 +439,7 @@ static float tiled_cost(const TileShape& t, int splits, int M, int N, int K) {
     float us;
     // eight waves, a unit to itself, one block after the other; a grid of parts of K that gives no
     // unit a second block measures shorter (the long K of a down product at 300 to 1,500 rows)
-    if (t.variant == 10) us = most == 1 ? steps * 0.73f + 2.f + 3.f : most * (steps * 0.80f + 8.f) + 3.f;
+    if (t.variant == 10) us = most == 1 && splits > 1 ? steps * 0.73f + 2.f + 3.f : most * (steps * 0.80f + 8.f) + 3.f;
     else us = steps * (0.10f * rounds + 0.0175f * kb * 0.5f * (mean + most)) + 3.f;
     if (splits > 1) us += 3.f + (float)M * N * 4.f * (2 * splits + 1) / 4.5e6f;
     return us;
