@@ -360,7 +360,12 @@ static int skinny_waves(int N, int K, int nw_hint, int T) {
     int nw = 4;
     while (nw < 16 && blocks * nw < 8 * fl_units()) nw *= 2;
     if (nw_hint > 0) nw = nw_hint;
-    if (T > 1 && nw > 8) nw = 8;              // two sets of w registers: blocks of 512 threads at most
+    // two row groups per block: a wave holds two sets of w registers, twice the bytes in flight (blocks of
+    // 512 threads at most), and with a long K four waves do better than eight (5120 x 32768 at 1 and 8 rows:
+    // 53 to 57 us against 60 to 63; with K of 4096 or 5120 the plain product is the same with either and
+    // the one that rotates and stores 2 us slower with four)
+    if (T > 1 && nw > 8) nw = 8;
+    if (T > 1 && n_steps >= 512 && nw > 4) nw = 4;
     while (nw > 1 && n_steps < nw * 2) nw /= 2;
     return nw < T ? T : nw;                   // wave t finishes row group t
 }
