@@ -13,8 +13,8 @@ ms per step and fraction of the roofline each).  Definitions follow the referenc
 the decode interval only, median of three repetitions.
 
 ``--config v01-window``: Mistral-7B-v0.1 sizes (window 4,096), 8 requests with 8,192-token prompts
-run in portions of 512, then 128 decoded tokens each.  ``--config 24b``: Mistral-Small-24B sizes, 64
-requests with prompts of 128 to 4,096 tokens and 256 decoded tokens each.  Both go through
+run in portions of 512, then 128 decoded tokens each.  ``--config 24b`` and ``--config 12b``: Mistral-Small-24B
+and Mistral-Nemo-12B sizes, 64 requests with prompts of 128 to 4,096 tokens and 256 decoded tokens each.  All go through
 ``LLMEngine`` as a serving loop would drive it and print a line of the same shape.
 """
 from __future__ import annotations
@@ -39,8 +39,11 @@ CONFIG_V01 = dict(CONFIG_7B, vocab_size=32000, rope_theta=10000.0, sliding_windo
 # Mistral-Small-24B / Devstral-Small sizes
 CONFIG_24B = dict(_BASE, num_hidden_layers=40, hidden_size=5120, num_attention_heads=32, num_key_value_heads=8,
                   head_dim=128, intermediate_size=32768, vocab_size=131072, rope_theta=1e8, sliding_window=None)
+# Mistral-Nemo-12B sizes: heads of 128 in a width of 5,120, the 7B feed-forward width, the large vocabulary
+CONFIG_12B = dict(_BASE, num_hidden_layers=40, hidden_size=5120, num_attention_heads=32, num_key_value_heads=8,
+                  head_dim=128, intermediate_size=14336, vocab_size=131072, rope_theta=1e6, sliding_window=None)
 CONFIGS = {"7b": ("Mistral-7B-v0.3 sizes", CONFIG_7B), "v01-window": ("Mistral-7B-v0.1 sizes", CONFIG_V01),
-           "24b": ("Mistral-Small-24B sizes", CONFIG_24B)}
+           "24b": ("Mistral-Small-24B sizes", CONFIG_24B), "12b": ("Mistral-Nemo-12B sizes", CONFIG_12B)}
 PEAK_HBM = 8.0e12            # bytes/s, MI355X
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 PROMPT_LEN = 2048
@@ -301,7 +304,7 @@ def bench_serving(a, name, label, cfg, dtype_name, el):
     r = sorted(runs, key=lambda x: x["t_decode"])[len(runs) // 2]
     window = cfg["sliding_window"] or 0
     extra_points = {}
-    if name == "24b" and not a.no_points:
+    if name in ("24b", "12b") and not a.no_points:
         # decode at batch 1 and 8 behind 2,048 tokens each (the cache filled with random values)
         for b in (1, 8):
             dtl, ctxl = run_decode_filled(model, b, PROMPT_LEN, steps=32, warmup=8)
