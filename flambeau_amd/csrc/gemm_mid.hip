@@ -40,7 +40,8 @@ template <> __device__ __forceinline__ void gm_store4<bf16_t>(bf16_t* p, f32x4 v
     *(bf16x4*)p = o;
 }
 
-#define GM_SCALE_PARTS 4          // parts of a token's sum of squares the row scale can add
+#define GM_SCALE_PARTS 4          // parts of a token's sum of squares the row scale keeps in registers
+#define GM_SCALE_MAX_PARTS 4096   // more parts than that (a producer with a part per 16 features) are added before the loop
 
 // GM_NW waves (row groups) per block, GM_CH k-steps per chunk
 template <int MT, int GM_NW, int GM_CH, typename TOut, bool SWIGLU>
@@ -131,13 +132,37 @@ __global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, c
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int p = 0; p < GM_SCALE_PARTS; ++p) ssq_part[mt][p] = 0.f;
-    if (in_ssq) {
+    if (in_ssq && in_parts <= GM_SCALE_PARTS) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int tok = min(mt * 16 + li, M - 1);
 #pragma unroll
             for (int p = 0; p < GM_SCALE_PARTS; ++p)
                 if (p < in_parts) ssq_part[mt][p] = in_ssq[(size_t)tok * in_parts + p];
+        }
+    } else if (in_ssq) {
+        // many parts (the skinny product leaves one per 16 features): the four lanes of a token add every
+        // fourth piece each, four loads at a time, and then each other's sums, in a fixed order
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const float* row = in_ssq + (size_t)min(mt * 16 + li, M - 1) * in_parts;
+            float t = 0.f;
+            if ((in_parts & 3) == 0) {
+                const int quads = in_parts >> 2;
+                for (int q = g; q < quads; q += 16) {
+                    f32x4 v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = *(const f32x4*)(row + 4 * min(q + 4 * e, quads - 1));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (q + 4 * e < quads) t += (v[e][0] + v[e][1]) + (v[e][2] + v[e][3]);
+                }
+            } else {
+                for (int q = g; q < in_parts; q += 4) t += row[q];
+            }
+            t += __shfl_xor(t, 16, 64);
+            t += __shfl_xor(t, 32, 64);
+            ssq_part[mt][0] = t;
         }
     }
     store_x(x_even, 0);
@@ -384,8 +409,9 @@ extern "C" int fl_gemm_mid_ex(const void* x, const void* w_packed, void* out, fl
     FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
              "gemm_mid: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK((uintptr_t)out % 16 == 0, "gemm_mid: operands must be 16-byte aligned");
-    FL_CHECK(!in_ssq || (in_parts > 0 && in_parts <= GM_SCALE_PARTS), "gemm_mid: a row scale over %d parts (at most %d)",
-             in_parts, GM_SCALE_PARTS);
+    FL_CHECK(!in_ssq || (in_parts > 0 && in_parts <= GM_SCALE_MAX_PARTS &&
+                         (in_parts <= GM_SCALE_PARTS || (in_parts & 3) || (uintptr_t)in_ssq % 16 == 0)),
+             "gemm_mid: a row scale over %d parts (at most %d; in fours they must be 16-byte aligned)", in_parts, GM_SCALE_MAX_PARTS);
     if (M == 0) return 0;
     const int mt = ceil_div(M, 16);
     const bf16_t* xb = (const bf16_t*)x;
@@ -437,8 +463,9 @@ extern "C" int fl_gemm_mid_partials(const void* x, const void* w_packed, float* 
                                     const float* in_ssq, int in_parts, float eps, hipStream_t stream) {
     if (mid_checks(x, w_packed, M, N, K)) return -1;
     FL_CHECK(workspace && (uintptr_t)workspace % 16 == 0, "gemm_mid_partials: needs a 16-byte aligned workspace");
-    FL_CHECK(!in_ssq || (in_parts > 0 && in_parts <= GM_SCALE_PARTS), "gemm_mid: a row scale over %d parts (at most %d)",
-             in_parts, GM_SCALE_PARTS);
+    FL_CHECK(!in_ssq || (in_parts > 0 && in_parts <= GM_SCALE_MAX_PARTS &&
+                         (in_parts <= GM_SCALE_PARTS || (in_parts & 3) || (uintptr_t)in_ssq % 16 == 0)),
+             "gemm_mid: a row scale over %d parts (at most %d; in fours they must be 16-byte aligned)", in_parts, GM_SCALE_MAX_PARTS);
     if (M == 0) return 0;
     const MidScale sc = {in_ssq, in_parts, eps};
     const MidPlan plan = mid_plan(N, K, 0, 0);

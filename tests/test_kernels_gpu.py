@@ -773,6 +773,50 @@ def test_gemm_mid_against_plain(out_dtype, waves, M, N, K):
         assert (got.double() - ref).abs().max() < tol * ref.abs().max(), (splits, n)
 
 
+@pytest.mark.parametrize("M,H,I", [(12, 1024, 352), (16, 640, 96), (9, 5120, 64), (40, 544, 48)])
+def test_gemm_mid_takes_a_row_scale_in_many_parts(M, H, I):
+    """The skinny product leaves a token's sum of squares in a part per 16 features (64 to 320 parts here,
+    or 34, which are not read in fours); the kernel for 17 to 64 rows, which large products use from 9 rows on, adds them
+    itself before its loop: norm(resid) W^T through the factors equals the formula."""
+    from flambeau_amd.kernels.packing import pack_weight
+    K0 = 96
+    x0, w0 = rnd(M, K0, dtype=torch.bfloat16, seed=31), rnd(H, K0, dtype=torch.bfloat16, seed=32, scale=0.1)
+    g = 1 + rnd(H, seed=33, scale=0.1)
+    resid = rnd(M, H, seed=34)
+    want = resid.double() + x0.double() @ w0.double().T
+    xg = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    if M <= 16:
+        ssq = torch.full((M, tuned().skinny_parts(H)), float("nan"), dtype=torch.float32, device=DEV)
+        rows = tuned().gemm_skinny_residual(x0, pack_weight(w0), resid, g, xg, ssq, 1e-5)
+    else:
+        # any producer's parts will do: here 34 parts, which are not read in fours
+        r = want.float()
+        parts = torch.zeros(M, H // 16, dtype=torch.float32, device=DEV)
+        for p_ in range(H // 16):
+            parts[:, p_] = (r[:, p_ * 16:(p_ + 1) * 16] ** 2).sum(dim=1)
+        resid.copy_(r)
+        xg.copy_((r * g).to(torch.bfloat16))
+        rows = tuned().NormedRows(xg, parts, 1e-5, resid, g)
+    assert rows.ssq.shape[1] > 4
+    normed = want * g.double() * torch.rsqrt((want * want).mean(dim=1, keepdim=True) + 1e-5)
+    # plain epilogue
+    w2 = rnd(200, H, dtype=torch.bfloat16, seed=35, scale=0.05)
+    out = torch.full((M, 200), float("nan"), dtype=torch.float32, device=DEV)
+    sp = tuned().gemm_mid_splits(M, 200, H)
+    ws = torch.empty(sp * M * 200, dtype=torch.float32, device=DEV) if sp > 1 else None
+    tuned().gemm_mid(rows.xg, pack_weight(w2), out, ws, row_scale=rows)
+    ref = normed @ w2.double().T
+    assert (out.double() - ref).abs().max() < 1e-2 * ref.abs().max()
+    # gate and up with the activation in the epilogue
+    Wgu = tuned().prepare_gate_up(rnd(I, H, dtype=torch.bfloat16, seed=36, scale=0.05), rnd(I, H, dtype=torch.bfloat16, seed=37, scale=0.05))
+    act = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    tuned().gemm_mid(rows.xg, Wgu.packed, act, swiglu_rows=Wgu.packed_rows, row_scale=rows)
+    gate = normed @ rnd(I, H, dtype=torch.bfloat16, seed=36, scale=0.05).double().T
+    up = normed @ rnd(I, H, dtype=torch.bfloat16, seed=37, scale=0.05).double().T
+    want_act = torch.nn.functional.silu(gate) * up
+    assert (act.double() - want_act).abs().max() < 2e-2 * want_act.abs().max()
+
+
 def test_gemm_mid_refuses_what_it_cannot_do():
     from flambeau_amd.kernels import KernelError
     from flambeau_amd.kernels.packing import pack_weight
