@@ -317,7 +317,7 @@ static int mid_waves(int N, int forced = 0) {
 // at least 4 chunks long, 8 for blocks of eight waves).  Measured at 64 rows: 5120 x 4096 in 80 blocks x 3
 // parts 15.4 us, x 2 18.0, x 4 20.0; 5120 x 32768 in 40 blocks of eight waves x 6 parts 59 us, in 80 of four
 // x 3 74, x 8 (more than two rounds) 80.  Eight waves stream about 30 GB/s per unit against 22 for four
-// and are taken where that outweighs their longer blocks, by 15 % if a block streams less than a megabyte
+// and are taken where that outweighs their longer blocks, by 15 % if a block streams less than half a megabyte
 // (in effect for the long K of a wide feed-forward's down product); the chip as a whole gives 6.3 TB/s; parts cost a kernel that adds them and their way to memory
 // and back.
 // (The entry points whose names end in _ex take waves per block and K-splits from the caller, for
@@ -338,7 +338,7 @@ static MidPlan mid_plan(int N, int K, int forced_waves, int forced_splits) {
         const float bytes = (float)groups * 32.f * K / total;                                   // of w per block
         const float rate = fminf(w == 8 ? 30e3f : 22e3f, 6.3e6f / (float)min(total, (long)units));   // bytes per us
         float us = (float)ceil_div((int)total, units) * bytes / rate + (s > 1 ? 4.5f + s * 64.f * N * 8.f / 5e6f : 0.f);
-        if (w == 8 && bytes < 1e6f) us *= 1.15f;      // (their higher rate shows in long streams only: no gain measured at 262 KB per block)
+        if (w == 8 && bytes < 5e5f) us *= 1.15f;      // (their higher rate shows in long streams only: 6 % at 611 KB per block, none at 458, a loss at 262)
         if (best_us == 0.f || us < best_us) { best = {w, s}; best_us = us; }
     }
     return best;

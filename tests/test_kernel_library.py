@@ -127,13 +127,14 @@ def test_the_tiled_attention_s_plan_for_few_tiles():
 
 def test_parts_of_k_for_products_of_17_to_64_rows():
     """One round of blocks that fills the chip as far as it goes (256 units): parts = units / blocks rounded
-    down, any number; blocks of eight waves only where a block streams a megabyte or more."""
+    down, any number; blocks of eight waves only where a block streams half a megabyte or more."""
     parts = lambda n, k: (tuned.gemm_mid_splits(64, n, k), tuned.gemm_mid_splits(64, n, k, 4, 0), tuned.gemm_mid_splits(64, n, k, 8, 0))
     assert parts(4096, 4096) == (4, 4, 4)             # 64 blocks of four waves x 4; eight waves: parts of 8 chunks at least
     assert parts(6144, 4096)[0] == 2                  # 96 blocks x 2 = 192 (x 3 would start a second round)
     assert parts(5120, 4096) == (3, 3, 4)             # 80 blocks x 3 = 240
     assert parts(5120, 32768) == (6, 3, 6)            # 40 blocks of eight waves x 6 = 240: 1.4 MB per block
     assert parts(4096, 14336)[:2] == (4, 4)
+    assert parts(5120, 14336) == (6, 3, 6)            # 611 KB per block: eight waves
     assert parts(32768, 4096) == (1, 1, 1) and parts(96, 64) == (1, 1, 1)
     for n in (1000, 2048, 4096, 5120, 6144, 8192, 28672):
         for k in (512, 4096, 14336, 32768):
