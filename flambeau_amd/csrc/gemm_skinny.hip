@@ -350,7 +350,11 @@ static int skinny_tiles(int M, int N, int tiles_hint) {
     if (M > 16) return 1;
     if (tiles_hint > 0) return tiles_hint;
     const int groups = ceil_div(N, 16);
-    return groups > fl_units() && groups <= 2 * fl_units() ? 2 : 1;      // (between one and two row groups per compute unit)
+    if (groups > fl_units() && groups <= 2 * fl_units()) return 2;        // (between one and two row groups per compute unit)
+    // from 9 rows on x is fetched by eight loads of two rows where eight rows take four: wide matrices, which
+    // have blocks to spare, then share it between two row groups (at 16 rows: 28672 x 4096 43 -> 42 us,
+    // 65536 x 5120 120 -> 103, 131072 x 5120 246 -> 209, 32768 x 4096 50 -> 46; at 8 rows no gain)
+    return M > 8 && groups >= 2 * fl_units() ? 2 : 1;
 }
 
 static int skinny_waves(int N, int K, int nw_hint, int T) {

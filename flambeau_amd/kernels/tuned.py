@@ -59,16 +59,19 @@ FUSED_NORM_MAX_ROWS = 16     # the skinny kernel's fusions with the norms around
 
 
 def mid_preferred(M: int, N: int, K: int) -> bool:
-    """Whether a product of at most 16 rows goes to the kernel that shares x through LDS although the
-    skinny kernel takes it: from 9 rows on the skinny kernel fetches twice the x per byte of w, which
-    large matrices feel first (measured, microseconds at 8 / 10 / 12 / 16 rows, the kernel that adds the
-    K-splits included: 5120 x 32768 skinny 65 / 67 / 68 / 72, mid 57 throughout; 65536 x 5120 108 / 112 /
-    115 / 125 against 107 to 108; 5120 x 14336 28 / 29 / 30 / 31.5 against 27; 4096 x 14336 22.9 / 23.6 / 24.2 /
-    25.5 against 23.0 to 23.4; 28672 x 4096 39.7 / 41.9 / 42.2 / 44.2 against 43.5)."""
-    if M <= 8 or K % 32:
+    """Whether the product that adds to the residual stream goes, at 9 to 16 rows, to the kernel that shares
+    x through LDS although the skinny kernel takes it: from 9 rows on the skinny kernel fetches twice the x
+    per byte of w, which a long K feels (measured, microseconds at 8 / 10 / 12 / 16 rows, the kernel that adds
+    the K-splits included: 5120 x 32768 skinny 65 / 67 / 68 / 72, mid 57 throughout; 5120 x 14336 28 / 29 /
+    30 / 31.5 against 27; 4096 x 14336 22.9 / 23.6 / 24.2 / 25.5 against 23.0 to 23.4).  Wide matrices with a
+    short K stay with the skinny kernel, which shares x between two row groups from 9 rows on and is then as
+    fast (65536 x 5120 at 16 rows: 107 us either way)."""
+    if M <= 8 or K % 32 or K < 8192:
         return False
     nbytes = 2 * N * K
-    return (nbytes >= 256e6 or (nbytes >= 140e6 and K >= 8192)) or (M >= 13 and nbytes >= 100e6 and K >= 8192)
+    return nbytes >= 140e6 or (M >= 13 and nbytes >= 100e6)
+
+
 MID_PART_COLS = 4096         # columns per partial sum of squares that gemm_mid_residual leaves
 MID_SCALE_PARTS = 4096       # parts the row scale of gemm_mid can add (up to 4 cost nothing, more a short loop before the product)
 
@@ -469,13 +472,12 @@ def gemm_swiglu(x, w: Weight, out, rt):
     x, scale = _rows_for(x, w, rt)
     M, K = x.shape
     if scale is not None and w.swiglu_cols:
-        skinny = M <= FUSED_NORM_MAX_ROWS and not (mid_preferred(M, w.packed_rows, K) and scale.ssq.shape[1] <= MID_SCALE_PARTS)
-        kernel = gemm_skinny if skinny else (gemm_mid if M <= SKINNY_MAX_ROWS else gemm_tiled)
+        kernel = gemm_skinny if M <= FUSED_NORM_MAX_ROWS else (gemm_mid if M <= SKINNY_MAX_ROWS else gemm_tiled)
         return kernel(x, w.packed, out, swiglu_rows=w.packed_rows, row_scale=scale)
     if scale is not None:
         x = scale.materialize(rt)
     if w.packed is not None and w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
-        if (SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0) or mid_preferred(M, w.packed_rows, K):
+        if SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0:
             return gemm_mid(x, w.packed, out, swiglu_rows=w.packed_rows)
         if M <= SKINNY_MAX_ROWS:
             return gemm_skinny(x, w.packed, out, swiglu_rows=w.packed_rows)
