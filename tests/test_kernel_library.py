@@ -141,3 +141,14 @@ def test_parts_of_k_for_products_of_17_to_64_rows():
             for w in (0, 4, 8):
                 s = tuned.gemm_mid_splits(64, n, k, w, 0)
                 assert 1 <= s <= 32 and (s == 1 or (k // 128) // s >= 4)
+
+
+def test_which_products_of_9_to_16_rows_leave_the_skinny_kernel():
+    """Only the product that adds to the residual stream with a long K (a feed-forward's way down) goes to the
+    kernel for 17 to 64 rows early; everything stays with the skinny kernel up to 8 rows."""
+    assert not any(tuned.mid_preferred(m, n, k) for m in (1, 8) for n, k in ((5120, 32768), (4096, 14336), (65536, 5120)))
+    assert all(tuned.mid_preferred(m, 5120, 32768) for m in (9, 12, 16))
+    assert all(tuned.mid_preferred(m, 5120, 14336) for m in (9, 16))
+    assert [tuned.mid_preferred(m, 4096, 14336) for m in (9, 12, 13, 16)] == [False, False, True, True]
+    assert not tuned.mid_preferred(16, 65536, 5120) and not tuned.mid_preferred(16, 4096, 4096)
+    assert not tuned.mid_preferred(16, 5120, 32768 + 8)          # K must be whole steps of 32 for that kernel
